@@ -1,0 +1,220 @@
+/*
+ * C ABI of the MI355X (gfx950) kernel library behind the llm_hip engine's dynamic-batching attention path.
+ *
+ * It takes the place of the un-vendored C++ library `ppl.llm.kernel.cuda` that the reference engine calls from
+ *   src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/multi_head_cache_attention_kernel.cc:170-230
+ *   (`dynamic_batching_multi_head_cache_attention::heuristic_prepare` + `forward`), and from
+ *   src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/key_value_cache_kernel.cc:23-114 (a stub there).
+ *
+ * Conventions: plain pointers and sizes only; every pointer named `d_*` or documented "device" is a device
+ * address valid on the current HIP device; `stream` is a `hipStream_t` passed as `void*` (NULL = default stream);
+ * every function returns a `pplhip_retcode` and enqueues work asynchronously on `stream` unless it says otherwise.
+ * Nothing here allocates device memory: the caller owns the KV slab, the tables, the outputs and the workspace.
+ */
+#ifndef PPL_LLM_KERNEL_HIP_H_
+#define PPL_LLM_KERNEL_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Same meaning (and order) as the ppl::common::RetCode values the reference wrappers return
+ * (src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/multi_head_cache_attention_kernel.cc:90-166). */
+typedef enum pplhip_retcode {
+    PPLHIP_RC_SUCCESS = 0,
+    PPLHIP_RC_OTHER_ERROR = 1,
+    PPLHIP_RC_UNSUPPORTED = 2,
+    PPLHIP_RC_OUT_OF_MEMORY = 3,
+    PPLHIP_RC_INVALID_VALUE = 4,
+    PPLHIP_RC_EXISTS = 5,
+    PPLHIP_RC_NOT_FOUND = 6,
+    PPLHIP_RC_PERMISSION_DENIED = 7,
+    PPLHIP_RC_HOST_MEMORY_ERROR = 8,
+    PPLHIP_RC_DEVICE_MEMORY_ERROR = 9,
+    PPLHIP_RC_DEVICE_RUNTIME_ERROR = 10,
+    PPLHIP_RC_OUT_OF_RANGE = 11,
+    PPLHIP_RC_INTERNAL_ERROR = 12
+} pplhip_retcode;
+
+/* Human-readable text of the last error raised on the calling thread ("" if none). Never NULL. */
+const char* pplhip_last_error(void);
+
+/* Library/ABI version: major*10000 + minor*100 + patch. */
+int32_t pplhip_version(void);
+
+/*
+ * Argument block of MultiHeadCacheAttention: one field per argument the reference passes to `heuristic_prepare`
+ * (multi_head_cache_attention_kernel.cc:170-212), in the same order and with the same meaning.
+ *
+ * Tensors (fp16 = IEEE binary16, NDARRAY, contiguous):
+ *   query         fp16 [S, num_heads, head_dim]       S = seqstarts[batch] packed new tokens
+ *   current_key   fp16 [S, num_kv_heads, head_dim]
+ *   current_value fp16 [S, num_kv_heads, head_dim]
+ *   seqstarts     i64  [batch+1]   prefix sums of new-token counts, seqstarts[0] = 0
+ *   kvstarts      i64  [batch+1]   prefix sums of kv lengths (start_pos + seqlen), kvstarts[0] = 0
+ *   cachestarts   i64  [batch]     first slab token of each sequence (cache_mode 0)
+ *   start_pos     i64  [batch]     tokens already cached before this call
+ *   cache         i8   element (tok, layer, kv, head, d) at
+ *                      tok*cache_stride_s + layer*cache_stride_l + kv*cache_stride_kv + head*cache_stride_h + d
+ *   scale         fp16 one per group of 8 channels; element strides are the cache strides divided by 8
+ *   output        fp16 [S, num_heads, head_dim]
+ * Sequences [0, decoding_batches) are decode steps (exactly one new token each) and attend over the int8 cache,
+ * the just-written token included; sequences [decoding_batches, batch) are prefill and attend over the fp16
+ * current_key/current_value (or over the cache when cache_prefill != 0, which also allows start_pos > 0).
+ */
+typedef struct pplhip_mhca_args {
+    const void* d_query;
+    const void* d_current_key;
+    const void* d_current_value;
+    const void* d_attn_mask; /* additive fp16 mask: must be NULL (no shipped model passes one) */
+    const int64_t* d_seqstarts;
+    const int64_t* d_kvstarts;
+    const int64_t* d_cachestarts;
+    const int64_t* d_start_pos;
+    const void* d_alibi_slopes; /* must be NULL: the reference rejects is_alibi (…_kernel.cc:95-98) */
+    int32_t is_causal;
+    int64_t batch;
+    int64_t decoding_batches;
+    int64_t max_seqlen;
+    int64_t max_kvlen;
+    int32_t layer_idx;
+    int32_t num_layer;
+    int32_t num_heads;
+    int32_t num_kv_heads;
+    int32_t head_dim;
+    int32_t cache_mode; /* 0 = contiguous region per sequence; 1 (paged) is rejected for now */
+    int32_t page_size;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestart_stride_b;
+    /* engine knobs, same values as EngineConfig (src/ppl/nn/engines/llm_cuda/engine_config.h:25-36) */
+    int32_t enable_cache_prefill;
+    int32_t enable_decoding_sharemem_mhca; /* accepted, ignored: one decode algorithm serves every shape */
+    int32_t enable_decoding_infinity_mhca; /* accepted, ignored */
+    int32_t enable_decoding_infinity_gqca; /* accepted, ignored */
+    int32_t specify_decoding_attn_split_k; /* 0 off, 1 heuristic, 2 always */
+    int32_t specify_decoding_attn_tpb; /* 0 heuristic, 256, 512 */
+    void* d_cache;
+    void* d_scale;
+    void* d_output;
+    int64_t total_new_tokens; /* S = query dim 0 (the reference passes the query TensorShape) */
+} pplhip_mhca_args;
+
+/* What `heuristic_prepare` stores in the reference kernel object's `.cfg` (…_kernel.cc:218-228 reads
+ * `cfg.workspace_size` and sets `cfg.workspace`). Filled by pplhip_mhca_prepare, consumed by pplhip_mhca_forward. */
+typedef struct pplhip_mhca_plan {
+    uint64_t workspace_bytes; /* device scratch the caller must pass to forward (may be 0) */
+    int32_t decode_chunk_tokens; /* cached tokens handled by one wavefront task (split-k granularity) */
+    int32_t decode_num_chunks; /* ceil(max_kvlen / decode_chunk_tokens) */
+    int32_t decode_waves_per_block;
+    int32_t prefill_q_tile; /* query rows per prefill workgroup */
+    int32_t prefill_num_q_tiles; /* ceil(max_seqlen / prefill_q_tile) */
+    int32_t reserved[3];
+} pplhip_mhca_plan;
+
+/* Host-only: validates `args` exactly like the reference wrapper + kernel library would
+ * (unsupported attrs -> PPLHIP_RC_UNSUPPORTED, inconsistent sizes -> PPLHIP_RC_INVALID_VALUE),
+ * picks the split-k decomposition and reports the workspace size. Replaces `heuristic_prepare`
+ * (multi_head_cache_attention_kernel.cc:170). Does not touch the device. */
+pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* args, pplhip_mhca_plan* plan);
+
+/* Enqueues: quantize-on-write of the new K/V tokens, decode attention (+ split-k merge) for the first
+ * `decoding_batches` sequences and causal prefill attention for the rest. Replaces `forward(stream)`
+ * (multi_head_cache_attention_kernel.cc:230). `d_workspace` must hold plan->workspace_bytes (256-byte aligned). */
+pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* args, const pplhip_mhca_plan* plan, void* d_workspace,
+                                   void* stream);
+
+/*
+ * Quantize-on-write alone: new token t of sequence b goes to slab token cachestarts[b] + start_pos[b] + t.
+ * Per (token, K|V, kv head, group of 8 channels): scale = max(fp16(absmax / 127), fp16(1e-5)),
+ * q = int8(rint(fp16(x / scale))). This is the first step of the reference's fused `forward`.
+ */
+typedef struct pplhip_kv_write_args {
+    const void* d_current_key; /* fp16 [S, num_kv_heads, head_dim] */
+    const void* d_current_value;
+    const int64_t* d_seqstarts; /* [batch+1] */
+    const int64_t* d_cachestarts; /* [batch] */
+    const int64_t* d_start_pos; /* [batch] */
+    int64_t batch;
+    int64_t total_new_tokens; /* S */
+    int32_t layer_idx;
+    int32_t num_layer;
+    int32_t num_kv_heads;
+    int32_t head_dim;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    void* d_cache;
+    void* d_scale;
+} pplhip_kv_write_args;
+
+pplhip_retcode pplhip_kv_quantize_write(const pplhip_kv_write_args* args, void* stream);
+
+/*
+ * opmx.dynamic_batching::KeyValueCache (inputs/outputs of
+ * src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/key_value_cache_kernel.cc:26-39, which is a stub that
+ * returns RC_UNSUPPORTED in the reference): quantize-on-write as above, then key/value outputs
+ * fp16 [kvstarts[batch], num_kv_heads, head_dim] = the dequantised cache rows of every sequence in batch order.
+ * `total_kv_tokens` = kvstarts[batch] (the reference reads it back for shape inference,
+ * src/ppl/nn/oputils/opmx/reshape_dynamic_batching_key_value_cache.cc:43-53).
+ */
+typedef struct pplhip_kv_cache_args {
+    pplhip_kv_write_args write;
+    const int64_t* d_kvstarts; /* [batch+1] */
+    int64_t total_kv_tokens;
+    int64_t max_kvlen;
+    int32_t num_repeat; /* only 1 (key_value_cache_kernel.cc:93-96) */
+    int32_t cache_mode; /* only 0 */
+    int32_t cache_layout; /* only 0 */
+    int32_t reserved;
+    void* d_key_out;
+    void* d_value_out;
+} pplhip_kv_cache_args;
+
+pplhip_retcode pplhip_kv_cache_forward(const pplhip_kv_cache_args* args, void* stream);
+
+/*
+ * On-device rebuild of the ragged-batch tables, replacing the host loops of
+ * tools/benchmark_llama/generation_state.cc:60-125 (FirstStep) and :127-192 (NextStep) plus the eight per-step
+ * uploads of tools/benchmark_llama/text_generator.cc:233-291.
+ *
+ * Slot state (device, one entry per slot, `num_slots` <= 1024):
+ *   slot_kvlen[i]   tokens cached for the slot's sequence BEFORE this step (0 for a fresh prompt)
+ *   slot_newlen[i]  new tokens this step: 0 = slot idle/retired, 1 with kvlen > 0 = decode step, otherwise prefill
+ *   slot_cachestart[i] first slab token of the slot's region
+ * Outputs (device): active sequences are compacted stably, decode sequences first, then prefill sequences;
+ *   seqstarts/kvstarts [num_slots+1] (entries past the batch repeat the total), cachestarts/start_pos/batch_slots
+ *   [num_slots] (batch_slots[b] = slot index of packed sequence b, -1 past the batch), and
+ *   header[0..5] = {batch, decoding_batches, max_seqlen, max_kvlen, total_new_tokens, total_kv_tokens}.
+ */
+typedef struct pplhip_pack_args {
+    const int64_t* d_slot_kvlen;
+    const int64_t* d_slot_newlen;
+    const int64_t* d_slot_cachestart;
+    int32_t num_slots;
+    int32_t reserved;
+    int64_t* d_seqstarts;
+    int64_t* d_kvstarts;
+    int64_t* d_cachestarts;
+    int64_t* d_start_pos;
+    int64_t* d_batch_slots;
+    int64_t* d_header; /* 6 x i64; may be pinned host memory mapped on the device */
+} pplhip_pack_args;
+
+pplhip_retcode pplhip_pack_tables(const pplhip_pack_args* args, void* stream);
+
+/* After a step: slot_kvlen += slot_newlen for every active slot (so the next pack sees the grown sequences). */
+pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot_newlen, int32_t num_slots,
+                                    void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PPL_LLM_KERNEL_HIP_H_ */

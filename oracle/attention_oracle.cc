@@ -1,0 +1,344 @@
+// TEST INFRASTRUCTURE ONLY. Scalar CPU restatement of the dynamic-batching attention path.
+// Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load this library; the product
+// (the HIP kernel library and the llm_hip engine) never links, imports or calls it.
+//
+// What it restates (the arithmetic itself lives in the un-vendored dependency `ppl.llm.kernel.cuda`,
+// fetched from GitHub branch `master` by cmake/deps.cmake:290-304, so it is absent from the reference tree):
+//   * argument meaning, tensor order, strides      src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/
+//                                                   multi_head_cache_attention_kernel.cc:27-41, 136-212
+//   * KeyValueCache I/O contract                    .../dynamic_batching/key_value_cache_kernel.cc:26-110 and
+//                                                   src/ppl/nn/oputils/opmx/reshape_dynamic_batching_key_value_cache.cc:26-53
+//   * table semantics (seqstarts/kvstarts/...)      tools/benchmark_llama/generation_state.cc:60-192
+//   * prefill reads fp16 K/V unless cache-prefill   include/ppl/nn/engines/llm_cuda/options.h:139-149
+//
+// PARITY STATUS (no reference test, fixture or golden vector covers any opmx op, and the reference cannot be
+// built or run offline, so each function is pinned by mathematics instead -- see tests/test_oracle_*.py):
+//   oracle_kv_quantize_*   rule DEFINED here (published text: "INT8 groupwise", fp16 absmax/127 scale per group
+//                          of 8); pinned by closed forms + a numpy restatement over all finite fp16 absmax values.
+//                          Bit pattern of the absent CUDA kernel: parity unpinned.
+//   oracle_mhca_forward    pinned against a float64 numpy softmax(QK^T/sqrt(d)+mask)V, closed forms
+//                          (kvlen 1, equal keys, dominant key), GQA==MHA, decode == last prefill row, NaN poison.
+//   oracle_kv_cache_forward pinned by |dequant(quant(x)) - x| <= scale/2 and row-order checks.
+//   oracle_pack_tables     pinned against a brute-force Python loop written from generation_state.cc.
+//   oracle_x86_attention   pinned against the same float64 textbook routine.
+
+#include "../include/ppl_llm_kernel_hip.h"
+#include "fp16_soft.h"
+
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <vector>
+
+using oracle::float_to_half;
+using oracle::half_to_float;
+
+namespace {
+
+const int kGroup = 8;
+
+inline uint16_t eps_half() {
+    return float_to_half(1e-5f); // 0x00a8, a binary16 subnormal ~= 1.0014e-5
+}
+
+// One group of 8 channels. Rule:
+//   a = max |x_i|                         (exact in binary16)
+//   s = max(fp16_rne(float(a) / 127.0f), fp16_rne(1e-5f))
+//   q_i = int8(rint_ties_even(float(fp16_rne(float(x_i) / float(s)))))
+void quantize_group(const uint16_t* x, int8_t* q, uint16_t* scale) {
+    float amax = 0.f;
+    for (int i = 0; i < kGroup; ++i) {
+        float v = fabsf(half_to_float(x[i]));
+        if (v > amax) amax = v; // NaN never wins; inf does
+    }
+    uint16_t s = float_to_half(amax / 127.0f);
+    const uint16_t e = eps_half();
+    if (half_to_float(s) < half_to_float(e)) s = e;
+    const float sf = half_to_float(s);
+    for (int i = 0; i < kGroup; ++i) {
+        const float ratio = half_to_float(float_to_half(half_to_float(x[i]) / sf));
+        float r = nearbyintf(ratio); // default rounding mode: ties to even
+        if (!(r >= -128.f)) r = -128.f; // also catches NaN
+        if (r > 127.f) r = 127.f;
+        q[i] = (int8_t)r;
+    }
+    *scale = s;
+}
+
+struct CacheView {
+    int8_t* cache;
+    uint16_t* scale;
+    int64_t ss, sl, sh, skv;
+    int layer;
+    int8_t* row(int64_t tok, int kv, int head) const {
+        return cache + tok * ss + layer * sl + kv * skv + head * sh;
+    }
+    uint16_t* srow(int64_t tok, int kv, int head) const {
+        return scale + (tok * ss + layer * sl + kv * skv + head * sh) / kGroup;
+    }
+};
+
+void write_new_tokens(const pplhip_kv_write_args* a) {
+    CacheView cv{(int8_t*)a->d_cache, (uint16_t*)a->d_scale, a->cache_stride_s, a->cache_stride_l,
+                 a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
+    const uint16_t* src[2] = {(const uint16_t*)a->d_current_key, (const uint16_t*)a->d_current_value};
+    const int KVH = a->num_kv_heads, Dh = a->head_dim;
+    for (int64_t b = 0; b < a->batch; ++b) {
+        const int64_t s0 = a->d_seqstarts[b], s1 = a->d_seqstarts[b + 1];
+        for (int64_t t = s0; t < s1; ++t) {
+            const int64_t tok = a->d_cachestarts[b] + a->d_start_pos[b] + (t - s0);
+            for (int kv = 0; kv < 2; ++kv)
+                for (int h = 0; h < KVH; ++h) {
+                    const uint16_t* x = src[kv] + (t * KVH + h) * Dh;
+                    int8_t* q = cv.row(tok, kv, h);
+                    uint16_t* s = cv.srow(tok, kv, h);
+                    for (int g = 0; g < Dh / kGroup; ++g) quantize_group(x + g * kGroup, q + g * kGroup, s + g);
+                }
+        }
+    }
+}
+
+inline void dequant_row(const int8_t* q, const uint16_t* s, int Dh, double* out) {
+    for (int d = 0; d < Dh; ++d) out[d] = (double)q[d] * (double)half_to_float(s[d / kGroup]);
+}
+
+} // namespace
+
+extern "C" {
+
+void oracle_half_to_float(const uint16_t* h, float* f, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) f[i] = half_to_float(h[i]);
+}
+void oracle_float_to_half(const float* f, uint16_t* h, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) h[i] = float_to_half(f[i]);
+}
+
+// n_groups groups of 8 binary16 values -> int8 bytes + one binary16 scale per group.
+void oracle_kv_quantize_groups(const uint16_t* x, int8_t* q, uint16_t* scale, int64_t n_groups) {
+    for (int64_t g = 0; g < n_groups; ++g) quantize_group(x + g * kGroup, q + g * kGroup, scale + g);
+}
+
+// q (int8) * scale (binary16) -> float32 (exact product of the two, rounded once to float32).
+void oracle_kv_dequant_groups(const int8_t* q, const uint16_t* scale, float* out, int64_t n_groups) {
+    for (int64_t g = 0; g < n_groups; ++g)
+        for (int i = 0; i < kGroup; ++i) out[g * kGroup + i] = (float)q[g * kGroup + i] * half_to_float(scale[g]);
+}
+
+// All pointers in the argument blocks are HOST pointers here.
+int oracle_kv_quantize_write(const pplhip_kv_write_args* a) {
+    if (a->head_dim % kGroup) return PPLHIP_RC_INVALID_VALUE;
+    write_new_tokens(a);
+    return PPLHIP_RC_SUCCESS;
+}
+
+// Write-then-attend. out_f64 (optional) receives the un-rounded double results, [S, H, Dh].
+int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
+    const int H = a->num_heads, KVH = a->num_kv_heads, Dh = a->head_dim;
+    if (H <= 0 || KVH <= 0 || H % KVH || Dh % kGroup) return PPLHIP_RC_INVALID_VALUE;
+    if (a->d_attn_mask || a->d_alibi_slopes || a->cache_mode != 0) return PPLHIP_RC_UNSUPPORTED;
+    pplhip_kv_write_args w;
+    memset(&w, 0, sizeof(w));
+    w.d_current_key = a->d_current_key;
+    w.d_current_value = a->d_current_value;
+    w.d_seqstarts = a->d_seqstarts;
+    w.d_cachestarts = a->d_cachestarts;
+    w.d_start_pos = a->d_start_pos;
+    w.batch = a->batch;
+    w.total_new_tokens = a->total_new_tokens;
+    w.layer_idx = a->layer_idx;
+    w.num_layer = a->num_layer;
+    w.num_kv_heads = KVH;
+    w.head_dim = Dh;
+    w.cache_stride_s = a->cache_stride_s;
+    w.cache_stride_l = a->cache_stride_l;
+    w.cache_stride_h = a->cache_stride_h;
+    w.cache_stride_kv = a->cache_stride_kv;
+    w.d_cache = a->d_cache;
+    w.d_scale = a->d_scale;
+    write_new_tokens(&w);
+
+    CacheView cv{(int8_t*)a->d_cache, (uint16_t*)a->d_scale, a->cache_stride_s, a->cache_stride_l,
+                 a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
+    const uint16_t* Q = (const uint16_t*)a->d_query;
+    const uint16_t* CK = (const uint16_t*)a->d_current_key;
+    const uint16_t* CV = (const uint16_t*)a->d_current_value;
+    uint16_t* O = (uint16_t*)a->d_output;
+    const int rep = H / KVH;
+    const double sm_scale = 1.0 / sqrt((double)Dh);
+
+#pragma omp parallel for collapse(2) schedule(dynamic, 1)
+    for (int64_t b = 0; b < a->batch; ++b) {
+        for (int h = 0; h < H; ++h) {
+            const int kvh = h / rep;
+            const int64_t s0 = a->d_seqstarts[b], seqlen = a->d_seqstarts[b + 1] - s0;
+            const int64_t sp = a->d_start_pos[b];
+            const int64_t kvlen = a->d_kvstarts[b + 1] - a->d_kvstarts[b];
+            const bool from_cache = (b < a->decoding_batches) || a->enable_cache_prefill;
+            // materialise this (sequence, kv head)'s keys and values as doubles
+            std::vector<double> K((size_t)kvlen * Dh), V((size_t)kvlen * Dh);
+            for (int64_t j = 0; j < kvlen; ++j) {
+                if (from_cache) {
+                    const int64_t tok = a->d_cachestarts[b] + j;
+                    dequant_row(cv.row(tok, 0, kvh), cv.srow(tok, 0, kvh), Dh, &K[j * Dh]);
+                    dequant_row(cv.row(tok, 1, kvh), cv.srow(tok, 1, kvh), Dh, &V[j * Dh]);
+                } else {
+                    // fp16 path: key j of the sequence is packed row seqstarts[b] + j (start_pos must be 0)
+                    const uint16_t* kr = CK + ((s0 + j) * KVH + kvh) * Dh;
+                    const uint16_t* vr = CV + ((s0 + j) * KVH + kvh) * Dh;
+                    for (int d = 0; d < Dh; ++d) {
+                        K[j * Dh + d] = half_to_float(kr[d]);
+                        V[j * Dh + d] = half_to_float(vr[d]);
+                    }
+                }
+            }
+            std::vector<double> p((size_t)kvlen), acc(Dh), q(Dh);
+            for (int64_t t = 0; t < seqlen; ++t) {
+                const uint16_t* qr = Q + ((s0 + t) * H + h) * Dh;
+                for (int d = 0; d < Dh; ++d) q[d] = half_to_float(qr[d]);
+                const int64_t last = a->is_causal ? std::min<int64_t>(sp + t, kvlen - 1) : kvlen - 1;
+                double m = -INFINITY;
+                for (int64_t j = 0; j <= last; ++j) {
+                    double s = 0;
+                    for (int d = 0; d < Dh; ++d) s += q[d] * K[j * Dh + d];
+                    p[j] = s * sm_scale;
+                    m = std::max(m, p[j]);
+                }
+                double l = 0;
+                for (int64_t j = 0; j <= last; ++j) {
+                    p[j] = exp(p[j] - m);
+                    l += p[j];
+                }
+                std::fill(acc.begin(), acc.end(), 0.0);
+                for (int64_t j = 0; j <= last; ++j)
+                    for (int d = 0; d < Dh; ++d) acc[d] += p[j] * V[j * Dh + d];
+                for (int d = 0; d < Dh; ++d) {
+                    const double o = acc[d] / l;
+                    const int64_t idx = ((s0 + t) * H + h) * Dh + d;
+                    if (out_f64) out_f64[idx] = o;
+                    O[idx] = float_to_half((float)o);
+                }
+            }
+        }
+    }
+    return PPLHIP_RC_SUCCESS;
+}
+
+// KeyValueCache op: write, then emit dequantised rows in batch order as binary16 (one rounding of q*scale).
+int oracle_kv_cache_forward(const pplhip_kv_cache_args* a) {
+    if (a->num_repeat != 1 || a->cache_mode != 0 || a->cache_layout != 0) return PPLHIP_RC_UNSUPPORTED;
+    const pplhip_kv_write_args* w = &a->write;
+    write_new_tokens(w);
+    CacheView cv{(int8_t*)w->d_cache, (uint16_t*)w->d_scale, w->cache_stride_s, w->cache_stride_l,
+                 w->cache_stride_h, w->cache_stride_kv, w->layer_idx};
+    const int KVH = w->num_kv_heads, Dh = w->head_dim;
+    uint16_t* outs[2] = {(uint16_t*)a->d_key_out, (uint16_t*)a->d_value_out};
+    for (int64_t b = 0; b < w->batch; ++b) {
+        const int64_t k0 = a->d_kvstarts[b], kvlen = a->d_kvstarts[b + 1] - k0;
+        for (int64_t j = 0; j < kvlen; ++j) {
+            const int64_t tok = w->d_cachestarts[b] + j;
+            for (int kv = 0; kv < 2; ++kv)
+                for (int h = 0; h < KVH; ++h) {
+                    const int8_t* q = cv.row(tok, kv, h);
+                    const uint16_t* s = cv.srow(tok, kv, h);
+                    uint16_t* o = outs[kv] + ((k0 + j) * KVH + h) * Dh;
+                    for (int d = 0; d < Dh; ++d)
+                        o[d] = float_to_half((float)q[d] * half_to_float(s[d / kGroup]));
+                }
+        }
+    }
+    return PPLHIP_RC_SUCCESS;
+}
+
+// Table rebuild: stable compaction (decode first, then prefill), prefix sums, maxima.
+// Follows tools/benchmark_llama/generation_state.cc:93-110 (prefix sums, start_pos, cachestarts) and :162-170.
+int oracle_pack_tables(const pplhip_pack_args* a) {
+    const int n = a->num_slots;
+    int64_t b = 0, max_seq = 0, max_kv = 0;
+    a->d_seqstarts[0] = 0;
+    a->d_kvstarts[0] = 0;
+    int64_t decoding = 0;
+    for (int pass = 0; pass < 2; ++pass) {
+        for (int i = 0; i < n; ++i) {
+            const int64_t nl = a->d_slot_newlen[i], kl = a->d_slot_kvlen[i];
+            if (nl <= 0) continue;
+            const bool is_decode = (nl == 1 && kl > 0);
+            if ((pass == 0) != is_decode) continue;
+            a->d_seqstarts[b + 1] = a->d_seqstarts[b] + nl;
+            a->d_kvstarts[b + 1] = a->d_kvstarts[b] + kl + nl;
+            a->d_cachestarts[b] = a->d_slot_cachestart[i];
+            a->d_start_pos[b] = kl;
+            a->d_batch_slots[b] = i;
+            max_seq = std::max(max_seq, nl);
+            max_kv = std::max(max_kv, kl + nl);
+            ++b;
+        }
+        if (pass == 0) decoding = b;
+    }
+    for (int64_t i = b; i < n; ++i) {
+        a->d_seqstarts[i + 1] = a->d_seqstarts[b];
+        a->d_kvstarts[i + 1] = a->d_kvstarts[b];
+        a->d_cachestarts[i] = 0;
+        a->d_start_pos[i] = 0;
+        a->d_batch_slots[i] = -1;
+    }
+    a->d_header[0] = b;
+    a->d_header[1] = decoding;
+    a->d_header[2] = max_seq;
+    a->d_header[3] = max_kv;
+    a->d_header[4] = a->d_seqstarts[b];
+    a->d_header[5] = a->d_kvstarts[b];
+    return PPLHIP_RC_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// CPU baseline with the x86 engine's op semantics: the ONNX subgraph
+//     MatMul(Q, K^T) -> Mul(1/sqrt(d)) -> Add(mask) -> Softmax(axis -1) -> MatMul(., V)
+// in fp32 NDARRAY, one head at a time ([heads, Lq, d] x [heads, d, Lk]); wrappers being restated:
+// src/ppl/nn/engines/x86/kernels/onnx/matmul_kernel.cc:44-52, add_kernel.cc:64-71, softmax_kernel.cc:41-56
+// (axis -1 default for opset >= 13: src/ppl/nn/models/onnx/parsers/onnx/parse_softmax_param.cc:29). The arithmetic
+// of those ops is in the un-vendored ppl.kernel.cpu; these are plain loops, threaded over heads with OpenMP the way
+// `pplnn --num-threads` threads the x86 engine (tools/pplnn.cc:332,377-380).
+// q [heads, Lq, d], k [kv_heads, Lk, d], v [kv_heads, Lk, d], mask [Lq, Lk] additive (may be NULL), out [heads, Lq, d].
+int oracle_x86_attention(const float* q, const float* k, const float* v, const float* mask, float* out, int heads,
+                         int kv_heads, int64_t Lq, int64_t Lk, int d, int num_threads) {
+    if (heads % kv_heads) return PPLHIP_RC_INVALID_VALUE;
+    const int rep = heads / kv_heads;
+    const float sm = 1.0f / sqrtf((float)d);
+    (void)num_threads;
+#pragma omp parallel for num_threads(num_threads > 0 ? num_threads : 1) schedule(dynamic, 1)
+    for (int h = 0; h < heads; ++h) {
+        const float* qh = q + (int64_t)h * Lq * d;
+        const float* kh = k + (int64_t)(h / rep) * Lk * d;
+        const float* vh = v + (int64_t)(h / rep) * Lk * d;
+        float* oh = out + (int64_t)h * Lq * d;
+        std::vector<float> s((size_t)Lk);
+        for (int64_t i = 0; i < Lq; ++i) {
+            float m = -INFINITY;
+            for (int64_t j = 0; j < Lk; ++j) { // MatMul + Mul + Add
+                float acc = 0.f;
+                for (int c = 0; c < d; ++c) acc += qh[i * d + c] * kh[j * d + c];
+                acc *= sm;
+                if (mask) acc += mask[i * Lk + j];
+                s[j] = acc;
+                m = std::max(m, acc);
+            }
+            float l = 0.f; // Softmax along the last axis
+            for (int64_t j = 0; j < Lk; ++j) {
+                s[j] = expf(s[j] - m);
+                l += s[j];
+            }
+            const float inv = 1.0f / l;
+            for (int c = 0; c < d; ++c) oh[i * d + c] = 0.f;
+            for (int64_t j = 0; j < Lk; ++j) { // MatMul with V
+                const float pj = s[j] * inv;
+                for (int c = 0; c < d; ++c) oh[i * d + c] += pj * vh[j * d + c];
+            }
+        }
+    }
+    return PPLHIP_RC_SUCCESS;
+}
+
+} // extern "C"

@@ -1,0 +1,126 @@
+"""ctypes mirror of include/ppl_llm_kernel_hip.h (field order and types must match the header exactly)."""
+import ctypes as C
+
+RC_SUCCESS = 0
+RC_OTHER_ERROR = 1
+RC_UNSUPPORTED = 2
+RC_OUT_OF_MEMORY = 3
+RC_INVALID_VALUE = 4
+RC_EXISTS = 5
+RC_NOT_FOUND = 6
+RC_PERMISSION_DENIED = 7
+RC_HOST_MEMORY_ERROR = 8
+RC_DEVICE_MEMORY_ERROR = 9
+RC_DEVICE_RUNTIME_ERROR = 10
+RC_OUT_OF_RANGE = 11
+RC_INTERNAL_ERROR = 12
+
+RC_NAMES = {
+    0: "RC_SUCCESS", 1: "RC_OTHER_ERROR", 2: "RC_UNSUPPORTED", 3: "RC_OUT_OF_MEMORY", 4: "RC_INVALID_VALUE",
+    5: "RC_EXISTS", 6: "RC_NOT_FOUND", 7: "RC_PERMISSION_DENIED", 8: "RC_HOST_MEMORY_ERROR",
+    9: "RC_DEVICE_MEMORY_ERROR", 10: "RC_DEVICE_RUNTIME_ERROR", 11: "RC_OUT_OF_RANGE", 12: "RC_INTERNAL_ERROR",
+}
+
+_p = C.c_void_p
+_i32 = C.c_int32
+_i64 = C.c_int64
+
+
+class MhcaArgs(C.Structure):
+    _fields_ = [
+        ("d_query", _p), ("d_current_key", _p), ("d_current_value", _p), ("d_attn_mask", _p),
+        ("d_seqstarts", _p), ("d_kvstarts", _p), ("d_cachestarts", _p), ("d_start_pos", _p),
+        ("d_alibi_slopes", _p),
+        ("is_causal", _i32),
+        ("batch", _i64), ("decoding_batches", _i64), ("max_seqlen", _i64), ("max_kvlen", _i64),
+        ("layer_idx", _i32), ("num_layer", _i32), ("num_heads", _i32), ("num_kv_heads", _i32),
+        ("head_dim", _i32), ("cache_mode", _i32), ("page_size", _i32),
+        ("cache_stride_s", _i64), ("cache_stride_l", _i64), ("cache_stride_h", _i64), ("cache_stride_kv", _i64),
+        ("cachestart_stride_b", _i64),
+        ("enable_cache_prefill", _i32), ("enable_decoding_sharemem_mhca", _i32),
+        ("enable_decoding_infinity_mhca", _i32), ("enable_decoding_infinity_gqca", _i32),
+        ("specify_decoding_attn_split_k", _i32), ("specify_decoding_attn_tpb", _i32),
+        ("d_cache", _p), ("d_scale", _p), ("d_output", _p),
+        ("total_new_tokens", _i64),
+    ]
+
+
+class MhcaPlan(C.Structure):
+    _fields_ = [
+        ("workspace_bytes", C.c_uint64),
+        ("decode_chunk_tokens", _i32), ("decode_num_chunks", _i32), ("decode_waves_per_block", _i32),
+        ("prefill_q_tile", _i32), ("prefill_num_q_tiles", _i32),
+        ("reserved", _i32 * 3),
+    ]
+
+
+class KvWriteArgs(C.Structure):
+    _fields_ = [
+        ("d_current_key", _p), ("d_current_value", _p),
+        ("d_seqstarts", _p), ("d_cachestarts", _p), ("d_start_pos", _p),
+        ("batch", _i64), ("total_new_tokens", _i64),
+        ("layer_idx", _i32), ("num_layer", _i32), ("num_kv_heads", _i32), ("head_dim", _i32),
+        ("cache_stride_s", _i64), ("cache_stride_l", _i64), ("cache_stride_h", _i64), ("cache_stride_kv", _i64),
+        ("d_cache", _p), ("d_scale", _p),
+    ]
+
+
+class KvCacheArgs(C.Structure):
+    _fields_ = [
+        ("write", KvWriteArgs),
+        ("d_kvstarts", _p),
+        ("total_kv_tokens", _i64), ("max_kvlen", _i64),
+        ("num_repeat", _i32), ("cache_mode", _i32), ("cache_layout", _i32), ("reserved", _i32),
+        ("d_key_out", _p), ("d_value_out", _p),
+    ]
+
+
+class PackArgs(C.Structure):
+    _fields_ = [
+        ("d_slot_kvlen", _p), ("d_slot_newlen", _p), ("d_slot_cachestart", _p),
+        ("num_slots", _i32), ("reserved", _i32),
+        ("d_seqstarts", _p), ("d_kvstarts", _p), ("d_cachestarts", _p), ("d_start_pos", _p),
+        ("d_batch_slots", _p), ("d_header", _p),
+    ]
+
+
+# name -> (restype, argtypes); every symbol the header declares
+PROTOTYPES = {
+    "pplhip_last_error": (C.c_char_p, []),
+    "pplhip_version": (_i32, []),
+    "pplhip_mhca_prepare": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan)]),
+    "pplhip_mhca_forward": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan), _p, _p]),
+    "pplhip_kv_quantize_write": (_i32, [C.POINTER(KvWriteArgs), _p]),
+    "pplhip_kv_cache_forward": (_i32, [C.POINTER(KvCacheArgs), _p]),
+    "pplhip_pack_tables": (_i32, [C.POINTER(PackArgs), _p]),
+    "pplhip_advance_slots": (_i32, [_p, _p, _i32, _p]),
+}
+
+
+def bind(lib):
+    """Attach prototypes to a loaded CDLL; raises AttributeError when a declared symbol is missing."""
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def cache_strides_layout0(num_layer, num_kv_heads, head_dim):
+    """(MaxT, L, 2, KVH, Dh) strides, as computed at multi_head_cache_attention_kernel.cc:141-148."""
+    return dict(
+        cache_stride_s=num_layer * 2 * num_kv_heads * head_dim,
+        cache_stride_l=2 * num_kv_heads * head_dim,
+        cache_stride_h=head_dim,
+        cache_stride_kv=num_kv_heads * head_dim,
+    )
+
+
+def cache_strides_layout3(num_layer, num_kv_heads, head_dim, max_tokens):
+    """(L, 2, KVH, MaxT, Dh) strides, as computed at multi_head_cache_attention_kernel.cc:149-155."""
+    return dict(
+        cache_stride_s=head_dim,
+        cache_stride_l=2 * num_kv_heads * max_tokens * head_dim,
+        cache_stride_h=max_tokens * head_dim,
+        cache_stride_kv=num_kv_heads * max_tokens * head_dim,
+    )

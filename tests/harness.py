@@ -1,0 +1,159 @@
+"""Shared test plumbing: runs one MultiHeadCacheAttention call through the CPU oracle and through the HIP
+library's C ABI on the same seeded inputs. torch is used only to own device memory and the stream."""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import __graft_entry__ as entry  # noqa: E402
+
+pkg = entry.load_package()
+from ppl_nn_amd import cabi, workloads  # noqa: E402,F401
+
+ABS_TOL = 2e-3  # BASELINE.json: attention outputs within 2e-3 absolute / 1e-2 relative in fp16
+REL_TOL = 1e-2
+CACHE_FILL = 0x5A
+SCALE_FILL = 0x3C00
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def new_slab(b):
+    shape = (b.max_tokens, b.num_layer, 2, b.num_kv_heads, b.head_dim)
+    cache = np.full(shape, CACHE_FILL, dtype=np.int8)
+    scale = np.full(shape[:-1] + (b.head_dim // 8,), SCALE_FILL, dtype=np.uint16).view(np.float16)
+    return cache, scale
+
+
+def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, scale, ptr=_ptr):
+    st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
+    w.d_current_key, w.d_current_value = ptr(key), ptr(value)
+    w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(seqstarts), ptr(cachestarts), ptr(start_pos)
+    w.batch, w.total_new_tokens = b.batch, int(key.shape[0])
+    w.layer_idx, w.num_layer, w.num_kv_heads, w.head_dim = b.layer_idx, b.num_layer, b.num_kv_heads, b.head_dim
+    for k, v in st.items():
+        setattr(w, k, v)
+    w.d_cache, w.d_scale = ptr(cache), ptr(scale)
+    return w
+
+
+def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out, ptr=_ptr,
+                   cache_prefill=0, split_k=1):
+    st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
+    a.d_query, a.d_current_key, a.d_current_value = ptr(q), ptr(k), ptr(v)
+    a.d_attn_mask = None
+    a.d_alibi_slopes = None
+    a.d_seqstarts, a.d_kvstarts = ptr(seqstarts), ptr(kvstarts)
+    a.d_cachestarts, a.d_start_pos = ptr(cachestarts), ptr(start_pos)
+    a.is_causal = b.is_causal
+    a.batch, a.decoding_batches = b.batch, b.decoding_batches
+    a.max_seqlen, a.max_kvlen = b.max_seqlen, b.max_kvlen
+    a.layer_idx, a.num_layer = b.layer_idx, b.num_layer
+    a.num_heads, a.num_kv_heads, a.head_dim = b.num_heads, b.num_kv_heads, b.head_dim
+    a.cache_mode, a.page_size = 0, 128
+    for kk, vv in st.items():
+        setattr(a, kk, vv)
+    a.cachestart_stride_b = 0
+    a.enable_cache_prefill = cache_prefill
+    a.enable_decoding_sharemem_mhca = a.enable_decoding_infinity_mhca = a.enable_decoding_infinity_gqca = 1
+    a.specify_decoding_attn_split_k = split_k
+    a.specify_decoding_attn_tpb = 0
+    a.d_cache, a.d_scale, a.d_output = ptr(cache), ptr(scale), ptr(out)
+    a.total_new_tokens = b.total_new_tokens
+    return a
+
+
+def run_oracle(b, t, cache_prefill=0, want_f64=True):
+    """History write + MHCA on the CPU oracle. Returns cache (int8), scale (fp16), output (fp16), output_f64."""
+    import oracle
+    L = oracle.lib()
+    cache, scale = new_slab(b)
+    zeros = np.zeros(b.batch, np.int64)
+    if b.total_hist_tokens:
+        w = fill_write_args(cabi.KvWriteArgs(), b, t["hist_key"], t["hist_value"], b.histstarts, zeros,
+                            b.cachestarts, cache, scale)
+        assert L.oracle_kv_quantize_write(C.byref(w)) == 0
+    out = np.zeros((b.total_new_tokens, b.num_heads, b.head_dim), np.float16)
+    out64 = np.zeros(out.shape, np.float64) if want_f64 else None
+    seqstarts, kvstarts, sp = b.seqstarts, b.kvstarts, b.start_pos.copy()
+    a = fill_mhca_args(cabi.MhcaArgs(), b, t["query"], t["current_key"], t["current_value"], seqstarts, kvstarts,
+                       b.cachestarts, sp, cache, scale, out, cache_prefill=cache_prefill)
+    rc = L.oracle_mhca_forward(C.byref(a), _ptr(out64))
+    assert rc == 0, rc
+    return dict(cache=cache, scale=scale, output=out, output_f64=out64)
+
+
+def dev_ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def to_dev(a):
+    import torch
+    if a.dtype == np.float16:
+        return torch.from_numpy(a.view(np.int16).copy()).cuda().view(torch.float16)
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None):
+    """Same call through the C ABI on cuda:0."""
+    import torch
+    lib = pkg.load_library()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    cache_h, scale_h = new_slab(b)
+    cache, scale = to_dev(cache_h), to_dev(scale_h)
+    d = {k: to_dev(v) for k, v in t.items()}
+    tabs = dict(seqstarts=b.seqstarts, kvstarts=b.kvstarts, cachestarts=b.cachestarts, start_pos=b.start_pos,
+                histstarts=b.histstarts, zeros=np.zeros(max(b.batch, 1), np.int64))
+    dt = {k: to_dev(v) for k, v in tabs.items()}
+    if b.total_hist_tokens:
+        w = fill_write_args(cabi.KvWriteArgs(), b, d["hist_key"], d["hist_value"], dt["histstarts"], dt["zeros"],
+                            dt["cachestarts"], cache, scale, ptr=dev_ptr)
+        pkg.check(lib.pplhip_kv_quantize_write(C.byref(w), stream), "kv_quantize_write(history)")
+    out = torch.zeros((b.total_new_tokens, b.num_heads, b.head_dim), dtype=torch.float16, device="cuda")
+    a = fill_mhca_args(cabi.MhcaArgs(), b, d["query"], d["current_key"], d["current_value"], dt["seqstarts"],
+                       dt["kvstarts"], dt["cachestarts"], dt["start_pos"], cache, scale, out, ptr=dev_ptr,
+                       cache_prefill=cache_prefill, split_k=split_k)
+    plan = cabi.MhcaPlan()
+    pkg.check(lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)), "mhca_prepare")
+    ws = torch.empty(max(int(plan.workspace_bytes), 256), dtype=torch.uint8, device="cuda")
+    pkg.check(lib.pplhip_mhca_forward(C.byref(a), C.byref(plan), dev_ptr(ws), stream), "mhca_forward")
+    torch.cuda.synchronize()
+    if plan_out is not None:
+        plan_out.append(plan)
+    return dict(cache=cache.cpu().numpy(), scale=scale.cpu().view(torch.int16).numpy().view(np.float16),
+                output=out.cpu().view(torch.int16).numpy().view(np.float16))
+
+
+def assert_attn_close(got_f16, ref_f64, abs_tol=ABS_TOL, rel_tol=REL_TOL, what="attention output"):
+    got = got_f16.astype(np.float64)
+    assert np.isfinite(got).all(), f"{what}: non-finite values"
+    err = np.abs(got - ref_f64)
+    lim = abs_tol + rel_tol * np.abs(ref_f64)
+    bad = err > lim
+    if bad.any():
+        i = np.unravel_index(np.argmax(err - lim), err.shape)
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.size} elements outside {abs_tol} abs + {rel_tol} rel; "
+                             f"worst at {i}: got {got[i]}, want {ref_f64[i]}")
+    return float(err.max())
+
+
+def textbook_attention(q, k, v, causal_offset=None):
+    """float64 softmax(q k^T / sqrt(d) + mask) v for one head. q [Lq, d], k/v [Lk, d].
+    causal_offset: query row i sees keys j <= causal_offset + i (None = no mask)."""
+    q, k, v = (x.astype(np.float64) for x in (q, k, v))
+    s = q @ k.T / np.sqrt(q.shape[-1])
+    if causal_offset is not None:
+        i = np.arange(q.shape[0])[:, None]
+        j = np.arange(k.shape[0])[None, :]
+        s = np.where(j <= causal_offset + i, s, -np.inf)
+    s = s - s.max(axis=-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=-1, keepdims=True)
+    return p @ v

@@ -1,0 +1,196 @@
+"""Pins oracle_mhca_forward / oracle_kv_cache_forward / oracle_x86_attention against a float64 textbook
+softmax(QK^T/sqrt(d)+mask)V and closed forms, so a dropped term, wrong index or transposed operand fails."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness
+from harness import cabi, workloads
+
+
+def dequant_slab(cache, scale):
+    return cache.astype(np.float64) * np.repeat(scale.astype(np.float64), 8, axis=-1)
+
+
+def textbook_batch(b, t, res, cache_prefill=0):
+    """Expected outputs from the oracle's own slab (dequantised independently in numpy) and fp16 tensors."""
+    deq = dequant_slab(res["cache"], res["scale"])
+    out = np.zeros((b.total_new_tokens, b.num_heads, b.head_dim))
+    rep = b.num_heads // b.num_kv_heads
+    ss = b.seqstarts
+    for i in range(b.batch):
+        s0, L, sp, kv = ss[i], b.seqlens[i], b.start_pos[i], b.kvlens[i]
+        for h in range(b.num_heads):
+            kvh = h // rep
+            if i < b.decoding_batches or cache_prefill:
+                rows = slice(b.cachestarts[i], b.cachestarts[i] + kv)
+                k, v = deq[rows, b.layer_idx, 0, kvh], deq[rows, b.layer_idx, 1, kvh]
+            else:
+                k, v = t["current_key"][s0:s0 + L, kvh], t["current_value"][s0:s0 + L, kvh]
+            out[s0:s0 + L, h] = harness.textbook_attention(
+                t["query"][s0:s0 + L, h], k, v, causal_offset=sp if b.is_causal else None)
+    return out
+
+
+@pytest.mark.parametrize("H,KVH,Dh,L,li", [(4, 4, 128, 1, 0), (8, 2, 128, 2, 1), (6, 1, 64, 3, 2)])
+def test_mixed_batch_vs_textbook(H, KVH, Dh, L, li):
+    b = workloads.Batch(H, KVH, Dh, [1, 1, 1, 9, 33, 1], [40, 1, 17, 0, 0, 0], 3, num_layer=L, layer_idx=li,
+                        slack_tokens=3)
+    t = workloads.make_tensors(b, seed=H * 100 + KVH)
+    res = harness.run_oracle(b, t)
+    want = textbook_batch(b, t, res)
+    assert np.abs(res["output_f64"] - want).max() < 1e-12
+    assert np.array_equal(res["output"], want.astype(np.float32).astype(np.float16))
+    # other layers and the slack tokens keep their fill pattern
+    other = [l for l in range(L) if l != li]
+    assert (res["cache"][:, other] == harness.CACHE_FILL).all()
+    for i in range(b.batch):
+        end = b.cachestarts[i] + b.kvlens[i]
+        assert (res["cache"][end:end + b.slack_tokens] == harness.CACHE_FILL).all()
+
+
+def test_cache_prefill_and_chunked_start_pos():
+    b = workloads.Batch(4, 2, 128, [1, 20, 7], [12, 30, 0], 1, num_layer=1)
+    t = workloads.make_tensors(b, seed=9)
+    res = harness.run_oracle(b, t, cache_prefill=1)
+    want = textbook_batch(b, t, res, cache_prefill=1)
+    assert np.abs(res["output_f64"] - want).max() < 1e-12
+
+
+def test_non_causal():
+    b = workloads.Batch(2, 2, 64, [5, 8], [0, 0], 0, is_causal=0)
+    t = workloads.make_tensors(b, seed=4)
+    res = harness.run_oracle(b, t)
+    assert np.abs(res["output_f64"] - textbook_batch(b, t, res)).max() < 1e-12
+
+
+def test_closed_forms():
+    # kvlen == 1: output is exactly the (dequantised) value row
+    b = workloads.Batch(4, 2, 128, [1, 1], [0, 0], 0)
+    t = workloads.make_tensors(b, seed=1)
+    res = harness.run_oracle(b, t)
+    for s in range(2):
+        for h in range(4):
+            assert np.array_equal(res["output"][s, h], t["current_value"][s, h // 2])
+    # all keys equal -> uniform softmax -> mean of values (prefill, non causal)
+    b = workloads.Batch(2, 1, 64, [6], [0], 0, is_causal=0)
+    t = workloads.make_tensors(b, seed=2)
+    t["current_key"][:] = t["current_key"][0]
+    res = harness.run_oracle(b, t)
+    mean = t["current_value"][:, 0].astype(np.float64).mean(axis=0)
+    assert np.abs(res["output_f64"][:, 0] - mean).max() < 1e-12
+    # one dominant key: q = 30*k_3 direction makes key 3 win by a huge margin
+    b = workloads.Batch(1, 1, 128, [1], [7], 1)
+    t = workloads.make_tensors(b, seed=3)
+    t["hist_key"][3, 0] = np.float16(4.0)
+    t["query"][0, 0] = np.float16(8.0)
+    t["hist_key"][[0, 1, 2, 4, 5, 6], 0] = np.float16(-4.0)
+    t["current_key"][0, 0] = np.float16(-4.0)
+    res = harness.run_oracle(b, t)
+    deq = dequant_slab(res["cache"], res["scale"])
+    assert np.abs(res["output_f64"][0, 0] - deq[3, 0, 1, 0]).max() < 1e-9
+
+
+def test_gqa_equals_mha_with_repeated_heads():
+    bg = workloads.Batch(8, 2, 128, [1, 11], [25, 0], 1)
+    tg = workloads.make_tensors(bg, seed=21)
+    rg = harness.run_oracle(bg, tg)
+    bm = workloads.Batch(8, 8, 128, [1, 11], [25, 0], 1)
+    tm = dict(tg)
+    for k in ("current_key", "current_value", "hist_key", "hist_value"):
+        tm[k] = np.ascontiguousarray(np.repeat(tg[k], 4, axis=1))
+    rm = harness.run_oracle(bm, tm)
+    assert np.array_equal(rg["output"], rm["output"])
+
+
+def test_decode_equals_last_row_of_cache_prefill_and_permutation():
+    # decode over history == last row of a causal prefill that reads the same cache
+    bd = workloads.Batch(4, 2, 128, [1], [29], 1)
+    t = workloads.make_tensors(bd, seed=31)
+    rd = harness.run_oracle(bd, t)
+    bp = workloads.Batch(4, 2, 128, [30], [0], 0)
+    tp = dict(
+        query=np.concatenate([np.zeros((29, 4, 128), np.float16), t["query"]]),
+        current_key=np.concatenate([t["hist_key"], t["current_key"]]),
+        current_value=np.concatenate([t["hist_value"], t["current_value"]]),
+        hist_key=np.zeros((0, 2, 128), np.float16), hist_value=np.zeros((0, 2, 128), np.float16))
+    rp = harness.run_oracle(bp, tp, cache_prefill=1)
+    assert np.array_equal(rp["cache"], rd["cache"])
+    assert np.abs(rp["output_f64"][29] - rd["output_f64"][0]).max() < 1e-12
+    # permuting the sequences permutes the outputs
+    b1 = workloads.Batch(4, 4, 64, [1, 1, 1], [5, 9, 2], 3)
+    t1 = workloads.make_tensors(b1, seed=32)
+    r1 = harness.run_oracle(b1, t1)
+    perm = [2, 0, 1]
+    b2 = workloads.Batch(4, 4, 64, [1, 1, 1], b1.start_pos[perm], 3)
+    hs = b1.histstarts
+    t2 = {k: t1[k][perm] for k in ("query", "current_key", "current_value")}
+    for k in ("hist_key", "hist_value"):
+        t2[k] = np.concatenate([t1[k][hs[i]:hs[i + 1]] for i in perm])
+    r2 = harness.run_oracle(b2, t2)
+    assert np.array_equal(r2["output"], r1["output"][perm])
+
+
+def test_causal_ignores_future_tokens():
+    b = workloads.Batch(2, 1, 64, [10], [0], 0)
+    t = workloads.make_tensors(b, seed=41)
+    r0 = harness.run_oracle(b, t)
+    t2 = {k: v.copy() for k, v in t.items()}
+    t2["current_key"][6:] = np.nan
+    t2["current_value"][6:] = np.nan
+    r1 = harness.run_oracle(b, t2)
+    assert np.array_equal(r0["output"][:6], r1["output"][:6])
+
+
+def test_kv_cache_op(olib):
+    b = workloads.Batch(4, 2, 128, [1, 6, 1], [9, 0, 3], 0, num_layer=2, layer_idx=1, slack_tokens=2)
+    t = workloads.make_tensors(b, seed=51)
+    cache, scale = harness.new_slab(b)
+    zeros = np.zeros(b.batch, np.int64)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, t["hist_key"], t["hist_value"], b.histstarts, zeros,
+                                b.cachestarts, cache, scale)
+    assert olib.oracle_kv_quantize_write(C.byref(w)) == 0
+    a = cabi.KvCacheArgs()
+    seqstarts, kvstarts, sp = b.seqstarts, b.kvstarts, b.start_pos
+    harness.fill_write_args(a.write, b, t["current_key"], t["current_value"], seqstarts, sp, b.cachestarts, cache,
+                            scale)
+    a.d_kvstarts = kvstarts.ctypes.data
+    a.total_kv_tokens, a.max_kvlen = int(kvstarts[-1]), b.max_kvlen
+    a.num_repeat, a.cache_mode, a.cache_layout = 1, 0, 0
+    ko = np.zeros((int(kvstarts[-1]), 2, 128), np.float16)
+    vo = np.zeros_like(ko)
+    a.d_key_out, a.d_value_out = ko.ctypes.data, vo.ctypes.data
+    assert olib.oracle_kv_cache_forward(C.byref(a)) == 0
+    # rows come out in batch order: [history of seq b, new tokens of seq b]; error <= (1/2+1/32)*scale + fp16 rounding
+    hs = b.histstarts
+    for i in range(b.batch):
+        want_k = np.concatenate([t["hist_key"][hs[i]:hs[i + 1]], t["current_key"][seqstarts[i]:seqstarts[i + 1]]])
+        want_v = np.concatenate([t["hist_value"][hs[i]:hs[i + 1]], t["current_value"][seqstarts[i]:seqstarts[i + 1]]])
+        rows = slice(b.cachestarts[i], b.cachestarts[i] + b.kvlens[i])
+        sk = np.repeat(scale[rows, 1, 0].astype(np.float64), 8, axis=-1)
+        sv = np.repeat(scale[rows, 1, 1].astype(np.float64), 8, axis=-1)
+        gk, gv = ko[kvstarts[i]:kvstarts[i + 1]].astype(np.float64), vo[kvstarts[i]:kvstarts[i + 1]].astype(np.float64)
+        assert (np.abs(gk - want_k) <= 0.54 * sk + 2e-3 * np.abs(want_k)).all()
+        assert (np.abs(gv - want_v) <= 0.54 * sv + 2e-3 * np.abs(want_v)).all()
+    deq = dequant_slab(cache, scale)
+    i = 1
+    assert np.array_equal(ko[kvstarts[i]:kvstarts[i + 1]],
+                          deq[b.cachestarts[i]:b.cachestarts[i] + b.kvlens[i], 1, 0].astype(np.float32).astype(np.float16))
+    a.num_repeat = 2
+    assert olib.oracle_kv_cache_forward(C.byref(a)) == cabi.RC_UNSUPPORTED
+
+
+def test_x86_baseline_vs_textbook(olib):
+    """Config 0 of the baseline: 8 heads, head_dim 64, fp32, lengths {17, 64, 3, 128}, causal -inf mask."""
+    rng = np.random.default_rng(0)
+    for L in (17, 64, 3, 128):
+        q, k, v = (rng.standard_normal((8, L, 64)).astype(np.float32) for _ in range(3))
+        mask = np.where(np.arange(L)[None, :] <= np.arange(L)[:, None], 0, -np.inf).astype(np.float32)
+        out = np.empty_like(q)
+        rc = olib.oracle_x86_attention(q.ctypes.data, k.ctypes.data, v.ctypes.data, mask.ctypes.data,
+                                       out.ctypes.data, 8, 8, L, L, 64, 2)
+        assert rc == 0
+        for h in range(8):
+            want = harness.textbook_attention(q[h], k[h], v[h], causal_offset=0)
+            assert np.abs(out[h] - want).max() < 2e-5
