@@ -25,8 +25,28 @@ def load_library():
             raise LibraryMissing(
                 f"{LIB_PATH} is not built; run `python __graft_entry__.py` (hipcc, --offload-arch=gfx950). "
                 "There is no CPU fallback for the attention kernels.")
+        # The tests and the bench own device memory through torch, which ships its own HIP runtime under the
+        # same soname: load torch's first so that this library binds to that one runtime instead of a second copy.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _LIB = cabi.bind(ctypes.CDLL(LIB_PATH))
+        _assert_single_hip_runtime()
     return _LIB
+
+
+def _assert_single_hip_runtime():
+    paths = set()
+    try:
+        with open("/proc/self/maps") as f:
+            for line in f:
+                if "libamdhip64" in line:
+                    paths.add(os.path.realpath(line.split()[-1]))
+    except OSError:
+        return
+    if len(paths) > 1:
+        raise RuntimeError(f"two HIP runtimes are loaded in this process: {sorted(paths)}")
 
 
 def check(rc, what=""):

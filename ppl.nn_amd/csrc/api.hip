@@ -1,0 +1,224 @@
+// C ABI entry points: argument validation (same outcomes as the reference wrapper's checks), the split-k
+// heuristic, and the launch sequence write -> decode(+merge) -> prefill on the caller's stream.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace pplhip {
+
+static thread_local char g_last_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+}
+
+static int device_cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256; // MI355X
+    }
+    return cus;
+}
+
+static pplhip_retcode validate_common(int num_kv_heads, int head_dim, int num_layer, int layer_idx,
+                                      int64_t stride_s, int64_t stride_l, int64_t stride_h, int64_t stride_kv,
+                                      const void* cache, const void* scale) {
+    if (num_kv_heads <= 0 || num_layer <= 0 || layer_idx < 0 || layer_idx >= num_layer)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "bad num_kv_heads/num_layer/layer_idx (%d/%d/%d)", num_kv_heads,
+                    num_layer, layer_idx);
+    if (head_dim != 128)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: the gfx950 kernels are specialised for head_dim 128", head_dim);
+    if (!cache) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache pointer is null");
+    if (!scale)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support quantized cache but scale not found");
+    if (stride_s <= 0 || stride_s % 16 || stride_l % 16 || stride_h % 16 || stride_kv % 16)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache strides must be positive multiples of 16 elements");
+    if (((uintptr_t)cache & 15) || ((uintptr_t)scale & 15))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache and scale must be 16-byte aligned");
+    return PPLHIP_RC_SUCCESS;
+}
+
+static void write_args_from_mhca(const pplhip_mhca_args* a, pplhip_kv_write_args* w) {
+    memset(w, 0, sizeof(*w));
+    w->d_current_key = a->d_current_key;
+    w->d_current_value = a->d_current_value;
+    w->d_seqstarts = a->d_seqstarts;
+    w->d_cachestarts = a->d_cachestarts;
+    w->d_start_pos = a->d_start_pos;
+    w->batch = a->batch;
+    w->total_new_tokens = a->total_new_tokens;
+    w->layer_idx = a->layer_idx;
+    w->num_layer = a->num_layer;
+    w->num_kv_heads = a->num_kv_heads;
+    w->head_dim = a->head_dim;
+    w->cache_stride_s = a->cache_stride_s;
+    w->cache_stride_l = a->cache_stride_l;
+    w->cache_stride_h = a->cache_stride_h;
+    w->cache_stride_kv = a->cache_stride_kv;
+    w->d_cache = a->d_cache;
+    w->d_scale = a->d_scale;
+}
+
+static pplhip_retcode validate_write(const pplhip_kv_write_args* a) {
+    if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (a->batch < 0 || a->total_new_tokens < 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "negative batch or token count");
+    pplhip_retcode rc = validate_common(a->num_kv_heads, a->head_dim, a->num_layer, a->layer_idx, a->cache_stride_s,
+                                        a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->d_cache, a->d_scale);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    if (a->batch > 0 && a->total_new_tokens > 0) {
+        if (!a->d_current_key || !a->d_current_value || !a->d_seqstarts || !a->d_cachestarts || !a->d_start_pos)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
+        if (((uintptr_t)a->d_current_key & 15) || ((uintptr_t)a->d_current_value & 15))
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "current_key/current_value must be 16-byte aligned");
+    }
+    return PPLHIP_RC_SUCCESS;
+}
+
+} // namespace pplhip
+
+using namespace pplhip;
+
+extern "C" {
+
+const char* pplhip_last_error(void) {
+    return g_last_error;
+}
+
+int32_t pplhip_version(void) {
+    return 100; // 0.1.0
+}
+
+pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* plan) {
+    if (!a || !plan) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    memset(plan, 0, sizeof(*plan));
+    if (a->d_alibi_slopes) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support is_alibi == false");
+    if (a->d_attn_mask) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "attn_mask is not supported");
+    if (a->cache_mode != 0) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support cache_mode == 0");
+    if (a->num_heads <= 0 || a->num_kv_heads <= 0 || a->num_heads % a->num_kv_heads)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d is not a multiple of num_kv_heads %d", a->num_heads,
+                    a->num_kv_heads);
+    if (a->num_heads / a->num_kv_heads > 16)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "more than 16 query heads per kv head");
+    pplhip_retcode rc = validate_common(a->num_kv_heads, a->head_dim, a->num_layer, a->layer_idx, a->cache_stride_s,
+                                        a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->d_cache, a->d_scale);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    if (a->batch < 0 || a->decoding_batches < 0 || a->decoding_batches > a->batch || a->total_new_tokens < a->batch ||
+        a->max_seqlen < 0 || a->max_kvlen < a->max_seqlen)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE,
+                    "inconsistent batch sizes: batch %lld decoding_batches %lld tokens %lld max_seqlen %lld max_kvlen %lld",
+                    (long long)a->batch, (long long)a->decoding_batches, (long long)a->total_new_tokens,
+                    (long long)a->max_seqlen, (long long)a->max_kvlen);
+    if (a->batch > 0) {
+        if (!a->d_query || !a->d_current_key || !a->d_current_value || !a->d_seqstarts || !a->d_kvstarts ||
+            !a->d_cachestarts || !a->d_start_pos || !a->d_output)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
+        if (((uintptr_t)a->d_query & 15) || ((uintptr_t)a->d_current_key & 15) || ((uintptr_t)a->d_current_value & 15) ||
+            ((uintptr_t)a->d_output & 15))
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "query/current_key/current_value/output must be 16-byte aligned");
+    }
+    if (a->specify_decoding_attn_split_k < 0 || a->specify_decoding_attn_split_k > 2)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_split_k must be 0, 1 or 2");
+    if (a->specify_decoding_attn_tpb != 0 && a->specify_decoding_attn_tpb != 256 && a->specify_decoding_attn_tpb != 512)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_tpb must be 0, 256 or 512");
+
+    // ---- decode: split the cached tokens into chunks so that the chip sees a few tasks per wave slot
+    plan->decode_waves_per_block = 4;
+    const int64_t nd = a->decoding_batches;
+    if (nd > 0 && a->max_kvlen > 0) {
+        const int64_t round = 64; // the kernel's inner block
+        int64_t chunk;
+        const int64_t whole = (a->max_kvlen + round - 1) / round * round;
+        if (a->specify_decoding_attn_split_k == 0) {
+            chunk = whole;
+        } else {
+            const int64_t slots = (int64_t)device_cu_count() * 8; // 2 waves per SIMD
+            const int64_t pairs = nd * a->num_kv_heads;
+            // aim at ~3 tasks per slot if every sequence were max_kvlen long (ragged batches average about half)
+            chunk = (a->max_kvlen * pairs + 3 * slots - 1) / (3 * slots);
+            chunk = (chunk + round - 1) / round * round;
+            if (chunk < 256) chunk = 256;
+            if (chunk > whole) chunk = whole;
+            if (a->specify_decoding_attn_split_k == 2 && chunk >= whole && whole > round)
+                chunk = (whole / 2 + round - 1) / round * round;
+        }
+        plan->decode_chunk_tokens = (int32_t)chunk;
+        plan->decode_num_chunks = (int32_t)((a->max_kvlen + chunk - 1) / chunk);
+        if (plan->decode_num_chunks > 1) {
+            const uint64_t rows = (uint64_t)nd * plan->decode_num_chunks * a->num_heads;
+            plan->workspace_bytes = rows * (a->head_dim + 2) * sizeof(float);
+        }
+    }
+    // ---- prefill
+    plan->prefill_q_tile = 128;
+    if (a->batch > a->decoding_batches)
+        plan->prefill_num_q_tiles = (int32_t)((a->max_seqlen + plan->prefill_q_tile - 1) / plan->prefill_q_tile);
+    plan->workspace_bytes = (plan->workspace_bytes + 255) / 256 * 256;
+    return PPLHIP_RC_SUCCESS;
+}
+
+pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* d_workspace,
+                                   void* stream) {
+    if (!a || !plan) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (a->batch == 0) return PPLHIP_RC_SUCCESS;
+    if (plan->workspace_bytes > 0 && (!d_workspace || ((uintptr_t)d_workspace & 255)))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "workspace of %llu bytes (256-byte aligned) required",
+                    (unsigned long long)plan->workspace_bytes);
+    if (a->decoding_batches > 0 && plan->decode_chunk_tokens <= 0)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
+    hipStream_t s = (hipStream_t)stream;
+    pplhip_kv_write_args w;
+    write_args_from_mhca(a, &w);
+    pplhip_retcode rc = launch_kv_quantize_write(&w, s);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    rc = launch_decode(a, plan, d_workspace, s);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    return launch_prefill(a, plan, s);
+}
+
+pplhip_retcode pplhip_kv_quantize_write(const pplhip_kv_write_args* a, void* stream) {
+    pplhip_retcode rc = validate_write(a);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    return launch_kv_quantize_write(a, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_kv_cache_forward(const pplhip_kv_cache_args* a, void* stream) {
+    if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (a->cache_layout != 0) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support cache_layout == 0");
+    if (a->cache_mode != 0) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support cache_mode == 0");
+    if (a->num_repeat != 1) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support num_repeat == 1");
+    pplhip_retcode rc = validate_write(&a->write);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    if (a->total_kv_tokens < 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "negative total_kv_tokens");
+    if (a->total_kv_tokens > 0 && (!a->d_kvstarts || !a->d_key_out || !a->d_value_out))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
+    if (((uintptr_t)a->d_key_out & 15) || ((uintptr_t)a->d_value_out & 15))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "key/value outputs must be 16-byte aligned");
+    rc = launch_kv_quantize_write(&a->write, (hipStream_t)stream);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    return launch_kv_gather_dequant(a, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_pack_tables(const pplhip_pack_args* a, void* stream) {
+    if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (!a->d_slot_kvlen || !a->d_slot_newlen || !a->d_slot_cachestart || !a->d_seqstarts || !a->d_kvstarts ||
+        !a->d_cachestarts || !a->d_start_pos || !a->d_batch_slots || !a->d_header)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null table pointer");
+    return launch_pack_tables(a, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot_newlen, int32_t num_slots,
+                                    void* stream) {
+    if (num_slots < 0 || (num_slots > 0 && (!d_slot_kvlen || !d_slot_newlen)))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "bad slot arrays");
+    return launch_advance_slots(d_slot_kvlen, d_slot_newlen, num_slots, (hipStream_t)stream);
+}
+
+} // extern "C"

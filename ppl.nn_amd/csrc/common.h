@@ -1,0 +1,75 @@
+// Shared host/device helpers of the gfx950 kernel library (internal; the public surface is the C ABI header).
+#ifndef PPLHIP_CSRC_COMMON_H_
+#define PPLHIP_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/ppl_llm_kernel_hip.h"
+
+namespace pplhip {
+
+// thread-local text behind pplhip_last_error()
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define PPLHIP_FAIL(rc, ...)              \
+    do {                                  \
+        ::pplhip::set_error(__VA_ARGS__); \
+        return (rc);                      \
+    } while (0)
+
+#define PPLHIP_CHECK_LAUNCH(what)                                                                 \
+    do {                                                                                          \
+        hipError_t e_ = hipGetLastError();                                                        \
+        if (e_ != hipSuccess)                                                                     \
+            PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "%s: %s", (what), hipGetErrorString(e_)); \
+    } while (0)
+
+constexpr int kQuantGroup = 8;
+constexpr int kWave = 64;
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// Where one KV head's row of `head_dim` int8 channels starts, and the matching row of head_dim/8 fp16 scales.
+struct CacheAddr {
+    int64_t stride_s, stride_l, stride_h, stride_kv;
+    int32_t layer;
+    __host__ __device__ inline int64_t row(int64_t tok, int kv, int head) const {
+        return tok * stride_s + (int64_t)layer * stride_l + (int64_t)kv * stride_kv + (int64_t)head * stride_h;
+    }
+};
+
+// first index b in [0, n) with starts[b+1] > x  (starts is a non-decreasing prefix-sum table with n+1 entries)
+__device__ inline int find_sequence(const int64_t* __restrict__ starts, int n, int64_t x) {
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (starts[mid + 1] > x)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    return lo;
+}
+
+inline int ceil_div(int64_t a, int64_t b) {
+    return (int)((a + b - 1) / b);
+}
+
+// launchers implemented in the .hip files
+pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream);
+pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream_t stream);
+pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
+pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, hipStream_t stream);
+pplhip_retcode launch_pack_tables(const pplhip_pack_args* a, hipStream_t stream);
+pplhip_retcode launch_advance_slots(int64_t* kvlen, const int64_t* newlen, int n, hipStream_t stream);
+
+} // namespace pplhip
+
+#endif

@@ -1,0 +1,143 @@
+// On-device rebuild of the ragged-batch tables (seqstarts / kvstarts / cachestarts / start_pos) from per-slot
+// state: stable compaction with decode sequences first, then prefill sequences, then prefix sums and maxima.
+// At most 1024 slots, so one workgroup does everything in LDS; the kernel is latency-bound (a few microseconds)
+// and replaces eight host-to-device uploads per step.
+#include "common.h"
+
+namespace pplhip {
+
+constexpr int kMaxSlots = 1024;
+
+struct PackParams {
+    const int64_t* slot_kvlen;
+    const int64_t* slot_newlen;
+    const int64_t* slot_cachestart;
+    int64_t* seqstarts;
+    int64_t* kvstarts;
+    int64_t* cachestarts;
+    int64_t* start_pos;
+    int64_t* batch_slots;
+    int64_t* header;
+    int32_t n;
+};
+
+// Inclusive scan of one int64 per thread across the workgroup (Hillis-Steele in LDS, ping-pong buffers).
+__device__ inline int64_t block_inclusive_scan(int64_t v, int64_t* buf /* 2 * kMaxSlots */, int nthreads) {
+    const int tid = threadIdx.x;
+    int cur = 0;
+    buf[tid] = v;
+    __syncthreads();
+    for (int off = 1; off < nthreads; off <<= 1) {
+        int64_t x = buf[cur * kMaxSlots + tid];
+        if (tid >= off) x += buf[cur * kMaxSlots + tid - off];
+        cur ^= 1;
+        buf[cur * kMaxSlots + tid] = x;
+        __syncthreads();
+    }
+    const int64_t r = buf[cur * kMaxSlots + tid];
+    __syncthreads();
+    return r;
+}
+
+__device__ inline int64_t block_max(int64_t v, int64_t* buf, int nthreads) {
+    const int tid = threadIdx.x;
+    buf[tid] = v;
+    __syncthreads();
+    for (int off = kMaxSlots / 2; off > 0; off >>= 1) {
+        if (tid < off && tid + off < nthreads) buf[tid] = buf[tid] > buf[tid + off] ? buf[tid] : buf[tid + off];
+        __syncthreads();
+    }
+    const int64_t r = buf[0];
+    __syncthreads();
+    return r;
+}
+
+__global__ __launch_bounds__(kMaxSlots) void pack_tables_kernel(const PackParams p) {
+    __shared__ int64_t scan_buf[2 * kMaxSlots];
+    __shared__ int64_t packed_new[kMaxSlots];
+    __shared__ int64_t packed_kv[kMaxSlots];
+    const int tid = threadIdx.x;
+    const int nt = blockDim.x;
+    const bool in = tid < p.n;
+    const int64_t kl = in ? p.slot_kvlen[tid] : 0;
+    const int64_t nl = in ? p.slot_newlen[tid] : 0;
+    const bool active = nl > 0;
+    const bool is_decode = active && nl == 1 && kl > 0;
+    const bool is_prefill = active && !is_decode;
+
+    const int64_t dec_incl = block_inclusive_scan(is_decode ? 1 : 0, scan_buf, nt);
+    const int64_t pre_incl = block_inclusive_scan(is_prefill ? 1 : 0, scan_buf, nt);
+    __shared__ int64_t totals[2];
+    if (tid == nt - 1) {
+        totals[0] = dec_incl;
+        totals[1] = pre_incl;
+    }
+    packed_new[tid] = 0;
+    packed_kv[tid] = 0;
+    __syncthreads();
+    const int64_t nd = totals[0];
+    const int64_t batch = nd + totals[1];
+    int64_t pos = -1;
+    if (is_decode) pos = dec_incl - 1;
+    if (is_prefill) pos = nd + pre_incl - 1;
+    if (pos >= 0) {
+        packed_new[pos] = nl;
+        packed_kv[pos] = kl + nl;
+        p.cachestarts[pos] = p.slot_cachestart[tid];
+        p.start_pos[pos] = kl;
+        p.batch_slots[pos] = tid;
+    }
+    __syncthreads();
+    const int64_t my_new = packed_new[tid], my_kv = packed_kv[tid];
+    const int64_t seq_incl = block_inclusive_scan(my_new, scan_buf, nt);
+    const int64_t kv_incl = block_inclusive_scan(my_kv, scan_buf, nt);
+    const int64_t max_new = block_max(my_new, scan_buf, nt);
+    const int64_t max_kv = block_max(my_kv, scan_buf, nt);
+    if (tid < p.n) {
+        p.seqstarts[tid + 1] = seq_incl; // entries past the batch repeat the total (their packed lengths are 0)
+        p.kvstarts[tid + 1] = kv_incl;
+        if (tid >= batch) {
+            p.cachestarts[tid] = 0;
+            p.start_pos[tid] = 0;
+            p.batch_slots[tid] = -1;
+        }
+    }
+    if (tid == 0) {
+        p.seqstarts[0] = 0;
+        p.kvstarts[0] = 0;
+    }
+    if (tid == nt - 1) {
+        p.header[0] = batch;
+        p.header[1] = nd;
+        p.header[2] = max_new;
+        p.header[3] = max_kv;
+        p.header[4] = seq_incl;
+        p.header[5] = kv_incl;
+    }
+}
+
+pplhip_retcode launch_pack_tables(const pplhip_pack_args* a, hipStream_t stream) {
+    if (a->num_slots <= 0 || a->num_slots > kMaxSlots)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "pack_tables: num_slots %d outside [1, %d]", a->num_slots, kMaxSlots);
+    PackParams p{a->d_slot_kvlen, a->d_slot_newlen, a->d_slot_cachestart, a->d_seqstarts, a->d_kvstarts,
+                 a->d_cachestarts, a->d_start_pos, a->d_batch_slots, a->d_header, a->num_slots};
+    int threads = 64;
+    while (threads < a->num_slots) threads <<= 1;
+    hipLaunchKernelGGL(pack_tables_kernel, dim3(1), dim3(threads), 0, stream, p);
+    PPLHIP_CHECK_LAUNCH("pack_tables");
+    return PPLHIP_RC_SUCCESS;
+}
+
+__global__ void advance_slots_kernel(int64_t* kvlen, const int64_t* newlen, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && newlen[i] > 0) kvlen[i] += newlen[i];
+}
+
+pplhip_retcode launch_advance_slots(int64_t* kvlen, const int64_t* newlen, int n, hipStream_t stream) {
+    if (n <= 0) return PPLHIP_RC_SUCCESS;
+    hipLaunchKernelGGL(advance_slots_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, kvlen, newlen, n);
+    PPLHIP_CHECK_LAUNCH("advance_slots");
+    return PPLHIP_RC_SUCCESS;
+}
+
+} // namespace pplhip

@@ -1,0 +1,108 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares, the ctypes
+mirrors match the header's field lists, and host-only validation returns the reference's error codes."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import harness
+from harness import cabi, workloads
+
+HEADER = os.path.join(harness.ROOT, "include", "ppl_llm_kernel_hip.h")
+
+
+def header_text():
+    with open(HEADER) as f:
+        return f.read()
+
+
+def test_library_exports_every_declared_symbol(hiplib):
+    txt = re.sub(r"/\*.*?\*/", "", header_text(), flags=re.S)
+    declared = set(re.findall(r"\b(pplhip_[a-z0-9_]+)\s*\(", txt))
+    assert declared == set(cabi.PROTOTYPES), declared ^ set(cabi.PROTOTYPES)
+    for name in declared:
+        assert hasattr(hiplib, name)
+    assert hiplib.pplhip_version() >= 100
+    assert hiplib.pplhip_last_error() is not None
+
+
+@pytest.mark.parametrize("cname,cls", [("pplhip_mhca_args", cabi.MhcaArgs), ("pplhip_mhca_plan", cabi.MhcaPlan),
+                                       ("pplhip_kv_write_args", cabi.KvWriteArgs),
+                                       ("pplhip_kv_cache_args", cabi.KvCacheArgs), ("pplhip_pack_args", cabi.PackArgs)])
+def test_ctypes_mirror_matches_header(cname, cls):
+    txt = re.sub(r"/\*.*?\*/", "", header_text(), flags=re.S)
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), txt, flags=re.S).group(1)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        names.append(re.sub(r"\[.*\]", "", decl.split()[-1].lstrip("*")))
+    assert names == [f[0] for f in cls._fields_]
+
+
+def _valid_args():
+    b = workloads.Batch(8, 2, 128, [1, 5], [10, 0], 1)
+    a = cabi.MhcaArgs()
+    fake = lambda t: C.c_void_p(0x1000)  # prepare never dereferences device pointers
+    harness.fill_mhca_args(a, b, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, ptr=fake)
+    return a
+
+
+def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
+    a, plan = _valid_args(), cabi.MhcaPlan()
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+    assert plan.decode_chunk_tokens >= 11 and plan.decode_chunk_tokens % 64 == 0
+    assert plan.decode_num_chunks == 1 and plan.workspace_bytes == 0
+    assert plan.prefill_q_tile == 128 and plan.prefill_num_q_tiles == 1
+    a.max_kvlen, a.specify_decoding_attn_split_k = 100000, 2
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+    assert plan.decode_num_chunks * plan.decode_chunk_tokens >= 100000 and plan.decode_num_chunks > 1
+    assert plan.workspace_bytes >= 1 * plan.decode_num_chunks * 8 * 130 * 4 and plan.workspace_bytes % 256 == 0
+
+
+@pytest.mark.parametrize("mutate,rc", [
+    (lambda a: setattr(a, "d_alibi_slopes", 0x10), cabi.RC_UNSUPPORTED),  # …_kernel.cc:95-98
+    (lambda a: setattr(a, "d_scale", None), cabi.RC_UNSUPPORTED),  # …_kernel.cc:100-103
+    (lambda a: setattr(a, "d_attn_mask", 0x10), cabi.RC_UNSUPPORTED),
+    (lambda a: setattr(a, "cache_mode", 1), cabi.RC_UNSUPPORTED),
+    (lambda a: setattr(a, "head_dim", 64), cabi.RC_UNSUPPORTED),
+    (lambda a: setattr(a, "num_kv_heads", 3), cabi.RC_INVALID_VALUE),
+    (lambda a: setattr(a, "layer_idx", 5), cabi.RC_INVALID_VALUE),
+    (lambda a: setattr(a, "decoding_batches", 3), cabi.RC_INVALID_VALUE),
+    (lambda a: setattr(a, "cache_stride_s", 100), cabi.RC_INVALID_VALUE),
+    (lambda a: setattr(a, "d_query", None), cabi.RC_INVALID_VALUE),
+    (lambda a: setattr(a, "specify_decoding_attn_split_k", 7), cabi.RC_INVALID_VALUE),
+    (lambda a: setattr(a, "specify_decoding_attn_tpb", 128), cabi.RC_INVALID_VALUE),
+])
+def test_prepare_rejects(hiplib, mutate, rc):
+    a, plan = _valid_args(), cabi.MhcaPlan()
+    mutate(a)
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == rc
+    assert len(hiplib.pplhip_last_error()) > 0
+
+
+def test_kv_cache_rejects_like_the_reference_stub(hiplib):
+    # key_value_cache_kernel.cc:73-96: layout != 0, mode != 0, num_repeat != 1 -> RC_UNSUPPORTED
+    for field in ("cache_layout", "cache_mode", "num_repeat"):
+        a = cabi.KvCacheArgs()
+        a.num_repeat = 1
+        setattr(a, field, 3)
+        assert hiplib.pplhip_kv_cache_forward(C.byref(a), None) == cabi.RC_UNSUPPORTED
+
+
+def test_pack_rejects_bad_slot_count(hiplib):
+    a = cabi.PackArgs()
+    for f, _ in cabi.PackArgs._fields_:
+        if f.startswith("d_"):
+            setattr(a, f, 0x1000)
+    a.num_slots = 5000
+    assert hiplib.pplhip_pack_tables(C.byref(a), None) == cabi.RC_INVALID_VALUE
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(harness.pkg, "_LIB", None)
+    monkeypatch.setattr(harness.pkg, "LIB_PATH", "/nonexistent/libppl_llm_kernel_hip.so")
+    with pytest.raises(harness.pkg.LibraryMissing):
+        harness.pkg.load_library()

@@ -1,0 +1,206 @@
+"""GPU parity tests: every call goes through the C ABI of the HIP library and is compared with the CPU oracle on
+the same seeded inputs. int8 cache bytes and fp16 scales must match bit-exactly; attention outputs must be within
+2e-3 absolute + 1e-2 relative of the oracle's float64 result."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness
+from harness import cabi, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def check(b, t, cache_prefill=0, split_k=1, plans=None):
+    print(f"case {b.name} H={b.num_heads} KVH={b.num_kv_heads} B={b.batch} nd={b.decoding_batches} "
+          f"S={b.total_new_tokens} hist={b.total_hist_tokens} split_k={split_k} cache_prefill={cache_prefill}",
+          flush=True)
+    ref = harness.run_oracle(b, t, cache_prefill=cache_prefill)
+    got = harness.run_device(b, t, cache_prefill=cache_prefill, split_k=split_k, plan_out=plans)
+    assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
+    assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
+    return harness.assert_attn_close(got["output"], ref["output_f64"]), ref, got
+
+
+def test_quantize_write_all_finite_absmax_bit_exact(hiplib, olib):
+    """Every non-negative finite fp16 as a group's absmax, with tie-prone companions, through the write kernel."""
+    import torch
+    finite = np.arange(0, 0x7c00, dtype=np.uint16).view(np.float16)
+    a32 = finite.astype(np.float32)
+    rng = np.random.default_rng(3)
+    cols = [finite, -finite] + [(a32 * np.float32((k + 0.5) / 127.0)).astype(np.float16) for k in (0, 1, 63, 125, 126)]
+    cols.append((a32 * rng.uniform(-1, 1, a32.size).astype(np.float32)).astype(np.float16))
+    groups = np.stack(cols, axis=1)  # [31744, 8]
+    n_tok = groups.shape[0] // 16  # 16 groups per 128-channel head row
+    key = np.ascontiguousarray(groups[:n_tok * 16].reshape(n_tok, 1, 128))
+    val = np.ascontiguousarray(-key[::-1])
+    b = workloads.Batch(1, 1, 128, [n_tok], [0], 0)
+    cache_o, scale_o = harness.new_slab(b)
+    zeros = np.zeros(1, np.int64)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, key, val, b.seqstarts, zeros, b.cachestarts, cache_o, scale_o)
+    assert olib.oracle_kv_quantize_write(C.byref(w)) == 0
+    cache_d, scale_d = harness.to_dev(harness.new_slab(b)[0]), harness.to_dev(harness.new_slab(b)[1])
+    kd, vd = harness.to_dev(key), harness.to_dev(val)
+    ss, cs, sp = harness.to_dev(b.seqstarts), harness.to_dev(b.cachestarts), harness.to_dev(zeros)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, kd, vd, ss, sp, cs, cache_d, scale_d, ptr=harness.dev_ptr)
+    harness.pkg.check(hiplib.pplhip_kv_quantize_write(C.byref(w), None), "kv_quantize_write")
+    torch.cuda.synchronize()
+    assert np.array_equal(cache_d.cpu().numpy(), cache_o)
+    assert np.array_equal(scale_d.cpu().view(torch.int16).numpy().view(np.uint16), scale_o.view(np.uint16))
+
+
+@pytest.mark.parametrize("H,KVH", [(4, 4), (8, 2), (8, 1), (32, 8), (16, 1), (40, 40)])
+def test_small_mixed_batches(H, KVH):
+    b = workloads.Batch(H, KVH, 128, [1, 1, 1, 1, 9, 130, 64, 1], [40, 0 + 1, 300, 63, 0, 0, 0, 0], 4,
+                        num_layer=2, layer_idx=1, slack_tokens=3, name="small_mixed")
+    t = workloads.make_tensors(b, seed=H * 100 + KVH)
+    check(b, t)
+
+
+def test_decode_only_and_prefill_only_and_layer_strides():
+    b = workloads.Batch(8, 2, 128, [1] * 7, [1, 15, 16, 17, 63, 64, 65], 7, num_layer=3, layer_idx=0, name="decode_only")
+    check(b, workloads.make_tensors(b, seed=1))
+    b = workloads.Batch(8, 2, 128, [1, 2, 31, 32, 33, 127, 128, 129, 257], [0] * 9, 0, num_layer=3, layer_idx=2,
+                        name="prefill_only")
+    check(b, workloads.make_tensors(b, seed=2))
+
+
+def test_prefill_non_causal():
+    b = workloads.Batch(4, 2, 128, [70, 5, 200], [0, 0, 0], 0, is_causal=0, name="non_causal")
+    check(b, workloads.make_tensors(b, seed=3))
+
+
+def test_cache_prefill_with_start_pos():
+    b = workloads.Batch(8, 4, 128, [1, 20, 130, 7], [12, 30, 100, 0], 1, name="cache_prefill")
+    check(b, workloads.make_tensors(b, seed=4), cache_prefill=1)
+
+
+def test_split_k_modes_agree():
+    """Split count must not change the result beyond fp32 reassociation."""
+    b = workloads.Batch(8, 2, 128, [1, 1, 1], [2999, 700, 64], 3, name="split_k")
+    t = workloads.make_tensors(b, seed=5)
+    outs, plans = [], []
+    for mode in (0, 1, 2):
+        _, ref, got = check(b, t, split_k=mode, plans=plans)
+        outs.append(got["output"].astype(np.float64))
+    assert plans[0].decode_num_chunks == 1 and plans[2].decode_num_chunks > 1
+    assert np.abs(outs[0] - outs[1]).max() < 1e-3 and np.abs(outs[0] - outs[2]).max() < 1e-3
+
+
+def test_closed_forms_on_device():
+    # kv length 1: output is exactly the dequantised value row (softmax over one key)
+    b = workloads.Batch(8, 2, 128, [1, 1], [0, 0], 0, name="kvlen1_prefill")
+    t = workloads.make_tensors(b, seed=6)
+    got = harness.run_device(b, t)
+    for s in range(2):
+        for h in range(8):
+            assert np.array_equal(got["output"][s, h], t["current_value"][s, h // 4])
+    # poisoned future tokens must not leak into causal rows (finite poison: masked probabilities are exact zeros,
+    # and 0 * finite = 0 in the PV product; NaN/Inf inputs are outside the op's contract)
+    b = workloads.Batch(2, 1, 128, [100], [0], 0, name="causal_poison")
+    t = workloads.make_tensors(b, seed=7)
+    clean = harness.run_device(b, t)["output"]
+    t["current_key"][60:] = np.float16(6e4)
+    t["current_value"][60:] = np.float16(-6e4)
+    dirty = harness.run_device(b, t)["output"]
+    assert np.array_equal(clean[:60], dirty[:60])
+
+
+def test_decode_equals_last_row_of_cache_prefill_on_device():
+    bd = workloads.Batch(8, 2, 128, [1], [199], 1, name="decode_vs_prefill")
+    t = workloads.make_tensors(bd, seed=8)
+    d = harness.run_device(bd, t)
+    bp = workloads.Batch(8, 2, 128, [200], [0], 0)
+    tp = dict(query=np.concatenate([np.zeros((199, 8, 128), np.float16), t["query"]]),
+              current_key=np.concatenate([t["hist_key"], t["current_key"]]),
+              current_value=np.concatenate([t["hist_value"], t["current_value"]]),
+              hist_key=np.zeros((0, 2, 128), np.float16), hist_value=np.zeros((0, 2, 128), np.float16))
+    pr = harness.run_device(bp, tp, cache_prefill=1)
+    assert np.array_equal(pr["cache"], d["cache"])
+    assert np.abs(pr["output"][199].astype(np.float64) - d["output"][0].astype(np.float64)).max() < 2e-3
+
+
+def test_kv_cache_op(hiplib, olib):
+    import torch
+    b = workloads.Batch(4, 4, 128, [1, 6, 1, 40], [9, 0, 3, 0], 0, num_layer=2, layer_idx=1, slack_tokens=2)
+    t = workloads.make_tensors(b, seed=9)
+    zeros = np.zeros(b.batch, np.int64)
+    total_kv = int(b.kvstarts[-1])
+
+    def run(lib_write, lib_fwd, ptr, conv, stream_args):
+        cache, scale = harness.new_slab(b)
+        cache, scale = conv(cache), conv(scale)
+        tt = {k: conv(v) for k, v in t.items()}
+        tabs = {k: conv(v) for k, v in dict(hs=b.histstarts, z=zeros, cs=b.cachestarts, ss=b.seqstarts,
+                                            ks=b.kvstarts, sp=b.start_pos).items()}
+        w = harness.fill_write_args(cabi.KvWriteArgs(), b, tt["hist_key"], tt["hist_value"], tabs["hs"], tabs["z"],
+                                    tabs["cs"], cache, scale, ptr=ptr)
+        assert lib_write(C.byref(w), *stream_args) == 0
+        a = cabi.KvCacheArgs()
+        harness.fill_write_args(a.write, b, tt["current_key"], tt["current_value"], tabs["ss"], tabs["sp"], tabs["cs"],
+                                cache, scale, ptr=ptr)
+        a.d_kvstarts = ptr(tabs["ks"])
+        a.total_kv_tokens, a.max_kvlen = total_kv, b.max_kvlen
+        a.num_repeat, a.cache_mode, a.cache_layout = 1, 0, 0
+        ko = conv(np.zeros((total_kv, 4, 128), np.float16))
+        vo = conv(np.zeros((total_kv, 4, 128), np.float16))
+        a.d_key_out, a.d_value_out = ptr(ko), ptr(vo)
+        assert lib_fwd(C.byref(a), *stream_args) == 0
+        return cache, scale, ko, vo
+
+    co, so, ko, vo = run(lambda w: olib.oracle_kv_quantize_write(w), lambda a: olib.oracle_kv_cache_forward(a),
+                         harness._ptr, lambda x: np.ascontiguousarray(x).copy(), ())
+    cd, sd, kd, vd = run(hiplib.pplhip_kv_quantize_write, hiplib.pplhip_kv_cache_forward, harness.dev_ptr,
+                         harness.to_dev, (None,))
+    torch.cuda.synchronize()
+    f16 = lambda x: x.cpu().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(cd.cpu().numpy(), co) and np.array_equal(f16(sd), so.view(np.uint16))
+    assert np.array_equal(f16(kd), ko.view(np.uint16)) and np.array_equal(f16(vd), vo.view(np.uint16))
+
+
+def test_pack_tables_random_and_churn(hiplib, olib):
+    import torch
+    import test_oracle_pack as top
+
+    def dev_pack(a_ptr):
+        return hiplib.pplhip_pack_tables(a_ptr, None)
+
+    def run_dev(kvlen, newlen, cs):
+        n = len(kvlen)
+        d = dict(kv=harness.to_dev(kvlen), nl=harness.to_dev(newlen), cs=harness.to_dev(cs))
+        out = {k: torch.full((m,), -7, dtype=torch.int64, device="cuda") for k, m in
+               dict(seqstarts=n + 1, kvstarts=n + 1, cachestarts=n, start_pos=n, batch_slots=n, header=6).items()}
+        a = cabi.PackArgs()
+        a.d_slot_kvlen, a.d_slot_newlen, a.d_slot_cachestart = d["kv"].data_ptr(), d["nl"].data_ptr(), d["cs"].data_ptr()
+        a.num_slots = n
+        a.d_seqstarts, a.d_kvstarts = out["seqstarts"].data_ptr(), out["kvstarts"].data_ptr()
+        a.d_cachestarts, a.d_start_pos = out["cachestarts"].data_ptr(), out["start_pos"].data_ptr()
+        a.d_batch_slots, a.d_header = out["batch_slots"].data_ptr(), out["header"].data_ptr()
+        harness.pkg.check(hiplib.pplhip_pack_tables(C.byref(a), None), "pack_tables")
+        torch.cuda.synchronize()
+        return {k: v.cpu().numpy() for k, v in out.items()}
+
+    rng = np.random.default_rng(12)
+    for n in (1, 2, 63, 64, 65, 256, 1000, 1024):
+        for _ in range(3):
+            kvlen = (rng.integers(0, 50, n) * (rng.random(n) < 0.7)).astype(np.int64)
+            newlen = np.where(rng.random(n) < 0.2, 0, np.where(kvlen > 0, 1, rng.integers(1, 40, n))).astype(np.int64)
+            newlen = np.where(rng.random(n) < 0.05, rng.integers(2, 9, n), newlen).astype(np.int64)
+            cs = (np.arange(n) * 1024).astype(np.int64)
+            got = run_dev(kvlen, newlen, cs)
+            want = top.run_pack(olib.oracle_pack_tables, kvlen, newlen, cs)
+            for k in want:
+                assert np.array_equal(got[k], want[k]), (n, k)
+    # churn schedule (the continuous-batching configuration), 100 steps, device state advanced on the device
+    sch = workloads.ChurnSchedule(seed=2)
+    for step in range(100):
+        kv, nl = sch.next_step()
+        got = run_dev(kv, nl, sch.cachestart)
+        want = top.run_pack(olib.oracle_pack_tables, kv, nl, sch.cachestart)
+        for k in want:
+            assert np.array_equal(got[k], want[k]), (step, k)
+        dkv, dnl = harness.to_dev(kv), harness.to_dev(nl)
+        harness.pkg.check(hiplib.pplhip_advance_slots(dkv.data_ptr(), dnl.data_ptr(), len(kv), None), "advance")
+        torch.cuda.synchronize()
+        assert np.array_equal(dkv.cpu().numpy(), kv + nl)
