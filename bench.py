@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the dynamic-batching attention path on one MI355X.
+
+Default workload = the Llama-3-8B mixed ragged batch of the baseline (120 decode sequences with kv length uniform
+in [256, 4096] + 8 causal prefill sequences with length uniform in [64, 1024]; H 32, KVH 8, Dh 128; int8 group-8
+KV cache). One "step" of the headline loop is one MultiHeadCacheAttention call through the C ABI on the decode
+part of that batch (quantize-on-write of the new tokens + split-k decode + merge); the prefill part and the fused
+mixed call are timed in the same run and reported as extra fields. Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3] [--no-cpu-baseline]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published (no sparsity)
+N_SLABS = 4  # distinct KV slabs rotated between steps so reads are served by HBM, not the 256 MB Infinity Cache
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--split-k", type=int, default=1)
+    return ap.parse_args()
+
+
+class DeviceBatch:
+    """Device-resident tensors + argument block of one MHCA call; history is quantised by the library itself."""
+
+    def __init__(self, pkg, lib, b, seed, n_slabs, split_k=1):
+        import torch
+        from ppl_nn_amd import cabi
+        self.pkg, self.lib, self.b, self.cabi = pkg, lib, b, cabi
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        S, Hs = b.total_new_tokens, b.total_hist_tokens
+        f16 = dict(dtype=torch.float16, device="cuda")
+        self.q = torch.randn((S, b.num_heads, b.head_dim), generator=g, **f16)
+        self.k = torch.randn((S, b.num_kv_heads, b.head_dim), generator=g, **f16)
+        self.v = torch.randn((S, b.num_kv_heads, b.head_dim), generator=g, **f16)
+        self.out = torch.zeros((S, b.num_heads, b.head_dim), **f16)
+        i64 = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).cuda()
+        self.seqstarts, self.kvstarts = i64(b.seqstarts), i64(b.kvstarts)
+        self.cachestarts, self.start_pos = i64(b.cachestarts), i64(b.start_pos)
+        histstarts, zeros = i64(b.histstarts), i64(np.zeros(max(b.batch, 1)))
+        shape = (b.max_tokens, b.num_layer, 2, b.num_kv_heads, b.head_dim)
+        self.slabs = []
+        self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        ptr = lambda t: C.c_void_p(t.data_ptr())
+        st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
+        for s in range(n_slabs):
+            cache = torch.zeros(shape, dtype=torch.int8, device="cuda")
+            scale = torch.zeros(shape[:-1] + (b.head_dim // 8,), **f16)
+            if Hs:
+                hk = torch.randn((Hs, b.num_kv_heads, b.head_dim), generator=g, **f16)
+                hv = torch.randn((Hs, b.num_kv_heads, b.head_dim), generator=g, **f16)
+                w = cabi.KvWriteArgs()
+                w.d_current_key, w.d_current_value = ptr(hk), ptr(hv)
+                w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(histstarts), ptr(self.cachestarts), ptr(zeros)
+                w.batch, w.total_new_tokens = b.batch, Hs
+                w.layer_idx, w.num_layer, w.num_kv_heads, w.head_dim = b.layer_idx, b.num_layer, b.num_kv_heads, b.head_dim
+                for kk, vv in st.items():
+                    setattr(w, kk, vv)
+                w.d_cache, w.d_scale = ptr(cache), ptr(scale)
+                pkg.check(lib.pplhip_kv_quantize_write(C.byref(w), self.stream), "history write")
+                torch.cuda.synchronize()
+                del hk, hv
+            self.slabs.append((cache, scale))
+        self.args = []
+        for cache, scale in self.slabs:
+            a = cabi.MhcaArgs()
+            a.d_query, a.d_current_key, a.d_current_value = ptr(self.q), ptr(self.k), ptr(self.v)
+            a.d_seqstarts, a.d_kvstarts = ptr(self.seqstarts), ptr(self.kvstarts)
+            a.d_cachestarts, a.d_start_pos = ptr(self.cachestarts), ptr(self.start_pos)
+            a.is_causal, a.batch, a.decoding_batches = 1, b.batch, b.decoding_batches
+            a.max_seqlen, a.max_kvlen = b.max_seqlen, b.max_kvlen
+            a.layer_idx, a.num_layer = b.layer_idx, b.num_layer
+            a.num_heads, a.num_kv_heads, a.head_dim = b.num_heads, b.num_kv_heads, b.head_dim
+            a.cache_mode, a.page_size = 0, 128
+            for kk, vv in st.items():
+                setattr(a, kk, vv)
+            a.enable_decoding_sharemem_mhca = a.enable_decoding_infinity_mhca = a.enable_decoding_infinity_gqca = 1
+            a.specify_decoding_attn_split_k = split_k
+            a.d_cache, a.d_scale, a.d_output = ptr(cache), ptr(scale), ptr(self.out)
+            a.total_new_tokens = S
+            self.args.append(a)
+        self.plan = cabi.MhcaPlan()
+        pkg.check(lib.pplhip_mhca_prepare(C.byref(self.args[0]), C.byref(self.plan)), "prepare")
+        self.ws = torch.empty(max(int(self.plan.workspace_bytes), 256), dtype=torch.uint8, device="cuda")
+        self.ws_ptr = ptr(self.ws)
+
+    def step(self, i):
+        a = self.args[i % len(self.args)]
+        rc = self.lib.pplhip_mhca_forward(C.byref(a), C.byref(self.plan), self.ws_ptr, self.stream)
+        if rc:
+            self.pkg.check(rc, "mhca_forward")
+
+
+def timed(db, steps, warmup):
+    """W untimed steps, then exactly K steps bracketed by synchronize; returns (wall ms/step, event ms/step)."""
+    import torch
+    for i in range(warmup):
+        db.step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        db.step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline(db, min_seconds=10.0, max_prepare=24):
+    """The decode part run through the x86-engine-semantics attention (fp32 MatMul/Mul/Softmax/MatMul, OpenMP over
+    heads) on the host cores, on dequantised K/V copied from the slab. A bounded sample: the first `max_prepare`
+    decode sequences, repeated until about `min_seconds` of CPU work has been timed."""
+    import oracle
+    L = oracle.lib()
+    b = db.b
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    cache, scale = db.slabs[0]
+    n = min(b.decoding_batches, max_prepare)
+    cases = []
+    for i in range(n):
+        kv = int(b.kvlens[i])
+        rows = slice(int(b.cachestarts[i]), int(b.cachestarts[i]) + kv)
+        deq = cache[rows, b.layer_idx].float() * scale[rows, b.layer_idx].float().repeat_interleave(8, dim=-1)
+        k = deq[:, 0].permute(1, 0, 2).contiguous().cpu().numpy()  # [KVH, kv, Dh]
+        v = deq[:, 1].permute(1, 0, 2).contiguous().cpu().numpy()
+        s0 = int(b.seqstarts[i])
+        q = db.q[s0:s0 + 1].float().permute(1, 0, 2).contiguous().cpu().numpy()  # [H, 1, Dh]
+        cases.append((q, k, v, np.empty_like(q), kv))
+    done_tokens, spent, passes = 0, 0.0, 0
+    while spent < min_seconds:
+        t0 = time.perf_counter()
+        for q, k, v, out, kv in cases:
+            rc = L.oracle_x86_attention(q.ctypes.data, k.ctypes.data, v.ctypes.data, None, out.ctypes.data,
+                                        b.num_heads, b.num_kv_heads, 1, kv, b.head_dim, cores)
+            assert rc == 0
+        dt = time.perf_counter() - t0
+        if passes > 0:  # the first pass warms caches and the OpenMP pool
+            spent += dt
+            done_tokens += len(cases)
+        passes += 1
+    return dict(value=done_tokens / spent, unit="tokens/s", cores=cores, kind="port",
+                sample=f"first {n} of {b.decoding_batches} decode sequences of the workload x {passes - 1} passes, "
+                       f"fp32 x86-engine-semantics attention (MatMul-Mul-Softmax-MatMul, OpenMP over heads) on "
+                       f"dequantised K/V resident in host memory, {spent:.1f} s of CPU work")
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the attention path has no collective; see DESIGN.md for how it "
+              "would shard by kv head). Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    pkg = entry.load_package()
+    lib = pkg.load_library()
+    from ppl_nn_amd import workloads
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+
+    if args.workload == "cfg2":
+        full = workloads.cfg2_llama3_8b_mixed()
+        dec_b, pre_b = workloads.cfg2_decode_part(), workloads.cfg2_prefill_part()
+        wname = "cfg2 Llama-3-8B mixed ragged batch (H32/KVH8/Dh128, int8 group-8 KV): decode part 120 seqs kv~U[256,4096]"
+    elif args.workload == "cfg1":
+        full, pre_b = None, None
+        dec_b = workloads.cfg1_llama2_7b_decode()
+        wname = "cfg1 Llama-2-7B pure decode (H32/KVH32/Dh128): 64 seqs kv~U[128,2048]"
+    else:
+        full, pre_b = None, None
+        dec_b = workloads.cfg3_long_context()
+        wname = "cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]"
+
+    dec = DeviceBatch(pkg, lib, dec_b, seed=1, n_slabs=N_SLABS, split_k=args.split_k)
+    wall_ms, ev_ms = timed(dec, args.steps, args.warmup)
+    nd = dec_b.decoding_batches
+    dec_bytes = dec_b.decode_bytes()
+    gbs = dec_bytes / (ev_ms * 1e-3) / 1e9
+    result = {
+        "metric": "decode attn tokens/s + % of HBM roofline; prefill attn TFLOPS, Llama-3-8B shape",
+        "value": nd / (wall_ms * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 KV + fp16 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": wname, "decode_seqs": nd, "kv_tokens": int(dec_b.kvlens.sum()),
+                   "chunk_tokens": int(dec.plan.decode_chunk_tokens), "num_chunks": int(dec.plan.decode_num_chunks),
+                   "slabs_rotated": N_SLABS},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "decode_int8kv_kernel (+ kv_quantize_write + decode_merge in the same call)",
+                     "algorithmic_bytes_per_launch": dec_bytes, "event_ms_per_launch": ev_ms},
+    }
+    if pre_b is not None:
+        pre = DeviceBatch(pkg, lib, pre_b, seed=2, n_slabs=1)
+        _, pre_ms = timed(pre, max(args.steps // 2, 10), max(args.warmup // 2, 3))
+        fl = pre_b.prefill_flops()
+        result["prefill"] = {"tflops": fl / (pre_ms * 1e-3) / 1e12, "ms": pre_ms, "flops": fl,
+                             "frac_of_fp16_mfma_peak": fl / (pre_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
+                             "peak_tflops": MFMA_FP16_PEAK_TFLOPS, "prefill_seqs": pre_b.batch,
+                             "prefill_tokens": pre_b.total_new_tokens}
+        del pre
+        mixed = DeviceBatch(pkg, lib, full, seed=3, n_slabs=N_SLABS)
+        _, mix_ms = timed(mixed, max(args.steps // 2, 10), max(args.warmup // 2, 3))
+        result["fused_mixed_call_ms"] = mix_ms
+        del mixed
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(dec)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

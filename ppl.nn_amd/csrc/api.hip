@@ -1,6 +1,7 @@
 // C ABI entry points: argument validation (same outcomes as the reference wrapper's checks), the split-k
 // heuristic, and the launch sequence write -> decode(+merge) -> prefill on the caller's stream.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "common.h"
@@ -129,25 +130,34 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     if (a->specify_decoding_attn_tpb != 0 && a->specify_decoding_attn_tpb != 256 && a->specify_decoding_attn_tpb != 512)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_tpb must be 0, 256 or 512");
 
-    // ---- decode: split the cached tokens into chunks so that the chip sees a few tasks per wave slot
+    // ---- decode: split the cached tokens into chunks, one workgroup (4 waves) per (sequence, kv head, chunk)
     plan->decode_waves_per_block = 4;
     const int64_t nd = a->decoding_batches;
     if (nd > 0 && a->max_kvlen > 0) {
-        const int64_t round = 64; // the kernel's inner block
+        const int64_t round = 128; // 4 waves x 32-token pipeline stages
         int64_t chunk;
         const int64_t whole = (a->max_kvlen + round - 1) / round * round;
         if (a->specify_decoding_attn_split_k == 0) {
             chunk = whole;
         } else {
-            const int64_t slots = (int64_t)device_cu_count() * 8; // 2 waves per SIMD
-            const int64_t pairs = nd * a->num_kv_heads;
-            // aim at ~3 tasks per slot if every sequence were max_kvlen long (ragged batches average about half)
-            chunk = (a->max_kvlen * pairs + 3 * slots - 1) / (3 * slots);
+            // Workgroup slots on the chip (2 resident workgroups per CU); a workgroup serves up to 4 kv heads of one
+            // (sequence, chunk). Aim at ~6 tasks per slot for a ragged batch whose sequences average half of
+            // max_kvlen, so that the tail of the launch is a small fraction of it.
+            const int64_t slots = (int64_t)device_cu_count() * 2;
+            int hpb = 1;
+            while (hpb < 4 && a->num_kv_heads % (hpb * 2) == 0) hpb *= 2;
+            const int64_t pairs = nd * (a->num_kv_heads / hpb);
+            chunk = (a->max_kvlen * pairs / 2 + 6 * slots - 1) / (6 * slots);
             chunk = (chunk + round - 1) / round * round;
-            if (chunk < 256) chunk = 256;
+            if (chunk < 256) chunk = 256; // below this the per-task partial (Dh+2 floats per head) stops being noise
             if (chunk > whole) chunk = whole;
             if (a->specify_decoding_attn_split_k == 2 && chunk >= whole && whole > round)
                 chunk = (whole / 2 + round - 1) / round * round;
+            if (const char* env = getenv("PPLHIP_DECODE_CHUNK")) { // tuning aid: force the split granularity
+                const int64_t forced = atoll(env);
+                if (forced > 0) chunk = (forced + round - 1) / round * round;
+                if (chunk > whole) chunk = whole;
+            }
         }
         plan->decode_chunk_tokens = (int32_t)chunk;
         plan->decode_num_chunks = (int32_t)((a->max_kvlen + chunk - 1) / chunk);

@@ -1,24 +1,35 @@
 // Decode attention over the int8 group-8 KV slab (one new token per sequence), split along the cached tokens.
 //
 // Roofline: HBM. Each cached token costs 2 * KVH * (Dh + Dh/4) bytes and is read exactly once; arithmetic
-// intensity is 1.6 .. 12.8 flop/B, so the kernel is organised around streaming bytes, and the contraction is put
-// on the matrix cores only so that dequantisation + FMA work does not become the limiter for grouped-query shapes.
+// intensity is 1.6 .. 12.8 flop/B. Three things have to stay below the HBM time for the kernel to sit on that
+// roofline: vector-ALU work (dequantisation), matrix-core work, and the number of vector-memory instructions the
+// texture addresser has to walk through. The design answers each:
+//   * Bytes travel global -> LDS with global_load_lds_dwordx4 (no registers, 16 B per lane, every instruction covers
+//     whole 128 B rows of the slab), ten instructions per 32 tokens instead of two dozen narrow gathers.
+//   * Each wave stages its own tokens in its own LDS region, double buffered: the DMA of the next 32 tokens is in
+//     flight while the current 32 are computed. Only wave-level waits are needed, no workgroup barriers.
+//   * All H/KVH query heads of a kv head ride in the 16-wide N dimension of v_mfma_f32_16x16x32_f16, so a KV byte is
+//     read once whatever the grouping, and the contraction costs two dozen MFMAs per 32 tokens.
 //
-// Work decomposition: one *wavefront task* = (sequence b, kv head, chunk of `chunk` cached tokens). All H/KVH query
-// heads that share the kv head ride in the 16-wide N dimension of v_mfma_f32_16x16x16_f16, so every KV byte is
-// loaded once per task. Waves are independent (no LDS, no barriers); a workgroup is just 4 adjacent tasks, ordered
-// so that its waves read adjacent kv heads of the same tokens (contiguous bytes in the (MaxT, L, 2, KVH, Dh) slab).
+// Work decomposition: one workgroup = one task (sequence b, kv head, chunk of `chunk` cached tokens); its 4 waves take
+// a quarter of the chunk each and combine their softmax states through LDS at the end. Tasks are ordered
+// kv-head-fastest so that neighbouring workgroups read neighbouring bytes of the (MaxT, L, 2, KVH, Dh) slab.
+//
+// LDS layout of one 32-token stage of one wave (10 KiB): K rows [32][128 B], V rows [32][128 B], K scales [32][32 B],
+// V scales [32][32 B]. Inside a K/V row the eight 16 B pieces are XOR-swizzled with (row & 7) by choosing which
+// global piece each DMA lane fetches, so the MFMA-layout reads below (16 different rows per instruction) spread over
+// all banks.
 //
 // Per 16-token block a lane (m = lane & 15, kq = lane >> 4) does:
-//   S^T = K_hat * Q^T   A = K_hat[token m][channels 64*jj + 16*kq + 4*i .. +3]   (two 16 B loads per lane per block)
+//   S^T = K_hat * Q^T   A = K_hat[token m][channels 32*kq + 16*j + 8*i .. +7]  (two ds_read_b128, one scale b64 per lane)
 //                       B = Q^T, held in registers for the whole task
 //         -> lane holds scores of head m for tokens 4*kq .. 4*kq+3
-//   O^T += V_hat^T * P^T  A = V_hat^T[channel 8*m + i][tokens 4*kq .. +3]         (four 8 B loads per lane per block,
-//                       transposed in registers with v_perm), B = P^T straight from the score registers
+//   O^T += V_hat^T * P^T  A = V_hat^T[channel 8*m + i][tokens 4*kq .. +3]  (four ds_read_b64 per lane, transposed in
+//                       registers with v_perm), B = P^T straight from the score registers
 // int8 -> fp16 is exact: (x ^ 0x80) placed under exponent byte 0x64 reads as 1024 + (x + 128); subtract 1152, then
 // multiply by the group's fp16 scale (packed fp16 ops). Softmax runs online in the exp2 domain with fp32 statistics.
 //
-// Each task writes an un-normalised partial (max, sum, acc[Dh]) per query head into the workspace and
+// Each task writes one un-normalised partial (max, sum, acc[Dh]) per query head into the workspace and
 // `decode_merge_kernel` combines the chunks of a sequence with the usual log-sum-exp weights. With a single chunk the
 // task normalises and writes fp16 output itself.
 #include "common.h"
@@ -27,7 +38,16 @@ namespace pplhip {
 
 constexpr int kDh = 128; // head_dim this kernel is specialised for
 constexpr int kDecodeWaves = 4;
-constexpr int kIterTokens = 64; // tokens per softmax update (4 MFMA sub-blocks of 16)
+constexpr int kStageTokens = 32; // tokens per pipeline stage (2 MFMA sub-blocks of 16)
+constexpr int kSubBlocks = kStageTokens / 16;
+// LDS bytes of one stage of one wave, and where its four arrays start
+constexpr int kLdsK = 0;
+constexpr int kLdsV = kStageTokens * 128;
+constexpr int kLdsKs = 2 * kStageTokens * 128;
+constexpr int kLdsVs = kLdsKs + kStageTokens * 32;
+constexpr int kStageBytes = kLdsVs + kStageTokens * 32; // 10240
+constexpr int kWaveLdsBytes = 2 * kStageBytes;
+constexpr int kDecodeLdsBytes = kDecodeWaves * kWaveLdsBytes; // 81920: two workgroups fill a CU's 160 KiB
 
 struct DecodeParams {
     const half_t* q; // [S, H, Dh]
@@ -42,10 +62,15 @@ struct DecodeParams {
     CacheAddr addr;
     int32_t nd; // decode sequences
     int32_t num_heads, kv_heads, rep; // rep = num_heads / kv_heads (<= 16)
-    int32_t chunk, num_chunks;
+    int32_t chunk, num_chunks; // chunk is a multiple of kDecodeWaves * kStageTokens
+    int32_t num_chunks_pad8; // num_chunks rounded up to a multiple of 8 (task grid only)
+    int32_t hpb; // kv heads per workgroup: min(kv_heads, 4), a power of two dividing kv_heads
     int64_t total_tasks;
     float score_scale; // log2(e) / sqrt(Dh)
 };
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 __device__ inline half2_t as_half2(uint32_t u) {
     half2_t h;
@@ -70,6 +95,14 @@ __device__ inline half2_t dequant2(uint32_t widened, half2_t s2) {
     const half2_t bias = {(half_t)1152.0f, (half_t)1152.0f};
     return (as_half2(widened) - bias) * s2;
 }
+// 8 int8 channels (one quantisation group) -> 8 fp16 values times the group scale
+__device__ inline half8_t dequant8(uint32_t w0, uint32_t w1, half_t scale) {
+    const half2_t s2 = {scale, scale};
+    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+    const half2_t a = dequant2(widen_lo(x0), s2), b = dequant2(widen_hi(x0), s2);
+    const half2_t c = dequant2(widen_lo(x1), s2), d = dequant2(widen_hi(x1), s2);
+    return half8_t{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
+}
 
 __device__ inline float wave_max_over_quads(float v) {
     v = fmaxf(v, __shfl_xor(v, 16));
@@ -82,217 +115,448 @@ __device__ inline float wave_sum_over_quads(float v) {
     return v;
 }
 
-__global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
-    const int lane = threadIdx.x & 63;
-    const int64_t task = (int64_t)blockIdx.x * kDecodeWaves + (threadIdx.x >> 6);
-    if (task >= p.total_tasks) return;
-    const int kvh = (int)(task % p.kv_heads);
-    const int64_t bc = task / p.kv_heads;
-    const int c = (int)(bc % p.num_chunks);
-    const int b = (int)(bc / p.num_chunks);
-    const int64_t kvlen = p.kvstarts[b + 1] - p.kvstarts[b];
-    const int64_t t_begin = (int64_t)c * p.chunk;
-    if (t_begin >= kvlen) return; // this sequence has fewer chunks; the merge pass never looks here
-    const int64_t t_end = (t_begin + p.chunk < kvlen) ? t_begin + p.chunk : kvlen;
-    const int64_t tok0 = p.cachestarts[b];
-    const int64_t qrow = p.seqstarts[b];
+// Pins a pointer that is wave-uniform by construction into scalar registers, so that memory instructions take the
+// "scalar base + 32-bit lane offset" addressing form.
+__device__ inline const char* make_uniform(const char* p) {
+    const uint64_t u = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+}
 
-    const int m = lane & 15;
-    const int kq = lane >> 4;
+// LDS reads of DMA-filled buffers go through inline assembly: for compiler-visible LDS loads the waitcnt pass cannot
+// tell which DMA transfer they depend on and drains ALL outstanding transfers first (vmcnt(0)), which would serialise
+// the pipeline. Here the ordering is explicit: PPLHIP_WAIT_VMCNT before the first read of a stage, and
+// PPLHIP_WAIT_LGKMCNT + a scheduling barrier before the first use of the values read.
+template <int OFF>
+__device__ inline uint4 lds_read_b128(uint32_t addr) {
+    uint4 r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+    return r;
+}
+template <int OFF>
+__device__ inline uint2 lds_read_b64(uint32_t addr) {
+    uint2 r;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+    return r;
+}
+template <int OFF>
+__device__ inline uint32_t lds_read_u16(uint32_t addr) {
+    uint32_t r;
+    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+    return r;
+}
+#define PPLHIP_WAIT_LGKMCNT(n)                                  \
+    do {                                                        \
+        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory"); \
+        __builtin_amdgcn_sched_barrier(0);                      \
+    } while (0)
 
-    // ---- Q^T as the B operand, kept for the whole task: qB[jj][i] = Q[head m][64*jj + 16*kq + 4*i .. +3]
-    half4_t qB[2][4];
-    {
-        const bool live = m < p.rep;
-        const half_t* qp = p.q + ((qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
+// s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at "no wait"), gfx9 encoding
+#define PPLHIP_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | 0x0f70)
+constexpr int kDmaPerStage = 2 * (kStageTokens / 8) + 2; // 4 K + 4 V + K scales + V scales
+
+// Per-lane source offsets of the stage DMA (relative to the wave-uniform stage base).
+struct DmaOffsets {
+    uint32_t kv[kStageTokens / 8]; // rows 8*i + lane/8: row * stride + swizzled piece * 16
+    uint32_t sc; // row lane/2: row * scale stride + (lane & 1) * 16
+};
+
+// rows_mem: rows of the stage that exist in the chunk (1..32); later rows are clamped onto the last one
+__device__ inline void make_dma_offsets(DmaOffsets& o, int lane, uint32_t stride, uint32_t sstride_b, int rows_mem) {
+#ifdef PPLHIP_X_NOSWZ
+    const int piece = (lane & 7);
+#else
+    const int piece = (lane & 7) ^ (lane >> 3); // LDS slot (lane & 7) of row r holds global piece slot ^ (r & 7)
+#endif
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-            uint4 lo = *reinterpret_cast<const uint4*>(qp + 64 * jj + 16 * kq);
-            uint4 hi = *reinterpret_cast<const uint4*>(qp + 64 * jj + 16 * kq + 8);
-            if (!live) lo = hi = make_uint4(0, 0, 0, 0);
-            half4_t tmp[4];
-            __builtin_memcpy(&tmp[0], &lo, 16);
-            __builtin_memcpy(&tmp[2], &hi, 16);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) qB[jj][i] = tmp[i];
-        }
+    for (int i = 0; i < kStageTokens / 8; ++i) {
+        int r = 8 * i + (lane >> 3);
+        r = r < rows_mem ? r : rows_mem - 1;
+        // the swizzle key is the LDS row (8*i + lane/8) & 7 = lane >> 3, whatever row the bytes come from
+        o.kv[i] = (uint32_t)r * stride + 16u * piece;
     }
+    int rs = lane >> 1;
+    rs = rs < rows_mem ? rs : rows_mem - 1;
+    o.sc = (uint32_t)rs * sstride_b + 16u * (lane & 1);
+}
 
-    const int8_t* kbase = p.cache + p.addr.row(tok0, 0, kvh);
-    const int8_t* vbase = p.cache + p.addr.row(tok0, 1, kvh);
-    const half_t* ksbase = p.scale + p.addr.row(tok0, 0, kvh) / kQuantGroup;
-    const half_t* vsbase = p.scale + p.addr.row(tok0, 1, kvh) / kQuantGroup;
-    const int64_t stride = p.addr.stride_s;
-    const int64_t sstride = p.addr.stride_s / kQuantGroup;
-
-    float4_t oacc[8];
+// Enqueues the 10 global->LDS transfers of one stage. cbase/sbase: K row 0 of the stage in the cache / scale tensors;
+// kv_off / kv_off_s: distance from a K row to the V row of the same token.
+__device__ inline void dma_stage(char* lds_stage, const char* cbase, const char* sbase, const DmaOffsets& o,
+                                 uint32_t kv_off, uint32_t kv_off_s) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY; // running max of head m (same value in the 4 lanes that share m)
-    float l_part = 0.f; // this lane's share of the running sum
-
-    const int64_t last_tok = t_end - 1;
-    for (int64_t t0 = t_begin; t0 < t_end; t0 += kIterTokens) {
-        // ---- issue all loads of this iteration (rows past the chunk end are clamped to its last row and masked)
-        uint4 kraw[4][2];
-        uint32_t ksc[4][2];
-        uint2 vraw[4][4];
-        half_t vsc[4][4];
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {
-            int64_t tk = t0 + 16 * sb + m;
-            tk = tk < last_tok ? tk : last_tok;
-            const int8_t* kr = kbase + tk * stride;
-            const half_t* ks = ksbase + tk * sstride;
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                kraw[sb][jj] = *reinterpret_cast<const uint4*>(kr + 64 * jj + 16 * kq);
-                ksc[sb][jj] = *reinterpret_cast<const uint32_t*>(ks + 8 * jj + 2 * kq);
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                int64_t tv = t0 + 16 * sb + 4 * kq + e;
-                tv = tv < last_tok ? tv : last_tok;
-                vraw[sb][e] = *reinterpret_cast<const uint2*>(vbase + tv * stride + 8 * m);
-                vsc[sb][e] = vsbase[tv * sstride + m];
-            }
-        }
-
-        // ---- scores: S^T[token, head] for 4 sub-blocks of 16 tokens
-        float4_t st[4];
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {
-            float4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                const uint32_t w[4] = {kraw[sb][jj].x, kraw[sb][jj].y, kraw[sb][jj].z, kraw[sb][jj].w};
-                const half2_t sc = as_half2(ksc[sb][jj]);
-                const half2_t s_lo = {sc.x, sc.x};
-                const half2_t s_hi = {sc.y, sc.y};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t x = w[i] ^ 0x80808080u;
-                    const half2_t s2 = (i < 2) ? s_lo : s_hi;
-                    const half2_t a01 = dequant2(widen_lo(x), s2);
-                    const half2_t a23 = dequant2(widen_hi(x), s2);
-                    const half4_t a = {a01.x, a01.y, a23.x, a23.y};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x16f16(a, qB[jj][i], acc, 0, 0, 0);
-                }
-            }
-            // lane now holds head m, tokens t0 + 16*sb + 4*kq + e
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int64_t tk = t0 + 16 * sb + 4 * kq + e;
-                acc[e] = (tk < t_end) ? acc[e] * p.score_scale : -INFINITY;
-            }
-            st[sb] = acc;
-        }
-
-        // ---- online softmax update (per head = per lane column m)
-        float mx = -INFINITY;
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) mx = fmaxf(mx, st[sb][e]);
-        mx = wave_max_over_quads(mx);
-        const float m_new = fmaxf(m_run, mx); // finite: the first token of every iteration is inside the chunk
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.f;
-        half4_t pB[4];
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {
-            float pe[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                pe[e] = __builtin_amdgcn_exp2f(st[sb][e] - m_new);
-                psum += pe[e];
-            }
-            pB[sb] = half4_t{(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
-        }
-        l_part = l_part * alpha + psum;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
-
-        // ---- O^T[channel, head] += V_hat^T * P^T
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {
-            half2_t d[4][4]; // [token e][channel pair c] dequantised, channels 8*m + 2c, 2c+1
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const half2_t s2 = {vsc[sb][e], vsc[sb][e]};
-                const uint32_t x0 = vraw[sb][e].x ^ 0x80808080u;
-                const uint32_t x1 = vraw[sb][e].y ^ 0x80808080u;
-                d[e][0] = dequant2(widen_lo(x0), s2);
-                d[e][1] = dequant2(widen_hi(x0), s2);
-                d[e][2] = dequant2(widen_lo(x1), s2);
-                d[e][3] = dequant2(widen_hi(x1), s2);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int cpair = i >> 1;
-                const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-                const uint32_t t01 = __builtin_amdgcn_perm(as_u32(d[1][cpair]), as_u32(d[0][cpair]), sel);
-                const uint32_t t23 = __builtin_amdgcn_perm(as_u32(d[3][cpair]), as_u32(d[2][cpair]), sel);
-                const half2_t h01 = as_half2(t01), h23 = as_half2(t23);
-                const half4_t a = {h01.x, h01.y, h23.x, h23.y};
-                oacc[i] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pB[sb], oacc[i], 0, 0, 0);
-            }
-        }
+    for (int i = 0; i < kStageTokens / 8; ++i) {
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + o.kv[i]), (lds_ptr_t)(lds_stage + kLdsK + 1024 * i), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + kv_off + o.kv[i]), (lds_ptr_t)(lds_stage + kLdsV + 1024 * i),
+                                         16, 0, 0);
     }
+#ifdef PPLHIP_X_NOSCALEDMA
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + o.kv[0]), (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + o.kv[1]), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
+#else
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + o.sc), (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + kv_off_s + o.sc), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
+#endif
+}
 
-    const float l_tot = wave_sum_over_quads(l_part);
-    if (m >= p.rep) return;
-    const int head = kvh * p.rep + m;
-    // lane (head m, r = kq) holds channels 8*(4*r + e) + i in oacc[i][e]
-    if (p.num_chunks == 1) {
-        const float inv = 1.0f / l_tot;
-        half_t* op = p.out + (qrow * p.num_heads + head) * kDh;
+// Per-lane LDS read offsets inside a stage (they are the same for every stage).
+struct ReadOffsets {
+    uint32_t k[2]; // K row m, pieces 2*kq and 2*kq + 1 (swizzled)      (+2048 per sub-block)
+    uint32_t ks; // K scale row m, groups 4*kq .. 4*kq + 3              (+512 per sub-block)
+    uint32_t v[4]; // V row 4*kq + e, 8 channels of group m (swizzled)   (+2048 per sub-block)
+    uint32_t vs; // V scale row 4*kq, group m                           (+32 per e, +512 per sub-block)
+};
+
+__device__ inline void make_read_offsets(ReadOffsets& r, int m, int kq) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) r.k[j] = kLdsK + m * 128 + (((2 * kq + j) ^ (m & 7)) * 16);
+    r.ks = kLdsKs + m * 32 + kq * 8;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int row = 4 * kq + e;
+        r.v[e] = kLdsV + row * 128 + (((m >> 1) ^ (row & 7)) * 16) + (m & 1) * 8;
+    }
+    r.vs = kLdsVs + (4 * kq) * 32 + m * 2;
+}
+
+struct SoftmaxState {
+    float4_t oacc[8]; // O^T: oacc[i][e] = channel 8*(4*kq + e) + i of head m
+    float m_run; // running max of head m in the exp2 domain (same in the 4 lanes that share m)
+    float l_part; // this lane's share of the running sum
+};
+
+template <int SB>
+__device__ inline void read_stage_sub(uint4 (&kr)[2], uint2& ksr, uint2 (&vr)[4], uint32_t (&vsr)[4], const uint32_t (&ak)[2],
+                                      uint32_t aks, const uint32_t (&av)[4], uint32_t avs) {
+    kr[0] = lds_read_b128<2048 * SB>(ak[0]);
+    kr[1] = lds_read_b128<2048 * SB>(ak[1]);
+    ksr = lds_read_b64<512 * SB>(aks);
+    vr[0] = lds_read_b64<2048 * SB>(av[0]);
+    vr[1] = lds_read_b64<2048 * SB>(av[1]);
+    vr[2] = lds_read_b64<2048 * SB>(av[2]);
+    vr[3] = lds_read_b64<2048 * SB>(av[3]);
+    vsr[0] = lds_read_u16<512 * SB + 0>(avs);
+    vsr[1] = lds_read_u16<512 * SB + 32>(avs);
+    vsr[2] = lds_read_u16<512 * SB + 64>(avs);
+    vsr[3] = lds_read_u16<512 * SB + 96>(avs);
+}
+
+// lds_stage: LDS byte address of the stage buffer. rows_valid: tokens of this stage that belong to the wave's range
+// (1..32); the rest is masked out of the softmax.
+__device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, SoftmaxState& ss,
+                                     const half8_t (&qB)[2][2], int kq, int rows_valid, float score_scale) {
+    static_assert(kSubBlocks == 2, "the stage is processed as two 16-token sub-blocks");
+    const uint32_t ak[2] = {ro.k[0] + lds_stage, ro.k[1] + lds_stage};
+    const uint32_t aks = ro.ks + lds_stage, avs = ro.vs + lds_stage;
+    const uint32_t av[4] = {ro.v[0] + lds_stage, ro.v[1] + lds_stage, ro.v[2] + lds_stage, ro.v[3] + lds_stage};
+    uint4 kr[kSubBlocks][2];
+    uint2 ksr[kSubBlocks];
+    uint2 vraw[kSubBlocks][4];
+    uint32_t vsr[kSubBlocks][4];
+    read_stage_sub<0>(kr[0], ksr[0], vraw[0], vsr[0], ak, aks, av, avs);
+    read_stage_sub<1>(kr[1], ksr[1], vraw[1], vsr[1], ak, aks, av, avs);
+    PPLHIP_WAIT_LGKMCNT(0);
+
+    // ---- scores S^T[token, head]: v_mfma_f32_16x16x32_f16, one quantisation group (8 channels) per lane per MFMA
+    float4_t sc[kSubBlocks];
+#pragma unroll
+    for (int sb = 0; sb < kSubBlocks; ++sb) {
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        const half2_t s01 = as_half2(ksr[sb].x), s23 = as_half2(ksr[sb].y);
+        const half_t gs[4] = {s01.x, s01.y, s23.x, s23.y};
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const half8_t a0 = dequant8(kr[sb][j].x, kr[sb][j].y, gs[2 * j]);
+            const half8_t a1 = dequant8(kr[sb][j].z, kr[sb][j].w, gs[2 * j + 1]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qB[j][0], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, qB[j][1], acc, 0, 0, 0);
+        }
+        // lane now holds head m, tokens 16*sb + 4*kq + e of the stage
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = (16 * sb + 4 * kq + e < rows_valid) ? acc[e] * score_scale : -INFINITY;
+        sc[sb] = acc;
+    }
+    // ---- online softmax update (per head = per lane column m)
+    float mx = -INFINITY;
+#pragma unroll
+    for (int sb = 0; sb < kSubBlocks; ++sb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mx = fmaxf(mx, sc[sb][e]);
+    mx = wave_max_over_quads(mx);
+    const float m_new = fmaxf(ss.m_run, mx); // finite: the first token of every computed stage is valid
+    const float alpha = __builtin_amdgcn_exp2f(ss.m_run - m_new);
+    ss.m_run = m_new;
+    float psum = 0.f;
+    float pe[kSubBlocks][4];
+#pragma unroll
+    for (int sb = 0; sb < kSubBlocks; ++sb)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            half_t o[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = (half_t)(oacc[i][e] * inv);
-            uint4 packed;
-            __builtin_memcpy(&packed, o, 16);
-            *reinterpret_cast<uint4*>(op + 8 * (4 * kq + e)) = packed;
+            pe[sb][e] = __builtin_amdgcn_exp2f(sc[sb][e] - m_new);
+            psum += pe[sb][e];
         }
-    } else {
-        const int64_t prow = ((int64_t)b * p.num_chunks + c) * p.num_heads + head;
-        float* pa = p.part_acc + prow * kDh;
+    // B operand of the PV product: k-slot e8 of this lane <-> token 16*(e8/4) + 4*kq + e8%4 of the stage
+    const half8_t pB = {(half_t)pe[0][0], (half_t)pe[0][1], (half_t)pe[0][2], (half_t)pe[0][3],
+                        (half_t)pe[1][0], (half_t)pe[1][1], (half_t)pe[1][2], (half_t)pe[1][3]};
+    ss.l_part = ss.l_part * alpha + psum;
+    if (__any(alpha != 1.0f)) { // once the running maxima have settled, the rescale is skipped (wave-uniform branch)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss.oacc[i] *= alpha;
+    }
+    // ---- O^T[channel, head] += V_hat^T * P^T over the stage's 32 tokens: one 16x16x32 MFMA per channel i
+    half2_t vs2[kSubBlocks][4];
+#pragma unroll
+    for (int sb = 0; sb < kSubBlocks; ++sb)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float4_t lo = {oacc[0][e], oacc[1][e], oacc[2][e], oacc[3][e]};
-            const float4_t hi = {oacc[4][e], oacc[5][e], oacc[6][e], oacc[7][e]};
-            *reinterpret_cast<float4_t*>(pa + 8 * (4 * kq + e)) = lo;
-            *reinterpret_cast<float4_t*>(pa + 8 * (4 * kq + e) + 4) = hi;
+            const uint32_t dup = vsr[sb][e] | (vsr[sb][e] << 16);
+            vs2[sb][e] = as_half2(dup);
         }
-        if (kq == 0) {
-            p.part_ml[prow * 2 + 0] = m_run;
-            p.part_ml[prow * 2 + 1] = l_tot;
+#pragma unroll
+    for (int cp = 0; cp < 4; ++cp) { // channel pair 8*m + 2*cp, 2*cp + 1 of this lane
+        half2_t d[kSubBlocks][4]; // dequantised [sb][token e]
+#pragma unroll
+        for (int sb = 0; sb < kSubBlocks; ++sb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t x = ((cp < 2) ? vraw[sb][e].x : vraw[sb][e].y) ^ 0x80808080u;
+                d[sb][e] = dequant2((cp & 1) ? widen_hi(x) : widen_lo(x), vs2[sb][e]);
+            }
+#pragma unroll
+        for (int odd = 0; odd < 2; ++odd) {
+            const uint32_t sel = odd ? 0x07060302u : 0x05040100u;
+            uint32_t t[4];
+#pragma unroll
+            for (int sb = 0; sb < kSubBlocks; ++sb) {
+                t[2 * sb + 0] = __builtin_amdgcn_perm(as_u32(d[sb][1]), as_u32(d[sb][0]), sel);
+                t[2 * sb + 1] = __builtin_amdgcn_perm(as_u32(d[sb][3]), as_u32(d[sb][2]), sel);
+            }
+            half8_t a;
+            __builtin_memcpy(&a, t, 16);
+            const int i = 2 * cp + odd;
+            ss.oacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pB, ss.oacc[i], 0, 0, 0);
         }
     }
 }
 
-// One workgroup of 128 lanes per (decode sequence, query head): out[d] = sum_c w_c acc_c[d] / sum_c w_c l_c,
-// w_c = exp2(m_c - max_c m_c), over the chunks the sequence really has.
-__global__ __launch_bounds__(kDh) void decode_merge_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
+    // Task = (sequence b, chunk c, group of hpb kv heads). The waves of the workgroup are (kv head within the group)
+    // x (token split): with 4 or more kv heads every wave owns one head and the whole chunk, so the workgroup as a
+    // whole reads hpb * 128 contiguous bytes of every token; with fewer heads the waves split the chunk's tokens.
+    //
+    // XCD-aware task order: workgroups are dealt round-robin to the 8 XCDs (workgroup i runs on XCD i % 8), each with
+    // its own L2. The head groups of one (sequence, chunk) read neighbouring rows of the same slab tokens, so they are
+    // given to workgroups i, i + 8, i + 16, ... that start on the same XCD at about the same time: their requests then
+    // meet in one L2 and reach the same DRAM pages together.
+    // Ragged batches: chunk c of sequence b goes to XCD (b + c) % 8, so a sequence's chunks walk round the XCDs starting
+    // at a different one per sequence and every XCD gets its share of the short and of the long sequences. The chunk
+    // count is padded to a multiple of 8 for that; padded tasks exit at once.
+    const int groups = p.kv_heads / p.hpb;
+    const int xcd = blockIdx.x & 7;
+    const int64_t j = blockIdx.x >> 3;
+    const int hg = (int)(j % groups);
+    const int64_t g = j / groups;
+    const int c8 = p.num_chunks_pad8 >> 3;
+    const int b = (int)(g / c8);
+    const int c = (int)(g % c8) * 8 + ((xcd - b) & 7);
+    if (c >= p.num_chunks) return;
+    const int kvh_local = wave & (p.hpb - 1);
+    const int kvh = hg * p.hpb + kvh_local;
+    const int tsplits = kDecodeWaves / p.hpb;
+    const int ts = wave / p.hpb;
+    const int64_t kv_lo = p.kvstarts[b], kv_hi = p.kvstarts[b + 1];
+    const int64_t tok0 = p.cachestarts[b];
+    const int64_t qrow = p.seqstarts[b];
+    const int64_t kvlen = kv_hi - kv_lo;
+    const int64_t c_begin = (int64_t)c * p.chunk;
+    if (c_begin >= kvlen) return; // block-uniform: this sequence has fewer chunks; the merge pass never looks here
+    const int64_t c_end = (c_begin + p.chunk < kvlen) ? c_begin + p.chunk : kvlen;
+    const int sub = p.chunk / tsplits;
+    const int64_t t_begin = c_begin + (int64_t)ts * sub;
+    const int64_t t_end = (t_begin + sub < c_end) ? t_begin + sub : c_end; // may be <= t_begin: wave has no tokens
+
+    const int m = lane & 15;
+    const int kq = lane >> 4;
+
+    // ---- Q^T as the B operand, kept for the whole task: qB[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
+    half8_t qB[2][2];
+    {
+        const bool live = m < p.rep;
+        const half_t* qp = p.q + ((qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                uint4 x = *reinterpret_cast<const uint4*>(qp + 32 * kq + 16 * j + 8 * i);
+                if (!live) x = make_uint4(0, 0, 0, 0);
+                __builtin_memcpy(&qB[j][i], &x, 16);
+            }
+    }
+
+    SoftmaxState ss;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss.oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    ss.m_run = -INFINITY;
+    ss.l_part = 0.f;
+
+    char* wave_lds = smem + wave * kWaveLdsBytes;
+    const uint32_t wave_lds_addr =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem + wave * kWaveLdsBytes;
+    if (t_begin < t_end) {
+        const uint32_t stride = (uint32_t)p.addr.stride_s; // bytes between tokens (int8 elements)
+        const uint32_t sstride_b = (uint32_t)(p.addr.stride_s / kQuantGroup) * 2u;
+        const uint32_t kv_off = (uint32_t)p.addr.stride_kv;
+        const uint32_t kv_off_s = (uint32_t)(p.addr.stride_kv / kQuantGroup) * 2u;
+        const int64_t row0 = p.addr.row(tok0 + t_begin, 0, kvh);
+        const char* cbase = reinterpret_cast<const char*>(p.cache) + row0;
+        const char* sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
+        const int64_t step_c = (int64_t)kStageTokens * stride, step_s = (int64_t)kStageTokens * sstride_b;
+        DmaOffsets full;
+        make_dma_offsets(full, lane, stride, sstride_b, kStageTokens);
+        ReadOffsets ro;
+        make_read_offsets(ro, m, kq);
+        // The wave's last stage may overhang: rows past the end of the CHUNK are clamped onto its last row (loads must
+        // stay inside memory the sequence owns) and everything past the wave's own range is masked in the softmax.
+        const int n_stages = (int)((t_end - t_begin + kStageTokens - 1) / kStageTokens);
+        const int64_t last_stage_t0 = t_begin + (int64_t)(n_stages - 1) * kStageTokens;
+        const int tail_rows_mem = (int)((c_end - last_stage_t0) < kStageTokens ? (c_end - last_stage_t0) : kStageTokens);
+        const int tail_rows_valid = (int)(t_end - last_stage_t0);
+        auto issue = [&](int idx) {
+            char* dst = wave_lds + (idx & 1) * kStageBytes;
+            const char* cb = make_uniform(cbase + idx * step_c);
+            const char* sb = make_uniform(sbase + idx * step_s);
+#ifdef PPLHIP_X_NODMA
+            if (idx > 0) return;
+#endif
+            if (idx == n_stages - 1 && tail_rows_mem < kStageTokens) { // wave-uniform, at most once per wave
+                DmaOffsets tail;
+                make_dma_offsets(tail, lane, stride, sstride_b, tail_rows_mem);
+                dma_stage(dst, cb, sb, tail, kv_off, kv_off_s);
+            } else {
+                dma_stage(dst, cb, sb, full, kv_off, kv_off_s);
+            }
+        };
+
+        issue(0);
+        // The query loads are older than stage 0's transfers: retire them here, with stage 0 already in flight, so that
+        // no full drain of the DMA queue is needed at their first use inside the loop.
+        PPLHIP_WAIT_VMCNT(kDmaPerStage);
+        for (int it = 0; it < n_stages; ++it) {
+            // the buffer stage it+1 lands in was last read by compute(it-1), which has finished in program order
+            if (it + 1 < n_stages) {
+                issue(it + 1);
+                PPLHIP_WAIT_VMCNT(kDmaPerStage); // everything but the transfers just enqueued has landed
+            } else {
+                PPLHIP_WAIT_VMCNT(0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#ifdef PPLHIP_X_NOCOMPUTE
+            if (it == 0)
+#endif
+            compute_stage(wave_lds_addr + (it & 1) * kStageBytes, ro, ss, qB, kq,
+                          it + 1 == n_stages ? tail_rows_valid : kStageTokens, p.score_scale);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    const float l_tot = wave_sum_over_quads(ss.l_part);
+
+    // ---- combine the token splits of each kv head: LDS layout [wave][head][Dh + 2] (acc, then max, sum), reusing the
+    // stage buffers
+    __syncthreads();
+    float* lds = reinterpret_cast<float*>(smem);
+    const int row_f = kDh + 2;
+    if (m < p.rep) {
+        float* dst = lds + ((size_t)wave * p.rep + m) * row_f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dst[8 * (4 * kq + e) + i] = ss.oacc[i][e];
+        if (kq == 0) {
+            dst[kDh] = ss.m_run;
+            dst[kDh + 1] = l_tot;
+        }
+    }
+    __syncthreads();
+    const int n_out = p.hpb * p.rep * kDh; // (kv head of the group, query head of the kv head, channel)
+    for (int idx = threadIdx.x; idx < n_out; idx += kDecodeWaves * kWave) {
+        const int d = idx & (kDh - 1);
+        const int hh = idx >> 7; // kv_local * rep + h
+        const int kl = hh / p.rep, h = hh - kl * p.rep;
+        float mx = -INFINITY;
+        for (int t = 0; t < tsplits; ++t) mx = fmaxf(mx, lds[((size_t)(t * p.hpb + kl) * p.rep + h) * row_f + kDh]);
+        float acc = 0.f, l = 0.f;
+        for (int t = 0; t < tsplits; ++t) {
+            const float* src = lds + ((size_t)(t * p.hpb + kl) * p.rep + h) * row_f;
+            const float wgt = __builtin_amdgcn_exp2f(src[kDh] - mx); // a wave without tokens has max -inf -> weight 0
+            acc += wgt * src[d];
+            l += wgt * src[kDh + 1];
+        }
+        const int head = (hg * p.hpb + kl) * p.rep + h;
+        if (p.num_chunks == 1) {
+            p.out[(qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
+        } else {
+            const int64_t prow = ((int64_t)b * p.num_chunks + c) * p.num_heads + head;
+            p.part_acc[prow * kDh + d] = acc;
+            if (d == 0) {
+                p.part_ml[prow * 2 + 0] = mx;
+                p.part_ml[prow * 2 + 1] = l;
+            }
+        }
+    }
+}
+
+// One workgroup of 256 lanes per (decode sequence, query head): 8 groups of 32 lanes stride over the chunks the
+// sequence really has, each lane owning 4 channels; the groups' running (max, sum, acc) are combined through LDS.
+// out[d] = sum_c w_c acc_c[d] / sum_c w_c l_c with w_c = exp2(m_c - max_c m_c).
+constexpr int kMergeGroups = 8;
+__global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p) {
+    __shared__ float red[kMergeGroups][kDh + 2];
     const int b = blockIdx.y;
     const int head = blockIdx.x;
-    const int d = threadIdx.x;
+    const int g = threadIdx.x >> 5;
+    const int d4 = (threadIdx.x & 31) * 4;
     const int64_t kvlen = p.kvstarts[b + 1] - p.kvstarts[b];
     const int nc = (int)((kvlen + p.chunk - 1) / p.chunk);
     const int64_t base = (int64_t)b * p.num_chunks * p.num_heads + head;
-    float mx = -INFINITY;
-    for (int c = 0; c < nc; ++c) mx = fmaxf(mx, p.part_ml[(base + (int64_t)c * p.num_heads) * 2]);
-    float acc = 0.f, l = 0.f;
-    for (int c = 0; c < nc; ++c) {
+    float mx = -INFINITY, l = 0.f;
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int c = g; c < nc; c += kMergeGroups) {
         const int64_t prow = base + (int64_t)c * p.num_heads;
-        const float w = __builtin_amdgcn_exp2f(p.part_ml[prow * 2] - mx);
-        l += w * p.part_ml[prow * 2 + 1];
-        acc += w * p.part_acc[prow * kDh + d];
+        const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
+        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
+        const float m_new = fmaxf(mx, mc);
+        const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc - m_new);
+        acc = acc * w_old + a * w_new;
+        l = l * w_old + lc * w_new;
+        mx = m_new;
     }
-    p.out[(p.seqstarts[b] * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
+    red[g][d4 + 0] = acc[0];
+    red[g][d4 + 1] = acc[1];
+    red[g][d4 + 2] = acc[2];
+    red[g][d4 + 3] = acc[3];
+    if ((threadIdx.x & 31) == 0) {
+        red[g][kDh] = mx;
+        red[g][kDh + 1] = l;
+    }
+    __syncthreads();
+    if (threadIdx.x < kDh) {
+        const int d = threadIdx.x;
+        float M = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < kMergeGroups; ++i) M = fmaxf(M, red[i][kDh]);
+        float a = 0.f, L = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMergeGroups; ++i) {
+            const float w = __builtin_amdgcn_exp2f(red[i][kDh] - M); // groups that saw no chunk have max -inf -> 0
+            a += w * red[i][d];
+            L += w * red[i][kDh + 1];
+        }
+        p.out[(p.seqstarts[b] * p.num_heads + head) * kDh + d] = (half_t)(a / L);
+    }
 }
 
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
@@ -313,19 +577,34 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     p.rep = a->num_heads / a->num_kv_heads;
     p.chunk = plan->decode_chunk_tokens;
     p.num_chunks = plan->decode_num_chunks;
-    p.total_tasks = (int64_t)nd * p.num_chunks * p.kv_heads;
+    p.hpb = 1;
+    while (p.hpb < kDecodeWaves && p.kv_heads % (p.hpb * 2) == 0) p.hpb *= 2;
+    p.num_chunks_pad8 = (p.num_chunks + 7) / 8 * 8;
+    p.total_tasks = (int64_t)nd * p.num_chunks_pad8 * (p.kv_heads / p.hpb);
+    if (p.chunk <= 0 || p.chunk % (kDecodeWaves * kStageTokens))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: chunk %d is not a multiple of %d", p.chunk, kDecodeWaves * kStageTokens);
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
     const size_t acc_bytes = (size_t)nd * p.num_chunks * p.num_heads * kDh * sizeof(float);
     p.part_acc = (float*)ws;
     p.part_ml = (float*)((char*)ws + acc_bytes);
     if (p.num_chunks > 1 && ws == nullptr)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: split-k needs the workspace reported by pplhip_mhca_prepare");
-    const int64_t blocks = (p.total_tasks + kDecodeWaves - 1) / kDecodeWaves;
+    const int64_t blocks = p.total_tasks;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many tasks");
-    hipLaunchKernelGGL(decode_int8kv_kernel, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), 0, stream, p);
+    const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
+    static bool lds_opt_in = false; // more than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in
+    if (!lds_opt_in) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_int8kv_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess)
+            PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
+                        lds_bytes, hipGetErrorString(e));
+        lds_opt_in = true;
+    }
+    hipLaunchKernelGGL(decode_int8kv_kernel, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
     if (p.num_chunks > 1) {
-        hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(kDh), 0, stream, p);
+        hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
         PPLHIP_CHECK_LAUNCH("decode_merge");
     }
     return PPLHIP_RC_SUCCESS;

@@ -41,6 +41,8 @@ def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, 
     for k, v in st.items():
         setattr(w, k, v)
     w.d_cache, w.d_scale = ptr(cache), ptr(scale)
+    # the struct only holds raw addresses: keep the arrays (often temporaries such as b.histstarts) alive with it
+    w._refs = getattr(w, "_refs", []) + [key, value, seqstarts, start_pos, cachestarts, cache, scale]
     return w
 
 
@@ -67,6 +69,7 @@ def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, c
     a.specify_decoding_attn_tpb = 0
     a.d_cache, a.d_scale, a.d_output = ptr(cache), ptr(scale), ptr(out)
     a.total_new_tokens = b.total_new_tokens
+    a._refs = [q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out]
     return a
 
 

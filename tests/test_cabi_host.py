@@ -53,7 +53,7 @@ def _valid_args():
 def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
     a, plan = _valid_args(), cabi.MhcaPlan()
     assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
-    assert plan.decode_chunk_tokens >= 11 and plan.decode_chunk_tokens % 64 == 0
+    assert plan.decode_chunk_tokens >= 11 and plan.decode_chunk_tokens % 128 == 0
     assert plan.decode_num_chunks == 1 and plan.workspace_bytes == 0
     assert plan.prefill_q_tile == 128 and plan.prefill_num_q_tiles == 1
     a.max_kvlen, a.specify_decoding_attn_split_k = 100000, 2

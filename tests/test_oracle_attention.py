@@ -156,6 +156,7 @@ def test_kv_cache_op(olib):
     harness.fill_write_args(a.write, b, t["current_key"], t["current_value"], seqstarts, sp, b.cachestarts, cache,
                             scale)
     a.d_kvstarts = kvstarts.ctypes.data
+    a._refs2 = [kvstarts]
     a.total_kv_tokens, a.max_kvlen = int(kvstarts[-1]), b.max_kvlen
     a.num_repeat, a.cache_mode, a.cache_layout = 1, 0, 0
     ko = np.zeros((int(kvstarts[-1]), 2, 128), np.float16)
