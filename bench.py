@@ -212,7 +212,7 @@ def main():
         "dtype": "int8 KV + fp16 (fp32 accumulate)",
         "data": "synthetic",
         "config": {"workload": wname, "decode_seqs": nd, "kv_tokens": int(dec_b.kvlens.sum()),
-                   "chunk_tokens": int(dec.plan.decode_chunk_tokens), "num_chunks": int(dec.plan.decode_num_chunks),
+                   "decode_ranges": int(dec.plan.decode_num_ranges), "kv_heads_per_workgroup": int(dec.plan.decode_heads_per_block),
                    "slabs_rotated": N_SLABS},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": None,

@@ -97,7 +97,7 @@ typedef struct pplhip_mhca_args {
     int32_t enable_decoding_sharemem_mhca; /* accepted, ignored: one decode algorithm serves every shape */
     int32_t enable_decoding_infinity_mhca; /* accepted, ignored */
     int32_t enable_decoding_infinity_gqca; /* accepted, ignored */
-    int32_t specify_decoding_attn_split_k; /* 0 off, 1 heuristic, 2 always */
+    int32_t specify_decoding_attn_split_k; /* 0 coarsest split (1 range per workgroup slot), 1 heuristic, 2 finest */
     int32_t specify_decoding_attn_tpb; /* 0 heuristic, 256, 512 */
     void* d_cache;
     void* d_scale;
@@ -109,8 +109,9 @@ typedef struct pplhip_mhca_args {
  * `cfg.workspace_size` and sets `cfg.workspace`). Filled by pplhip_mhca_prepare, consumed by pplhip_mhca_forward. */
 typedef struct pplhip_mhca_plan {
     uint64_t workspace_bytes; /* device scratch the caller must pass to forward (may be 0) */
-    int32_t decode_chunk_tokens; /* cached tokens handled by one wavefront task (split-k granularity) */
-    int32_t decode_num_chunks; /* ceil(max_kvlen / decode_chunk_tokens) */
+    int32_t decode_num_ranges; /* S: the cached tokens of all decode sequences, laid end to end, are cut into S equal
+                                  ranges on the device (split-k granularity); one workgroup per range and head group */
+    int32_t decode_heads_per_block; /* kv heads served by one decode workgroup (1, 2 or 4) */
     int32_t decode_waves_per_block;
     int32_t prefill_q_tile; /* query rows per prefill workgroup */
     int32_t prefill_num_q_tiles; /* ceil(max_seqlen / prefill_q_tile) */
@@ -119,7 +120,7 @@ typedef struct pplhip_mhca_plan {
 
 /* Host-only: validates `args` exactly like the reference wrapper + kernel library would
  * (unsupported attrs -> PPLHIP_RC_UNSUPPORTED, inconsistent sizes -> PPLHIP_RC_INVALID_VALUE),
- * picks the split-k decomposition and reports the workspace size. Replaces `heuristic_prepare`
+ * picks the split-k decomposition (how many equal token ranges) and reports the workspace size. Replaces `heuristic_prepare`
  * (multi_head_cache_attention_kernel.cc:170). Does not touch the device. */
 pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* args, pplhip_mhca_plan* plan);
 

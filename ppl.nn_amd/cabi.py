@@ -48,7 +48,7 @@ class MhcaArgs(C.Structure):
 class MhcaPlan(C.Structure):
     _fields_ = [
         ("workspace_bytes", C.c_uint64),
-        ("decode_chunk_tokens", _i32), ("decode_num_chunks", _i32), ("decode_waves_per_block", _i32),
+        ("decode_num_ranges", _i32), ("decode_heads_per_block", _i32), ("decode_waves_per_block", _i32),
         ("prefill_q_tile", _i32), ("prefill_num_q_tiles", _i32),
         ("reserved", _i32 * 3),
     ]

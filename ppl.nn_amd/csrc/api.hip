@@ -130,41 +130,29 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     if (a->specify_decoding_attn_tpb != 0 && a->specify_decoding_attn_tpb != 256 && a->specify_decoding_attn_tpb != 512)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_tpb must be 0, 256 or 512");
 
-    // ---- decode: split the cached tokens into chunks, one workgroup (4 waves) per (sequence, kv head, chunk)
+    // ---- decode: the kernel cuts the decode sequences' cached tokens, laid end to end, into S equal ranges on the
+    // device; the host only picks S from the chip size. One workgroup (4 waves) per range and group of <= 4 kv heads,
+    // two resident workgroups per CU.
     plan->decode_waves_per_block = 4;
     const int64_t nd = a->decoding_batches;
-    if (nd > 0 && a->max_kvlen > 0) {
-        const int64_t round = 128; // 4 waves x 32-token pipeline stages
-        int64_t chunk;
-        const int64_t whole = (a->max_kvlen + round - 1) / round * round;
-        if (a->specify_decoding_attn_split_k == 0) {
-            chunk = whole;
-        } else {
-            // Workgroup slots on the chip (2 resident workgroups per CU); a workgroup serves up to 4 kv heads of one
-            // (sequence, chunk). Aim at ~6 tasks per slot for a ragged batch whose sequences average half of
-            // max_kvlen, so that the tail of the launch is a small fraction of it.
-            const int64_t slots = (int64_t)device_cu_count() * 2;
-            int hpb = 1;
-            while (hpb < 4 && a->num_kv_heads % (hpb * 2) == 0) hpb *= 2;
-            const int64_t pairs = nd * (a->num_kv_heads / hpb);
-            chunk = (a->max_kvlen * pairs / 2 + 6 * slots - 1) / (6 * slots);
-            chunk = (chunk + round - 1) / round * round;
-            if (chunk < 256) chunk = 256; // below this the per-task partial (Dh+2 floats per head) stops being noise
-            if (chunk > whole) chunk = whole;
-            if (a->specify_decoding_attn_split_k == 2 && chunk >= whole && whole > round)
-                chunk = (whole / 2 + round - 1) / round * round;
-            if (const char* env = getenv("PPLHIP_DECODE_CHUNK")) { // tuning aid: force the split granularity
-                const int64_t forced = atoll(env);
-                if (forced > 0) chunk = (forced + round - 1) / round * round;
-                if (chunk > whole) chunk = whole;
-            }
+    if (nd > 0) {
+        const int hpb = decode_heads_per_block(a->num_kv_heads);
+        const int64_t groups = a->num_kv_heads / hpb;
+        const int64_t slots = (int64_t)device_cu_count() * 2;
+        int64_t per_slot = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
+        if (const char* env = getenv("PPLHIP_DECODE_TASKS_PER_SLOT")) { // tuning aid
+            if (atoll(env) > 0) per_slot = atoll(env);
         }
-        plan->decode_chunk_tokens = (int32_t)chunk;
-        plan->decode_num_chunks = (int32_t)((a->max_kvlen + chunk - 1) / chunk);
-        if (plan->decode_num_chunks > 1) {
-            const uint64_t rows = (uint64_t)nd * plan->decode_num_chunks * a->num_heads;
-            plan->workspace_bytes = rows * (a->head_dim + 2) * sizeof(float);
-        }
+        int64_t ranges = (slots * per_slot + groups - 1) / groups;
+        // never more ranges than 128-token pieces of the worst case (every sequence max_kvlen long)
+        const int64_t cap = (nd * a->max_kvlen + 127) / 128;
+        if (ranges > cap) ranges = cap;
+        ranges = (ranges + 7) / 8 * 8;
+        if (ranges > 0x3fffffff) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many ranges");
+        plan->decode_num_ranges = (int32_t)ranges;
+        plan->decode_heads_per_block = hpb;
+        const uint64_t rows = ((uint64_t)ranges + (uint64_t)nd) * a->num_heads;
+        plan->workspace_bytes = rows * (a->head_dim + 2) * sizeof(float);
     }
     // ---- prefill
     plan->prefill_q_tile = 128;
@@ -181,7 +169,7 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     if (plan->workspace_bytes > 0 && (!d_workspace || ((uintptr_t)d_workspace & 255)))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "workspace of %llu bytes (256-byte aligned) required",
                     (unsigned long long)plan->workspace_bytes);
-    if (a->decoding_batches > 0 && plan->decode_chunk_tokens <= 0)
+    if (a->decoding_batches > 0 && plan->decode_num_ranges <= 0)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
     hipStream_t s = (hipStream_t)stream;
     pplhip_kv_write_args w;

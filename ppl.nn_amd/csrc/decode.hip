@@ -11,9 +11,14 @@
 //   * All H/KVH query heads of a kv head ride in the 16-wide N dimension of v_mfma_f32_16x16x32_f16, so a KV byte is
 //     read once whatever the grouping, and the contraction costs two dozen MFMAs per 32 tokens.
 //
-// Work decomposition: one workgroup = one task (sequence b, kv head, chunk of `chunk` cached tokens); its 4 waves take
-// a quarter of the chunk each and combine their softmax states through LDS at the end. Tasks are ordered
-// kv-head-fastest so that neighbouring workgroups read neighbouring bytes of the (MaxT, L, 2, KVH, Dh) slab.
+// Work decomposition (balanced on the device, no host knowledge of the lengths): the cached tokens of all decode
+// sequences, laid end to end (kvstarts is exactly that prefix sum), are cut into S equal ranges. One workgroup owns one
+// range for a group of up to 4 kv heads; where its range crosses sequence boundaries it handles the pieces ("segments")
+// one after the other. Every workgroup therefore streams the same number of bytes, whatever the raggedness of the batch,
+// and there is no tail of long sequences. Inside a workgroup each wave owns one kv head (the workgroup then reads
+// hpb * 128 contiguous bytes of every token) or, with fewer than 4 kv heads, a share of the segment's tokens.
+// Workgroups are numbered so that the head groups of one range start on the same XCD (workgroup i runs on XCD i % 8):
+// their neighbouring rows then meet in one L2 and reach the same DRAM pages together.
 //
 // LDS layout of one 32-token stage of one wave (10 KiB): K rows [32][128 B], V rows [32][128 B], K scales [32][32 B],
 // V scales [32][32 B]. Inside a K/V row the eight 16 B pieces are XOR-swizzled with (row & 7) by choosing which
@@ -29,9 +34,10 @@
 // int8 -> fp16 is exact: (x ^ 0x80) placed under exponent byte 0x64 reads as 1024 + (x + 128); subtract 1152, then
 // multiply by the group's fp16 scale (packed fp16 ops). Softmax runs online in the exp2 domain with fp32 statistics.
 //
-// Each task writes one un-normalised partial (max, sum, acc[Dh]) per query head into the workspace and
-// `decode_merge_kernel` combines the chunks of a sequence with the usual log-sum-exp weights. With a single chunk the
-// task normalises and writes fp16 output itself.
+// A segment that is a whole sequence is normalised and written as fp16 output directly. Otherwise the workgroup writes
+// one un-normalised partial (max, sum, acc[Dh]) per query head into workspace slot (range index + sequence index) --
+// consecutive (range, sequence) segments get consecutive slots -- and `decode_merge_kernel` combines the slots of a
+// sequence with the usual log-sum-exp weights.
 #include "common.h"
 
 namespace pplhip {
@@ -57,17 +63,22 @@ struct DecodeParams {
     const int64_t* kvstarts;
     const int64_t* cachestarts;
     half_t* out; // [S, H, Dh]
-    float* part_acc; // [nd, chunks, H, Dh]
-    float* part_ml; // [nd, chunks, H, 2]
+    float* part_acc; // [slots, H, Dh], slots = num_ranges + nd
+    float* part_ml; // [slots, H, 2]
     CacheAddr addr;
-    int32_t nd; // decode sequences
+    int32_t nd; // decode sequences (the first nd entries of the tables)
     int32_t num_heads, kv_heads, rep; // rep = num_heads / kv_heads (<= 16)
-    int32_t chunk, num_chunks; // chunk is a multiple of kDecodeWaves * kStageTokens
-    int32_t num_chunks_pad8; // num_chunks rounded up to a multiple of 8 (task grid only)
+    int32_t num_ranges; // S, a multiple of 8
     int32_t hpb; // kv heads per workgroup: min(kv_heads, 4), a power of two dividing kv_heads
-    int64_t total_tasks;
     float score_scale; // log2(e) / sqrt(Dh)
 };
+
+// Tokens per range: the total is only known on the device. At least 128 so that tiny batches are not shredded.
+__device__ inline int64_t range_tokens(int64_t total, int num_ranges) {
+    int64_t r = (total + num_ranges - 1) / num_ranges;
+    r = (r + 31) & ~(int64_t)31;
+    return r < 128 ? 128 : r;
+}
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
@@ -164,11 +175,7 @@ struct DmaOffsets {
 
 // rows_mem: rows of the stage that exist in the chunk (1..32); later rows are clamped onto the last one
 __device__ inline void make_dma_offsets(DmaOffsets& o, int lane, uint32_t stride, uint32_t sstride_b, int rows_mem) {
-#ifdef PPLHIP_X_NOSWZ
-    const int piece = (lane & 7);
-#else
     const int piece = (lane & 7) ^ (lane >> 3); // LDS slot (lane & 7) of row r holds global piece slot ^ (r & 7)
-#endif
 #pragma unroll
     for (int i = 0; i < kStageTokens / 8; ++i) {
         int r = 8 * i + (lane >> 3);
@@ -191,13 +198,8 @@ __device__ inline void dma_stage(char* lds_stage, const char* cbase, const char*
         __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + kv_off + o.kv[i]), (lds_ptr_t)(lds_stage + kLdsV + 1024 * i),
                                          16, 0, 0);
     }
-#ifdef PPLHIP_X_NOSCALEDMA
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + o.kv[0]), (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + o.kv[1]), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
-#else
     __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + o.sc), (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
     __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + kv_off_s + o.sc), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
-#endif
 }
 
 // Per-lane LDS read offsets inside a stage (they are the same for every stage).
@@ -344,174 +346,168 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
-    // Task = (sequence b, chunk c, group of hpb kv heads). The waves of the workgroup are (kv head within the group)
-    // x (token split): with 4 or more kv heads every wave owns one head and the whole chunk, so the workgroup as a
-    // whole reads hpb * 128 contiguous bytes of every token; with fewer heads the waves split the chunk's tokens.
-    //
-    // XCD-aware task order: workgroups are dealt round-robin to the 8 XCDs (workgroup i runs on XCD i % 8), each with
-    // its own L2. The head groups of one (sequence, chunk) read neighbouring rows of the same slab tokens, so they are
-    // given to workgroups i, i + 8, i + 16, ... that start on the same XCD at about the same time: their requests then
-    // meet in one L2 and reach the same DRAM pages together.
-    // Ragged batches: chunk c of sequence b goes to XCD (b + c) % 8, so a sequence's chunks walk round the XCDs starting
-    // at a different one per sequence and every XCD gets its share of the short and of the long sequences. The chunk
-    // count is padded to a multiple of 8 for that; padded tasks exit at once.
     const int groups = p.kv_heads / p.hpb;
     const int xcd = blockIdx.x & 7;
     const int64_t j = blockIdx.x >> 3;
     const int hg = (int)(j % groups);
-    const int64_t g = j / groups;
-    const int c8 = p.num_chunks_pad8 >> 3;
-    const int b = (int)(g / c8);
-    const int c = (int)(g % c8) * 8 + ((xcd - b) & 7);
-    if (c >= p.num_chunks) return;
+    const int64_t s_idx = (j / groups) * 8 + xcd; // range index
+    const int64_t total = p.kvstarts[p.nd];
+    const int64_t R = range_tokens(total, p.num_ranges);
+    const int64_t r0 = s_idx * R;
+    if (r0 >= total) return;
+    const int64_t r1 = (r0 + R < total) ? r0 + R : total;
+
     const int kvh_local = wave & (p.hpb - 1);
     const int kvh = hg * p.hpb + kvh_local;
     const int tsplits = kDecodeWaves / p.hpb;
     const int ts = wave / p.hpb;
-    const int64_t kv_lo = p.kvstarts[b], kv_hi = p.kvstarts[b + 1];
-    const int64_t tok0 = p.cachestarts[b];
-    const int64_t qrow = p.seqstarts[b];
-    const int64_t kvlen = kv_hi - kv_lo;
-    const int64_t c_begin = (int64_t)c * p.chunk;
-    if (c_begin >= kvlen) return; // block-uniform: this sequence has fewer chunks; the merge pass never looks here
-    const int64_t c_end = (c_begin + p.chunk < kvlen) ? c_begin + p.chunk : kvlen;
-    const int sub = p.chunk / tsplits;
-    const int64_t t_begin = c_begin + (int64_t)ts * sub;
-    const int64_t t_end = (t_begin + sub < c_end) ? t_begin + sub : c_end; // may be <= t_begin: wave has no tokens
-
     const int m = lane & 15;
     const int kq = lane >> 4;
 
-    // ---- Q^T as the B operand, kept for the whole task: qB[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
-    half8_t qB[2][2];
-    {
-        const bool live = m < p.rep;
-        const half_t* qp = p.q + ((qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                uint4 x = *reinterpret_cast<const uint4*>(qp + 32 * kq + 16 * j + 8 * i);
-                if (!live) x = make_uint4(0, 0, 0, 0);
-                __builtin_memcpy(&qB[j][i], &x, 16);
-            }
-    }
-
-    SoftmaxState ss;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) ss.oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    ss.m_run = -INFINITY;
-    ss.l_part = 0.f;
-
+    const uint32_t stride = (uint32_t)p.addr.stride_s; // bytes between tokens (int8 elements)
+    const uint32_t sstride_b = (uint32_t)(p.addr.stride_s / kQuantGroup) * 2u;
+    const uint32_t kv_off = (uint32_t)p.addr.stride_kv;
+    const uint32_t kv_off_s = (uint32_t)(p.addr.stride_kv / kQuantGroup) * 2u;
+    const int64_t step_c = (int64_t)kStageTokens * stride, step_s = (int64_t)kStageTokens * sstride_b;
+    DmaOffsets full;
+    make_dma_offsets(full, lane, stride, sstride_b, kStageTokens);
+    ReadOffsets ro;
+    make_read_offsets(ro, m, kq);
     char* wave_lds = smem + wave * kWaveLdsBytes;
     const uint32_t wave_lds_addr =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem + wave * kWaveLdsBytes;
-    if (t_begin < t_end) {
-        const uint32_t stride = (uint32_t)p.addr.stride_s; // bytes between tokens (int8 elements)
-        const uint32_t sstride_b = (uint32_t)(p.addr.stride_s / kQuantGroup) * 2u;
-        const uint32_t kv_off = (uint32_t)p.addr.stride_kv;
-        const uint32_t kv_off_s = (uint32_t)(p.addr.stride_kv / kQuantGroup) * 2u;
-        const int64_t row0 = p.addr.row(tok0 + t_begin, 0, kvh);
-        const char* cbase = reinterpret_cast<const char*>(p.cache) + row0;
-        const char* sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
-        const int64_t step_c = (int64_t)kStageTokens * stride, step_s = (int64_t)kStageTokens * sstride_b;
-        DmaOffsets full;
-        make_dma_offsets(full, lane, stride, sstride_b, kStageTokens);
-        ReadOffsets ro;
-        make_read_offsets(ro, m, kq);
-        // The wave's last stage may overhang: rows past the end of the CHUNK are clamped onto its last row (loads must
-        // stay inside memory the sequence owns) and everything past the wave's own range is masked in the softmax.
-        const int n_stages = (int)((t_end - t_begin + kStageTokens - 1) / kStageTokens);
-        const int64_t last_stage_t0 = t_begin + (int64_t)(n_stages - 1) * kStageTokens;
-        const int tail_rows_mem = (int)((c_end - last_stage_t0) < kStageTokens ? (c_end - last_stage_t0) : kStageTokens);
-        const int tail_rows_valid = (int)(t_end - last_stage_t0);
-        auto issue = [&](int idx) {
-            char* dst = wave_lds + (idx & 1) * kStageBytes;
-            const char* cb = make_uniform(cbase + idx * step_c);
-            const char* sb = make_uniform(sbase + idx * step_s);
-#ifdef PPLHIP_X_NODMA
-            if (idx > 0) return;
-#endif
-            if (idx == n_stages - 1 && tail_rows_mem < kStageTokens) { // wave-uniform, at most once per wave
-                DmaOffsets tail;
-                make_dma_offsets(tail, lane, stride, sstride_b, tail_rows_mem);
-                dma_stage(dst, cb, sb, tail, kv_off, kv_off_s);
-            } else {
-                dma_stage(dst, cb, sb, full, kv_off, kv_off_s);
-            }
-        };
-
-        issue(0);
-        // The query loads are older than stage 0's transfers: retire them here, with stage 0 already in flight, so that
-        // no full drain of the DMA queue is needed at their first use inside the loop.
-        PPLHIP_WAIT_VMCNT(kDmaPerStage);
-        for (int it = 0; it < n_stages; ++it) {
-            // the buffer stage it+1 lands in was last read by compute(it-1), which has finished in program order
-            if (it + 1 < n_stages) {
-                issue(it + 1);
-                PPLHIP_WAIT_VMCNT(kDmaPerStage); // everything but the transfers just enqueued has landed
-            } else {
-                PPLHIP_WAIT_VMCNT(0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#ifdef PPLHIP_X_NOCOMPUTE
-            if (it == 0)
-#endif
-            compute_stage(wave_lds_addr + (it & 1) * kStageBytes, ro, ss, qB, kq,
-                          it + 1 == n_stages ? tail_rows_valid : kStageTokens, p.score_scale);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    const float l_tot = wave_sum_over_quads(ss.l_part);
-
-    // ---- combine the token splits of each kv head: LDS layout [wave][head][Dh + 2] (acc, then max, sum), reusing the
-    // stage buffers
-    __syncthreads();
     float* lds = reinterpret_cast<float*>(smem);
     const int row_f = kDh + 2;
-    if (m < p.rep) {
-        float* dst = lds + ((size_t)wave * p.rep + m) * row_f;
+
+    int b = find_sequence(p.kvstarts, p.nd, r0);
+    for (int64_t pos = r0; pos < r1; ++b) {
+        // ---- segment = the part of sequence b inside this range, as token positions of that sequence
+        const int64_t seq_lo = p.kvstarts[b], seq_hi = p.kvstarts[b + 1];
+        const int64_t seg_begin = pos - seq_lo;
+        const int64_t seg_end = ((r1 < seq_hi) ? r1 : seq_hi) - seq_lo;
+        pos = seq_lo + seg_end;
+        const bool whole_sequence = seg_begin == 0 && seg_end == seq_hi - seq_lo;
+        const int64_t tok0 = p.cachestarts[b];
+        const int64_t qrow = p.seqstarts[b];
+        int64_t sub = (seg_end - seg_begin + tsplits - 1) / tsplits;
+        sub = (sub + kStageTokens - 1) / kStageTokens * kStageTokens;
+        const int64_t t_begin = seg_begin + (int64_t)ts * sub;
+        const int64_t t_end = (t_begin + sub < seg_end) ? t_begin + sub : seg_end; // may be <= t_begin: no tokens
+
+        // ---- Q^T as the B operand, kept for the whole segment: qB[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
+        half8_t qB[2][2];
+        {
+            const bool live = m < p.rep;
+            const half_t* qp = p.q + ((qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
+            for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) dst[8 * (4 * kq + e) + i] = ss.oacc[i][e];
-        if (kq == 0) {
-            dst[kDh] = ss.m_run;
-            dst[kDh + 1] = l_tot;
+                for (int i = 0; i < 2; ++i) {
+                    uint4 x = *reinterpret_cast<const uint4*>(qp + 32 * kq + 16 * jj + 8 * i);
+                    if (!live) x = make_uint4(0, 0, 0, 0);
+                    __builtin_memcpy(&qB[jj][i], &x, 16);
+                }
         }
-    }
-    __syncthreads();
-    const int n_out = p.hpb * p.rep * kDh; // (kv head of the group, query head of the kv head, channel)
-    for (int idx = threadIdx.x; idx < n_out; idx += kDecodeWaves * kWave) {
-        const int d = idx & (kDh - 1);
-        const int hh = idx >> 7; // kv_local * rep + h
-        const int kl = hh / p.rep, h = hh - kl * p.rep;
-        float mx = -INFINITY;
-        for (int t = 0; t < tsplits; ++t) mx = fmaxf(mx, lds[((size_t)(t * p.hpb + kl) * p.rep + h) * row_f + kDh]);
-        float acc = 0.f, l = 0.f;
-        for (int t = 0; t < tsplits; ++t) {
-            const float* src = lds + ((size_t)(t * p.hpb + kl) * p.rep + h) * row_f;
-            const float wgt = __builtin_amdgcn_exp2f(src[kDh] - mx); // a wave without tokens has max -inf -> weight 0
-            acc += wgt * src[d];
-            l += wgt * src[kDh + 1];
-        }
-        const int head = (hg * p.hpb + kl) * p.rep + h;
-        if (p.num_chunks == 1) {
-            p.out[(qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
-        } else {
-            const int64_t prow = ((int64_t)b * p.num_chunks + c) * p.num_heads + head;
-            p.part_acc[prow * kDh + d] = acc;
-            if (d == 0) {
-                p.part_ml[prow * 2 + 0] = mx;
-                p.part_ml[prow * 2 + 1] = l;
+
+        SoftmaxState ss;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss.oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+        ss.m_run = -INFINITY;
+        ss.l_part = 0.f;
+
+        if (t_begin < t_end) {
+            const int64_t row0 = p.addr.row(tok0 + t_begin, 0, kvh);
+            const char* cbase = reinterpret_cast<const char*>(p.cache) + row0;
+            const char* sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
+            // The wave's last stage may overhang: rows past the end of the SEGMENT are clamped onto its last row (loads
+            // must stay inside memory the sequence owns) and everything past the wave's own range is masked.
+            const int n_stages = (int)((t_end - t_begin + kStageTokens - 1) / kStageTokens);
+            const int64_t last_stage_t0 = t_begin + (int64_t)(n_stages - 1) * kStageTokens;
+            const int tail_rows_mem =
+                (int)((seg_end - last_stage_t0) < kStageTokens ? (seg_end - last_stage_t0) : kStageTokens);
+            const int tail_rows_valid = (int)(t_end - last_stage_t0);
+            auto issue = [&](int idx) {
+                char* dst = wave_lds + (idx & 1) * kStageBytes;
+                const char* cb = make_uniform(cbase + idx * step_c);
+                const char* sb = make_uniform(sbase + idx * step_s);
+                if (idx == n_stages - 1 && tail_rows_mem < kStageTokens) { // wave-uniform, at most once per segment
+                    DmaOffsets tail;
+                    make_dma_offsets(tail, lane, stride, sstride_b, tail_rows_mem);
+                    dma_stage(dst, cb, sb, tail, kv_off, kv_off_s);
+                } else {
+                    dma_stage(dst, cb, sb, full, kv_off, kv_off_s);
+                }
+            };
+
+            issue(0);
+            // The query loads are older than stage 0's transfers: retire them here, with stage 0 already in flight, so
+            // that no full drain of the DMA queue is needed at their first use inside the loop.
+            PPLHIP_WAIT_VMCNT(kDmaPerStage);
+            for (int it = 0; it < n_stages; ++it) {
+                // the buffer stage it+1 lands in was last read by compute(it-1), which has finished in program order
+                if (it + 1 < n_stages) {
+                    issue(it + 1);
+                    PPLHIP_WAIT_VMCNT(kDmaPerStage); // everything but the transfers just enqueued has landed
+                } else {
+                    PPLHIP_WAIT_VMCNT(0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                compute_stage(wave_lds_addr + (it & 1) * kStageBytes, ro, ss, qB, kq,
+                              it + 1 == n_stages ? tail_rows_valid : kStageTokens, p.score_scale);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+        const float l_tot = wave_sum_over_quads(ss.l_part);
+
+        // ---- combine the token splits of each kv head: LDS layout [wave][head][Dh + 2] (acc, then max, sum), reusing
+        // the stage buffers
+        __syncthreads();
+        if (m < p.rep) {
+            float* dst = lds + ((size_t)wave * p.rep + m) * row_f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) dst[8 * (4 * kq + e) + i] = ss.oacc[i][e];
+            if (kq == 0) {
+                dst[kDh] = ss.m_run;
+                dst[kDh + 1] = l_tot;
+            }
+        }
+        __syncthreads();
+        const int n_out = p.hpb * p.rep * kDh; // (kv head of the group, query head of the kv head, channel)
+        for (int idx = threadIdx.x; idx < n_out; idx += kDecodeWaves * kWave) {
+            const int d = idx & (kDh - 1);
+            const int hh = idx >> 7; // kv_local * rep + h
+            const int kl = hh / p.rep, h = hh - kl * p.rep;
+            float mx = -INFINITY;
+            for (int t = 0; t < tsplits; ++t) mx = fmaxf(mx, lds[((size_t)(t * p.hpb + kl) * p.rep + h) * row_f + kDh]);
+            float acc = 0.f, l = 0.f;
+            for (int t = 0; t < tsplits; ++t) {
+                const float* src = lds + ((size_t)(t * p.hpb + kl) * p.rep + h) * row_f;
+                const float wgt = __builtin_amdgcn_exp2f(src[kDh] - mx); // a wave without tokens has max -inf -> 0
+                acc += wgt * src[d];
+                l += wgt * src[kDh + 1];
+            }
+            const int head = (hg * p.hpb + kl) * p.rep + h;
+            if (whole_sequence) {
+                p.out[(qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
+            } else {
+                const int64_t prow = (s_idx + b) * p.num_heads + head;
+                p.part_acc[prow * kDh + d] = acc;
+                if (d == 0) {
+                    p.part_ml[prow * 2 + 0] = mx;
+                    p.part_ml[prow * 2 + 1] = l;
+                }
+            }
+        }
+        __syncthreads(); // the next segment's transfers overwrite the combine area
     }
 }
 
-// One workgroup of 256 lanes per (decode sequence, query head): 8 groups of 32 lanes stride over the chunks the
-// sequence really has, each lane owning 4 channels; the groups' running (max, sum, acc) are combined through LDS.
-// out[d] = sum_c w_c acc_c[d] / sum_c w_c l_c with w_c = exp2(m_c - max_c m_c).
+// One workgroup of 256 lanes per (decode sequence, query head): 8 groups of 32 lanes stride over the partial slots of
+// the sequence (one per range it touches), each lane owning 4 channels; the groups' running (max, sum, acc) are combined
+// through LDS. out[d] = sum_s w_s acc_s[d] / sum_s w_s l_s with w_s = exp2(m_s - max_s m_s). Sequences that lie inside a
+// single range were already written by the decode kernel.
 constexpr int kMergeGroups = 8;
 __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p) {
     __shared__ float red[kMergeGroups][kDh + 2];
@@ -519,13 +515,13 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
     const int head = blockIdx.x;
     const int g = threadIdx.x >> 5;
     const int d4 = (threadIdx.x & 31) * 4;
-    const int64_t kvlen = p.kvstarts[b + 1] - p.kvstarts[b];
-    const int nc = (int)((kvlen + p.chunk - 1) / p.chunk);
-    const int64_t base = (int64_t)b * p.num_chunks * p.num_heads + head;
+    const int64_t R = range_tokens(p.kvstarts[p.nd], p.num_ranges);
+    const int64_t s_lo = p.kvstarts[b] / R, s_hi = (p.kvstarts[b + 1] - 1) / R;
+    if (s_lo == s_hi) return;
     float mx = -INFINITY, l = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c = g; c < nc; c += kMergeGroups) {
-        const int64_t prow = base + (int64_t)c * p.num_heads;
+    for (int64_t s = s_lo + g; s <= s_hi; s += kMergeGroups) {
+        const int64_t prow = (s + b) * p.num_heads + head;
         const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
         const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
         const float m_new = fmaxf(mx, mc);
@@ -551,12 +547,18 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
         float a = 0.f, L = 0.f;
 #pragma unroll
         for (int i = 0; i < kMergeGroups; ++i) {
-            const float w = __builtin_amdgcn_exp2f(red[i][kDh] - M); // groups that saw no chunk have max -inf -> 0
+            const float w = __builtin_amdgcn_exp2f(red[i][kDh] - M); // groups that saw no slot have max -inf -> 0
             a += w * red[i][d];
             L += w * red[i][kDh + 1];
         }
         p.out[(p.seqstarts[b] * p.num_heads + head) * kDh + d] = (half_t)(a / L);
     }
+}
+
+int decode_heads_per_block(int kv_heads) {
+    int hpb = 1;
+    while (hpb < kDecodeWaves && kv_heads % (hpb * 2) == 0) hpb *= 2;
+    return hpb;
 }
 
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
@@ -575,21 +577,16 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     p.num_heads = a->num_heads;
     p.kv_heads = a->num_kv_heads;
     p.rep = a->num_heads / a->num_kv_heads;
-    p.chunk = plan->decode_chunk_tokens;
-    p.num_chunks = plan->decode_num_chunks;
-    p.hpb = 1;
-    while (p.hpb < kDecodeWaves && p.kv_heads % (p.hpb * 2) == 0) p.hpb *= 2;
-    p.num_chunks_pad8 = (p.num_chunks + 7) / 8 * 8;
-    p.total_tasks = (int64_t)nd * p.num_chunks_pad8 * (p.kv_heads / p.hpb);
-    if (p.chunk <= 0 || p.chunk % (kDecodeWaves * kStageTokens))
-        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: chunk %d is not a multiple of %d", p.chunk, kDecodeWaves * kStageTokens);
+    p.num_ranges = plan->decode_num_ranges;
+    p.hpb = decode_heads_per_block(p.kv_heads);
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
-    const size_t acc_bytes = (size_t)nd * p.num_chunks * p.num_heads * kDh * sizeof(float);
+    if (p.num_ranges <= 0 || (p.num_ranges & 7) || plan->decode_heads_per_block != p.hpb)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: plan was not produced by pplhip_mhca_prepare for these arguments");
+    if (ws == nullptr) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: needs the workspace reported by pplhip_mhca_prepare");
+    const size_t slots = (size_t)p.num_ranges + nd;
     p.part_acc = (float*)ws;
-    p.part_ml = (float*)((char*)ws + acc_bytes);
-    if (p.num_chunks > 1 && ws == nullptr)
-        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: split-k needs the workspace reported by pplhip_mhca_prepare");
-    const int64_t blocks = p.total_tasks;
+    p.part_ml = (float*)((char*)ws + slots * p.num_heads * kDh * sizeof(float));
+    const int64_t blocks = (int64_t)p.num_ranges * (p.kv_heads / p.hpb);
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many tasks");
     const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
     static bool lds_opt_in = false; // more than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in
@@ -603,10 +600,8 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     }
     hipLaunchKernelGGL(decode_int8kv_kernel, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
-    if (p.num_chunks > 1) {
-        hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
-        PPLHIP_CHECK_LAUNCH("decode_merge");
-    }
+    hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
+    PPLHIP_CHECK_LAUNCH("decode_merge");
     return PPLHIP_RC_SUCCESS;
 }
 

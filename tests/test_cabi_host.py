@@ -53,13 +53,18 @@ def _valid_args():
 def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
     a, plan = _valid_args(), cabi.MhcaPlan()
     assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
-    assert plan.decode_chunk_tokens >= 11 and plan.decode_chunk_tokens % 128 == 0
-    assert plan.decode_num_chunks == 1 and plan.workspace_bytes == 0
+    # 1 decode sequence of 11 tokens: one 128-token piece at most -> 8 ranges (one per XCD), 2 kv heads per workgroup
+    assert plan.decode_num_ranges == 8 and plan.decode_heads_per_block == 2 and plan.decode_waves_per_block == 4
+    assert plan.workspace_bytes >= (8 + 1) * 8 * 130 * 4 and plan.workspace_bytes % 256 == 0
     assert plan.prefill_q_tile == 128 and plan.prefill_num_q_tiles == 1
-    a.max_kvlen, a.specify_decoding_attn_split_k = 100000, 2
-    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
-    assert plan.decode_num_chunks * plan.decode_chunk_tokens >= 100000 and plan.decode_num_chunks > 1
-    assert plan.workspace_bytes >= 1 * plan.decode_num_chunks * 8 * 130 * 4 and plan.workspace_bytes % 256 == 0
+    sizes = []
+    for mode in (0, 1, 2):
+        a.max_kvlen, a.specify_decoding_attn_split_k = 1000000, mode
+        assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+        assert plan.decode_num_ranges % 8 == 0
+        assert plan.workspace_bytes >= (plan.decode_num_ranges + 1) * 8 * 130 * 4
+        sizes.append(plan.decode_num_ranges)
+    assert sizes[0] < sizes[1] < sizes[2]
 
 
 @pytest.mark.parametrize("mutate,rc", [

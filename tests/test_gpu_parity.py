@@ -78,13 +78,13 @@ def test_cache_prefill_with_start_pos():
 
 def test_split_k_modes_agree():
     """Split count must not change the result beyond fp32 reassociation."""
-    b = workloads.Batch(8, 2, 128, [1, 1, 1], [2999, 700, 64], 3, name="split_k")
+    b = workloads.Batch(8, 2, 128, [1, 1, 1], [49999, 7000, 64], 3, name="split_k")
     t = workloads.make_tensors(b, seed=5)
     outs, plans = [], []
     for mode in (0, 1, 2):
         _, ref, got = check(b, t, split_k=mode, plans=plans)
         outs.append(got["output"].astype(np.float64))
-    assert plans[0].decode_num_chunks == 1 and plans[2].decode_num_chunks > 1
+    assert plans[0].decode_num_ranges < plans[1].decode_num_ranges <= plans[2].decode_num_ranges
     assert np.abs(outs[0] - outs[1]).max() < 1e-3 and np.abs(outs[0] - outs[2]).max() < 1e-3
 
 
