@@ -139,11 +139,13 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         const int hpb = decode_heads_per_block(a->num_kv_heads);
         const int64_t groups = a->num_kv_heads / hpb;
         const int64_t slots = (int64_t)device_cu_count() * 2;
-        int64_t per_slot = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
-        if (const char* env = getenv("PPLHIP_DECODE_TASKS_PER_SLOT")) { // tuning aid
-            if (atoll(env) > 0) per_slot = atoll(env);
+        // halves of a slot: every workgroup streams the same number of bytes, so one workgroup per slot (a single,
+        // perfectly filled round) measures best; the knob moves it to half or twice that
+        int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
+        if (const char* env = getenv("PPLHIP_DECODE_TASKS_PER_SLOT")) { // tuning aid, in workgroups per slot
+            if (atoll(env) > 0) half_slots = 2 * atoll(env);
         }
-        int64_t ranges = (slots * per_slot + groups - 1) / groups;
+        int64_t ranges = (slots * half_slots / 2 + groups - 1) / groups;
         // never more ranges than 128-token pieces of the worst case (every sequence max_kvlen long)
         const int64_t cap = (nd * a->max_kvlen + 127) / 128;
         if (ranges > cap) ranges = cap;

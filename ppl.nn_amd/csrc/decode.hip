@@ -379,7 +379,15 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     float* lds = reinterpret_cast<float*>(smem);
     const int row_f = kDh + 2;
 
-    int b = find_sequence(p.kvstarts, p.nd, r0);
+    // First sequence of the range: count the sequences that end at or before r0. One coalesced vector load per 64
+    // table entries and a ballot, instead of a binary search whose scalar loads would each wait for the previous one.
+    int b = 0;
+    for (int base = 0; base < p.nd; base += kWave) {
+        const int i = base + lane;
+        const bool ends_before = i < p.nd && p.kvstarts[i + 1] <= r0;
+        b += __builtin_popcountll(__ballot(ends_before));
+    }
+    b = __builtin_amdgcn_readfirstlane(b);
     for (int64_t pos = r0; pos < r1; ++b) {
         // ---- segment = the part of sequence b inside this range, as token positions of that sequence
         const int64_t seq_lo = p.kvstarts[b], seq_hi = p.kvstarts[b + 1];
