@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--split-k", type=int, default=1)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device-to-device copy (the reference point for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this same command)")
     return ap.parse_args()
 
 
@@ -165,6 +168,30 @@ def cpu_baseline(db, min_seconds=10.0, max_prepare=24):
                        f"dequantised K/V resident in host memory, {spent:.1f} s of CPU work")
 
 
+PROFILE_TRAFFIC = os.path.join(ROOT, "profiles", "decode_int8kv_cfg2_hbm_traffic.txt")
+
+
+def recorded_traffic(workload):
+    """HBM bytes per decode launch measured offline with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the
+    copy-kernel factor); the summary file carries the commands. None when no figure is recorded for the workload."""
+    if workload != "cfg2" or not os.path.exists(PROFILE_TRAFFIC):
+        return None
+    with open(PROFILE_TRAFFIC) as f:
+        for line in f:
+            if line.startswith("traffic_bytes_per_launch="):
+                return float(line.split("=", 1)[1])
+    return None
+
+
+def copy_calibration():
+    import torch
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(3)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -215,7 +242,7 @@ def main():
                    "decode_ranges": int(dec.plan.decode_num_ranges), "kv_heads_per_workgroup": int(dec.plan.decode_heads_per_block),
                    "slabs_rotated": N_SLABS},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": recorded_traffic(args.workload),
                      "kernel": "decode_int8kv_kernel (+ kv_quantize_write + decode_merge in the same call)",
                      "algorithmic_bytes_per_launch": dec_bytes, "event_ms_per_launch": ev_ms},
     }
@@ -232,6 +259,8 @@ def main():
         _, mix_ms = timed(mixed, max(args.steps // 2, 10), max(args.warmup // 2, 3))
         result["fused_mixed_call_ms"] = mix_ms
         del mixed
+    if args.copy_calibration:
+        copy_calibration()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(dec)
     print(json.dumps(result))
