@@ -53,3 +53,63 @@ def check(rc, what=""):
     if rc != cabi.RC_SUCCESS:
         msg = load_library().pplhip_last_error().decode()
         raise RuntimeError(f"{what} failed: {cabi.RC_NAMES.get(rc, rc)}: {msg}")
+
+
+ENGINE_LIB_PATH = os.path.join(_HERE, "lib", "libpplnn_llm_hip.so")
+_ENGINE = None
+
+
+def load_engine_library():
+    """dlopen the llm_hip host engine (C++) and bind its flat C entry points."""
+    global _ENGINE
+    if _ENGINE is None:
+        load_library()  # the kernel library (and torch's HIP runtime, when present) first
+        if not os.path.exists(ENGINE_LIB_PATH):
+            raise LibraryMissing(f"{ENGINE_LIB_PATH} is not built; run `python __graft_entry__.py`.")
+        L = ctypes.CDLL(ENGINE_LIB_PATH)
+        vp, u32, u64, i64p = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64)
+        sig = {
+            "pplnn_hip_last_error": (ctypes.c_char_p, []),
+            "pplnn_hip_set_log_level": (None, [ctypes.c_int]),
+            "pplnn_hip_engine_create": (vp, [u32, u32]),
+            "pplnn_hip_engine_name": (ctypes.c_char_p, [vp]),
+            "pplnn_hip_engine_configure_u32": (u32, [vp, u32, u32]),
+            "pplnn_hip_engine_destroy": (None, [vp]),
+            "pplnn_hip_builder_create": (vp, []),
+            "pplnn_hip_builder_load_model": (u32, [vp, ctypes.c_char_p, u64]),
+            "pplnn_hip_builder_load_model_file": (u32, [vp, ctypes.c_char_p]),
+            "pplnn_hip_builder_set_engine": (u32, [vp, vp]),
+            "pplnn_hip_builder_preprocess": (u32, [vp]),
+            "pplnn_hip_builder_create_runtime": (vp, [vp]),
+            "pplnn_hip_builder_destroy": (None, [vp]),
+            "pplnn_hip_runtime_input_count": (u32, [vp]),
+            "pplnn_hip_runtime_output_count": (u32, [vp]),
+            "pplnn_hip_runtime_input": (vp, [vp, u32]),
+            "pplnn_hip_runtime_output": (vp, [vp, u32]),
+            "pplnn_hip_runtime_run": (u32, [vp]),
+            "pplnn_hip_runtime_set_profiling": (u32, [vp, u32]),
+            "pplnn_hip_runtime_profiling": (u32, [vp, ctypes.POINTER(u64), ctypes.POINTER(u32), u32]),
+            "pplnn_hip_runtime_destroy": (None, [vp]),
+            "pplnn_hip_tensor_name": (ctypes.c_char_p, [vp]),
+            "pplnn_hip_tensor_reshape": (None, [vp, i64p, u32]),
+            "pplnn_hip_tensor_dims": (u32, [vp, i64p, u32]),
+            "pplnn_hip_tensor_dtype": (u32, [vp]),
+            "pplnn_hip_tensor_set_buffer_ptr": (None, [vp, vp]),
+            "pplnn_hip_tensor_buffer_ptr": (vp, [vp]),
+            "pplnn_hip_tensor_copy_from_host": (u32, [vp, vp]),
+            "pplnn_hip_tensor_copy_to_host": (u32, [vp, vp]),
+            "pplnn_hip_tensor_use_host_device": (None, [vp]),
+            "pplnn_hip_selftest_registry": (u32, []),
+            "pplnn_hip_arena_create_host": (vp, [u64, u64]),
+            "pplnn_hip_arena_alloc": (u32, [vp, u64, ctypes.POINTER(vp), ctypes.POINTER(u64)]),
+            "pplnn_hip_arena_free": (None, [vp, vp]),
+            "pplnn_hip_arena_buffered_bytes": (u64, [vp]),
+            "pplnn_hip_arena_used_bytes": (u64, [vp]),
+            "pplnn_hip_arena_destroy": (None, [vp]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _ENGINE = L
+    return _ENGINE

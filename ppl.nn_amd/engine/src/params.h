@@ -1,0 +1,50 @@
+// Op parameter structs, field for field as in the reference:
+//   src/ppl/nn/params/opmx/multi_head_cache_attention_param.h:10-38
+//   src/ppl/nn/params/opmx/key_value_cache_param.h:10-30
+#ifndef PPLNN_LLM_HIP_PARAMS_H_
+#define PPLNN_LLM_HIP_PARAMS_H_
+
+#include "core.h"
+
+namespace ppl { namespace nn { namespace opmx {
+
+struct MultiHeadCacheAttentionParam final : public ir::Attr {
+    int32_t num_heads = 0;
+    int32_t num_kv_heads = 0;
+    int32_t head_dim = 0;
+    bool is_causal = true;
+    bool is_alibi = false;
+    int32_t num_layer = 0;
+    int32_t layer_idx = 0;
+    int32_t quant_bit = 0;
+    int32_t quant_group = 8;
+    int32_t cache_mode = 0;
+    int32_t cache_layout = 0;
+    int32_t page_size = 128;
+    bool operator==(const MultiHeadCacheAttentionParam& p) const {
+        return num_heads == p.num_heads && num_kv_heads == p.num_kv_heads && head_dim == p.head_dim &&
+            is_causal == p.is_causal && is_alibi == p.is_alibi && num_layer == p.num_layer && layer_idx == p.layer_idx &&
+            quant_bit == p.quant_bit && quant_group == p.quant_group && cache_mode == p.cache_mode &&
+            cache_layout == p.cache_layout && (cache_mode == 0 || page_size == p.page_size);
+    }
+};
+
+struct KeyValueCacheParam final : public ir::Attr {
+    int32_t num_layer = 0;
+    int32_t layer_idx = 0;
+    int32_t quant_bit = 0;
+    int32_t quant_group = 8;
+    int32_t num_repeat = 1;
+    int32_t cache_mode = 0;
+    int32_t cache_layout = 0;
+    int32_t page_size = 128;
+    bool operator==(const KeyValueCacheParam& p) const {
+        return num_layer == p.num_layer && layer_idx == p.layer_idx && quant_bit == p.quant_bit &&
+            quant_group == p.quant_group && num_repeat == p.num_repeat && cache_mode == p.cache_mode &&
+            cache_layout == p.cache_layout && (cache_mode == 0 || page_size == p.page_size);
+    }
+};
+
+}}} // namespace ppl::nn::opmx
+
+#endif

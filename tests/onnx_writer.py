@@ -1,0 +1,107 @@
+"""Minimal ONNX ModelProto writer (protobuf wire format by hand; no onnx / protobuf package needed).
+Field numbers follow onnx.proto: ModelProto{ir_version=1, graph=7, opset_import=8}, GraphProto{node=1, name=2,
+input=11, output=12}, NodeProto{input=1, output=2, name=3, op_type=4, attribute=5, domain=7},
+AttributeProto{name=1, f=2, i=3, type=20}, ValueInfoProto{name=1, type=2}."""
+import struct
+
+FLOAT, INT8, INT64, FLOAT16 = 1, 3, 7, 10
+
+
+def _varint(v):
+    v &= (1 << 64) - 1
+    out = bytearray()
+    while True:
+        b = v & 0x7F
+        v >>= 7
+        out.append(b | (0x80 if v else 0))
+        if not v:
+            return bytes(out)
+
+
+def _key(field, wt):
+    return _varint((field << 3) | wt)
+
+
+def _ld(field, payload):
+    return _key(field, 2) + _varint(len(payload)) + payload
+
+
+def _str(field, s):
+    return _ld(field, s.encode())
+
+
+def _int(field, v):
+    return _key(field, 0) + _varint(v)
+
+
+def attr_int(name, v):
+    return _str(1, name) + _int(3, v) + _int(20, 2)
+
+
+def attr_float(name, v):
+    return _str(1, name) + _key(2, 5) + struct.pack("<f", v) + _int(20, 1)
+
+
+def value_info(name, elem_type, dims):
+    """dims: ints, or strings for symbolic dimensions."""
+    shape = b"".join(_ld(1, _int(1, d) if isinstance(d, int) else _str(2, d)) for d in dims)
+    tensor = _int(1, elem_type) + _ld(2, shape)
+    return _str(1, name) + _ld(2, _ld(1, tensor))
+
+
+def node(op_type, inputs, outputs, name="", domain="", attrs=()):
+    b = b"".join(_str(1, i) for i in inputs) + b"".join(_str(2, o) for o in outputs)
+    if name:
+        b += _str(3, name)
+    b += _str(4, op_type) + b"".join(_ld(5, a) for a in attrs)
+    if domain:
+        b += _str(7, domain)
+    return b
+
+
+def model(nodes, inputs, outputs, opsets, graph_name="g"):
+    graph = b"".join(_ld(1, n) for n in nodes) + _str(2, graph_name) + b"".join(_ld(11, i) for i in inputs) + \
+        b"".join(_ld(12, o) for o in outputs)
+    m = _int(1, 8) + _ld(7, graph)
+    for domain, version in opsets:
+        m += _ld(8, (_str(1, domain) if domain else b"") + _int(2, version))
+    return m
+
+
+MHCA_INPUTS = ["query", "current_key", "current_value", "seqstarts", "kvstarts", "cachestarts", "start_pos",
+               "decoding_batches", "max_seqlen", "max_kvlen", "cache", "scale"]
+
+
+def mhca_model(num_heads, num_kv_heads, head_dim, num_layer, layer_idx, extra_attrs=(), drop_attrs=(), with_scale=True,
+               domain="opmx.dynamic_batching", opsets=None):
+    attrs = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, num_layer=num_layer,
+                 layer_idx=layer_idx, quant_bit=8, quant_group=8)
+    attrs.update(dict(extra_attrs))
+    for k in drop_attrs:
+        attrs.pop(k)
+    names = list(MHCA_INPUTS) if with_scale else MHCA_INPUTS[:-1]
+    n = node("MultiHeadCacheAttention", names, ["attn_output"], name="attn", domain=domain,
+             attrs=[attr_int(k, v) for k, v in attrs.items()])
+    types = {"query": FLOAT16, "current_key": FLOAT16, "current_value": FLOAT16, "cache": INT8, "scale": FLOAT16}
+    ranks = {"query": 3, "current_key": 3, "current_value": 3, "seqstarts": 1, "kvstarts": 1, "cachestarts": 1,
+             "start_pos": 1, "decoding_batches": 0, "max_seqlen": 0, "max_kvlen": 0, "cache": 5, "scale": 5}
+    ins = [value_info(x, types.get(x, INT64), ["d%d" % i for i in range(ranks[x])]) for x in names]
+    outs = [value_info("attn_output", FLOAT16, ["s", "h", "d"])]
+    return model([n], ins, outs, opsets if opsets is not None else [("", 11), (domain, 1)])
+
+
+KVC_INPUTS = ["current_key", "current_value", "seqstarts", "kvstarts", "cachestarts", "start_pos", "max_seqlen",
+              "max_kvlen", "cache", "scale"]
+
+
+def kv_cache_model(num_layer, layer_idx, extra_attrs=()):
+    attrs = dict(num_layer=num_layer, layer_idx=layer_idx, quant_bit=8, quant_group=8)
+    attrs.update(dict(extra_attrs))
+    n = node("KeyValueCache", KVC_INPUTS, ["key", "value"], name="kvcache", domain="opmx.dynamic_batching",
+             attrs=[attr_int(k, v) for k, v in attrs.items()])
+    types = {"current_key": FLOAT16, "current_value": FLOAT16, "cache": INT8, "scale": FLOAT16}
+    ranks = {"current_key": 3, "current_value": 3, "seqstarts": 1, "kvstarts": 1, "cachestarts": 1, "start_pos": 1,
+             "max_seqlen": 0, "max_kvlen": 0, "cache": 5, "scale": 5}
+    ins = [value_info(x, types.get(x, INT64), ["d%d" % i for i in range(ranks[x])]) for x in KVC_INPUTS]
+    outs = [value_info("key", FLOAT16, ["t", "h", "d"]), value_info("value", FLOAT16, ["t", "h", "d"])]
+    return model([n], ins, outs, [("", 11), ("opmx.dynamic_batching", 1)])

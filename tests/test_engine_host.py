@@ -1,0 +1,126 @@
+"""CPU-side tests of the llm_hip host engine (no GPU): registry, arena, ONNX wire reader and attribute parsers,
+engine configuration and the error conventions of the reference."""
+import ctypes as C
+import os
+
+import pytest
+
+import harness
+import onnx_writer as ow
+from harness import cabi
+
+
+@pytest.fixture(scope="module")
+def eng():
+    L = harness.pkg.load_engine_library()
+    L.pplnn_hip_set_log_level(4)  # silence expected error logs
+    return L
+
+
+def test_registry_overlapping_versions_give_rc_exists(eng):
+    # src/ppl/nn/utils/op_info_manager.h:49-71
+    assert eng.pplnn_hip_selftest_registry() == cabi.RC_EXISTS
+
+
+def test_arena_known_answers_of_the_reference_buffer_manager_tests(eng):
+    # tests/utils/stack_buffer_manager_test.cc:24-38: Realloc(1243) -> non-null address, buffered bytes >= 1243
+    a = eng.pplnn_hip_arena_create_host(64, 1 << 20)
+    addr, desc = C.c_void_p(), C.c_uint64()
+    assert eng.pplnn_hip_arena_alloc(a, 1243, C.byref(addr), C.byref(desc)) == 0
+    assert addr.value and desc.value >= 1243 and eng.pplnn_hip_arena_buffered_bytes(a) >= 1243
+    eng.pplnn_hip_arena_destroy(a)
+    # tests/utils/compact_buffer_manager_test.cc:43-58: Realloc(1000) with 128-byte alignment and 1024-byte blocks
+    # -> aligned address, desc >= 1000, buffered bytes == one 1024-byte block
+    a = eng.pplnn_hip_arena_create_host(128, 1024)
+    assert eng.pplnn_hip_arena_alloc(a, 1000, C.byref(addr), C.byref(desc)) == 0
+    assert desc.value >= 1000 and eng.pplnn_hip_arena_buffered_bytes(a) == 1024
+    first = addr.value
+    # free + realloc reuses the block instead of growing; neighbours coalesce
+    eng.pplnn_hip_arena_free(a, addr)
+    assert eng.pplnn_hip_arena_used_bytes(a) == 0
+    assert eng.pplnn_hip_arena_alloc(a, 512, C.byref(addr), C.byref(desc)) == 0 and addr.value == first
+    b2, d2 = C.c_void_p(), C.c_uint64()
+    assert eng.pplnn_hip_arena_alloc(a, 512, C.byref(b2), C.byref(d2)) == 0 and b2.value == first + 512
+    assert eng.pplnn_hip_arena_buffered_bytes(a) == 1024
+    eng.pplnn_hip_arena_free(a, addr)
+    eng.pplnn_hip_arena_free(a, b2)
+    assert eng.pplnn_hip_arena_alloc(a, 1024, C.byref(addr), C.byref(desc)) == 0 and addr.value == first
+    assert eng.pplnn_hip_arena_buffered_bytes(a) == 1024
+    eng.pplnn_hip_arena_destroy(a)
+
+
+def _load(eng, buf):
+    b = eng.pplnn_hip_builder_create()
+    rc = eng.pplnn_hip_builder_load_model(b, buf, len(buf))
+    return b, rc
+
+
+def test_reference_conv_onnx_parses(eng):
+    # tests/models/onnx/onnx_model_parser_test.cc:28-35 expects RC_SUCCESS for this file
+    with open(os.path.join(harness.ROOT, "tests", "golden", "conv.onnx"), "rb") as f:
+        buf = f.read()
+    assert len(buf) == 456
+    b, rc = _load(eng, buf)
+    assert rc == cabi.RC_SUCCESS
+    # no engine here supports ONNX Conv: partitioning must say so
+    e = eng.pplnn_hip_engine_create(0, 1)
+    assert eng.pplnn_hip_builder_set_engine(b, e) == 0
+    assert eng.pplnn_hip_builder_preprocess(b) == cabi.RC_UNSUPPORTED
+    eng.pplnn_hip_builder_destroy(b)
+    eng.pplnn_hip_engine_destroy(e)
+
+
+def test_mhca_graph_loads_and_preprocesses(eng):
+    e = eng.pplnn_hip_engine_create(0, 1)
+    assert e and eng.pplnn_hip_engine_name(e) == b"llm_hip"
+    b, rc = _load(eng, ow.mhca_model(32, 8, 128, 2, 1))
+    assert rc == 0
+    assert eng.pplnn_hip_builder_set_engine(b, e) == 0
+    assert eng.pplnn_hip_builder_preprocess(b) == 0
+    eng.pplnn_hip_builder_destroy(b)
+    eng.pplnn_hip_engine_destroy(e)
+
+
+@pytest.mark.parametrize("missing", ["num_heads", "head_dim", "num_layer", "layer_idx"])
+def test_mhca_required_attrs(eng, missing):
+    # parse_multi_head_cache_attention_param.cc:16-34 -> RC_INVALID_VALUE
+    b, rc = _load(eng, ow.mhca_model(32, 8, 128, 2, 1, drop_attrs=[missing]))
+    assert rc == cabi.RC_INVALID_VALUE and missing.encode() in eng.pplnn_hip_last_error()
+    eng.pplnn_hip_builder_destroy(b)
+
+
+def test_unimported_domain_and_garbage(eng):
+    b, rc = _load(eng, ow.mhca_model(32, 8, 128, 1, 0, opsets=[("", 11)]))  # graph_parser.cc:166-172
+    assert rc == cabi.RC_NOT_FOUND
+    eng.pplnn_hip_builder_destroy(b)
+    b, rc = _load(eng, b"\xff\xff\xff\xff\x07garbage")
+    assert rc == cabi.RC_INVALID_VALUE
+    eng.pplnn_hip_builder_destroy(b)
+    b = eng.pplnn_hip_builder_create()
+    assert eng.pplnn_hip_builder_preprocess(b) == cabi.RC_INVALID_VALUE  # nothing loaded
+    assert eng.pplnn_hip_builder_load_model_file(b, b"/nonexistent/model.onnx") == cabi.RC_NOT_FOUND
+    eng.pplnn_hip_builder_destroy(b)
+
+
+def test_wrong_version_is_not_supported(eng):
+    e = eng.pplnn_hip_engine_create(0, 1)
+    b, rc = _load(eng, ow.mhca_model(32, 8, 128, 1, 0, opsets=[("", 11), ("opmx.dynamic_batching", 2)]))
+    assert rc == 0  # no parser for version 2: attributes are simply not parsed
+    assert eng.pplnn_hip_builder_set_engine(b, e) == 0
+    assert eng.pplnn_hip_builder_preprocess(b) == cabi.RC_UNSUPPORTED  # registered for versions [1, 1] only
+    eng.pplnn_hip_builder_destroy(b)
+    eng.pplnn_hip_engine_destroy(e)
+
+
+def test_engine_configure_like_the_reference(eng):
+    e = eng.pplnn_hip_engine_create(0, 1)
+    ok = [(1, 0), (2, 1), (1000, 0), (1001, 1), (1002, 1), (1003, 0), (1003, 2), (1004, 256), (1004, 512), (1005, 1)]
+    for opt, val in ok:
+        assert eng.pplnn_hip_engine_configure_u32(e, opt, val) == 0, (opt, val)
+    assert eng.pplnn_hip_engine_configure_u32(e, 1003, 3) == cabi.RC_INVALID_VALUE  # engine.cc:150-170
+    assert eng.pplnn_hip_engine_configure_u32(e, 1004, 128) == cabi.RC_INVALID_VALUE
+    assert eng.pplnn_hip_engine_configure_u32(e, 0, 0) == cabi.RC_UNSUPPORTED  # NCCL comm: one GPU only
+    assert eng.pplnn_hip_engine_configure_u32(e, 77, 0) == cabi.RC_INVALID_VALUE
+    assert eng.pplnn_hip_engine_configure_u32(e, 1006, 0) == cabi.RC_INVALID_VALUE
+    eng.pplnn_hip_engine_destroy(e)
+    assert not eng.pplnn_hip_engine_create(0, 99)  # unknown mm_policy: factories return nullptr on failure

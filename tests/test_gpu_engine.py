@@ -1,0 +1,189 @@
+"""End to end through the llm_hip host engine on the GPU: an ONNX graph with one OPMX node is loaded by the wire reader,
+partitioned to the engine, and run by the sequential runtime; results must equal the oracle's (same bar as the C ABI)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness
+import onnx_writer as ow
+from harness import cabi, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _i64(*dims):
+    return (C.c_int64 * len(dims))(*dims), len(dims)
+
+
+class Session:
+    def __init__(self, eng, model_bytes, configure=()):
+        self.eng = eng
+        self.engine = eng.pplnn_hip_engine_create(0, 1)
+        assert self.engine
+        for opt, val in configure:
+            assert eng.pplnn_hip_engine_configure_u32(self.engine, opt, val) == 0
+        self.builder = eng.pplnn_hip_builder_create()
+        assert eng.pplnn_hip_builder_load_model(self.builder, model_bytes, len(model_bytes)) == 0
+        assert eng.pplnn_hip_builder_set_engine(self.builder, self.engine) == 0
+        assert eng.pplnn_hip_builder_preprocess(self.builder) == 0, eng.pplnn_hip_last_error()
+        self.rt = eng.pplnn_hip_builder_create_runtime(self.builder)
+        assert self.rt, eng.pplnn_hip_last_error()
+        self.keep = []
+
+    def input(self, i):
+        return self.eng.pplnn_hip_runtime_input(self.rt, i)
+
+    def set_device_tensor(self, i, t):  # borrowed device memory, like the caller-owned KV slab
+        tensor = self.input(i)
+        dims, n = _i64(*t.shape)
+        self.eng.pplnn_hip_tensor_reshape(tensor, dims, n)
+        self.eng.pplnn_hip_tensor_set_buffer_ptr(tensor, t.data_ptr())
+        self.keep.append(t)
+
+    def set_table(self, i, a):  # copied into an arena buffer of the engine's device
+        tensor = self.input(i)
+        dims, n = _i64(*a.shape)
+        self.eng.pplnn_hip_tensor_reshape(tensor, dims, n)
+        a = np.ascontiguousarray(a)
+        assert self.eng.pplnn_hip_tensor_copy_from_host(tensor, a.ctypes.data) == 0
+        self.keep.append(a)
+
+    def set_host_scalar(self, i, v):  # decoding_batches / max_seqlen / max_kvlen live on the host device
+        tensor = self.input(i)
+        self.eng.pplnn_hip_tensor_use_host_device(tensor)
+        self.eng.pplnn_hip_tensor_reshape(tensor, None, 0)
+        a = np.array([v], np.int64)
+        assert self.eng.pplnn_hip_tensor_copy_from_host(tensor, a.ctypes.data) == 0
+
+    def output(self, i, dtype):
+        tensor = self.eng.pplnn_hip_runtime_output(self.rt, i)
+        dims = (C.c_int64 * 8)()
+        n = self.eng.pplnn_hip_tensor_dims(tensor, dims, 8)
+        out = np.empty(tuple(dims[:n]), dtype)
+        assert self.eng.pplnn_hip_tensor_copy_to_host(tensor, out.ctypes.data) == 0
+        return out
+
+    def close(self):
+        self.eng.pplnn_hip_runtime_destroy(self.rt)
+        self.eng.pplnn_hip_builder_destroy(self.builder)
+        self.eng.pplnn_hip_engine_destroy(self.engine)
+
+
+def _prepare_slab(b, t, hiplib):
+    """History written through the C ABI into torch-owned slab memory (the caller owns the slab)."""
+    import torch
+    cache_h, scale_h = harness.new_slab(b)
+    cache, scale = harness.to_dev(cache_h), harness.to_dev(scale_h)
+    if b.total_hist_tokens:
+        hk, hv = harness.to_dev(t["hist_key"]), harness.to_dev(t["hist_value"])
+        hs, z, cs = harness.to_dev(b.histstarts), harness.to_dev(np.zeros(b.batch, np.int64)), harness.to_dev(b.cachestarts)
+        w = harness.fill_write_args(cabi.KvWriteArgs(), b, hk, hv, hs, z, cs, cache, scale, ptr=harness.dev_ptr)
+        harness.pkg.check(hiplib.pplhip_kv_quantize_write(C.byref(w), None), "history")
+        torch.cuda.synchronize()
+    return cache, scale
+
+
+@pytest.mark.parametrize("cache_prefill", [0, 1])
+def test_mhca_graph_through_the_engine(hiplib, cache_prefill):
+    import torch
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(32, 8, 128, [1, 1, 1, 1, 70, 200], [500, 3, 77, 1300, 0, 0], 4, num_layer=2, layer_idx=1,
+                        name="engine_mhca")
+    t = workloads.make_tensors(b, seed=77)
+    ref = harness.run_oracle(b, t, cache_prefill=cache_prefill)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    s = Session(eng, ow.mhca_model(32, 8, 128, 2, 1), configure=[(1005, cache_prefill)])
+    assert eng.pplnn_hip_runtime_input_count(s.rt) == 12 and eng.pplnn_hip_runtime_output_count(s.rt) == 1
+    assert eng.pplnn_hip_runtime_set_profiling(s.rt, 1) == 0
+    s.set_device_tensor(0, harness.to_dev(t["query"]))
+    s.set_device_tensor(1, harness.to_dev(t["current_key"]))
+    s.set_device_tensor(2, harness.to_dev(t["current_value"]))
+    s.set_table(3, b.seqstarts)
+    s.set_table(4, b.kvstarts)
+    s.set_table(5, b.cachestarts)
+    s.set_table(6, b.start_pos)
+    s.set_host_scalar(7, b.decoding_batches)
+    s.set_host_scalar(8, b.max_seqlen)
+    s.set_host_scalar(9, b.max_kvlen)
+    s.set_device_tensor(10, cache)
+    s.set_device_tensor(11, scale)
+    for _ in range(2):  # the second run reuses arena buffers and must give the same answer
+        assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+        out = s.output(0, np.float16)
+        assert out.shape == (b.total_new_tokens, 32, 128)
+        harness.assert_attn_close(out, ref["output_f64"])
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), ref["cache"])
+    assert np.array_equal(scale.cpu().view(torch.int16).numpy().view(np.uint16), ref["scale"].view(np.uint16))
+    micros, counts = (C.c_uint64 * 4)(), (C.c_uint32 * 4)()
+    assert eng.pplnn_hip_runtime_profiling(s.rt, micros, counts, 4) == 1
+    assert counts[0] == 2 and micros[0] > 0
+    s.close()
+
+
+def test_engine_error_paths_on_device(hiplib):
+    eng = harness.pkg.load_engine_library()
+    eng.pplnn_hip_set_log_level(4)
+    b = workloads.Batch(8, 2, 128, [1, 5], [10, 0], 1)
+    t = workloads.make_tensors(b, seed=5)
+    cache, scale = _prepare_slab(b, t, hiplib)
+
+    def run(model, skip=()):
+        s = Session(eng, model)
+        tensors = [harness.to_dev(t["query"]), harness.to_dev(t["current_key"]), harness.to_dev(t["current_value"])]
+        for i in range(3):
+            s.set_device_tensor(i, tensors[i])
+        for i, a in zip(range(3, 7), (b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)):
+            s.set_table(i, a)
+        for i, v in zip(range(7, 10), (b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+            s.set_host_scalar(i, v)
+        s.set_device_tensor(10, cache)
+        if 11 not in skip and eng.pplnn_hip_runtime_input_count(s.rt) > 11:
+            s.set_device_tensor(11, scale)
+        rc = eng.pplnn_hip_runtime_run(s.rt)
+        s.close()
+        return rc
+
+    assert run(ow.mhca_model(8, 2, 128, 1, 0)) == 0
+    assert run(ow.mhca_model(8, 2, 128, 1, 0, extra_attrs={"is_alibi": 1})) == cabi.RC_UNSUPPORTED  # …_kernel.cc:95-98
+    assert run(ow.mhca_model(8, 2, 128, 1, 0, with_scale=False)) == cabi.RC_UNSUPPORTED  # …_kernel.cc:100-103
+    assert run(ow.mhca_model(8, 2, 128, 1, 0, extra_attrs={"cache_layout": 2})) == cabi.RC_UNSUPPORTED  # :156-159
+    assert run(ow.mhca_model(8, 2, 128, 1, 0, extra_attrs={"cache_mode": 1})) == cabi.RC_INVALID_VALUE  # :163-166
+    assert run(ow.mhca_model(8, 2, 128, 1, 0, extra_attrs={"quant_bit": 4, "quant_group": 4})) == cabi.RC_UNSUPPORTED
+
+
+def test_kv_cache_graph_through_the_engine(hiplib, olib):
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(4, 4, 128, [1, 6, 1, 40], [9, 0, 3, 0], 0, num_layer=2, layer_idx=1)
+    t = workloads.make_tensors(b, seed=9)
+    # oracle
+    cache_o, scale_o = harness.new_slab(b)
+    zeros = np.zeros(b.batch, np.int64)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, t["hist_key"], t["hist_value"], b.histstarts, zeros, b.cachestarts,
+                                cache_o, scale_o)
+    assert olib.oracle_kv_quantize_write(C.byref(w)) == 0
+    a = cabi.KvCacheArgs()
+    ss, ks = b.seqstarts, b.kvstarts
+    harness.fill_write_args(a.write, b, t["current_key"], t["current_value"], ss, b.start_pos, b.cachestarts, cache_o, scale_o)
+    a.d_kvstarts, a.total_kv_tokens, a.max_kvlen = ks.ctypes.data, int(ks[-1]), b.max_kvlen
+    a.num_repeat = 1
+    ko, vo = np.zeros((int(ks[-1]), 4, 128), np.float16), np.zeros((int(ks[-1]), 4, 128), np.float16)
+    a.d_key_out, a.d_value_out = ko.ctypes.data, vo.ctypes.data
+    assert olib.oracle_kv_cache_forward(C.byref(a)) == 0
+    # engine
+    cache, scale = _prepare_slab(b, t, hiplib)
+    s = Session(eng, ow.kv_cache_model(2, 1))
+    s.set_device_tensor(0, harness.to_dev(t["current_key"]))
+    s.set_device_tensor(1, harness.to_dev(t["current_value"]))
+    for i, tab in zip(range(2, 6), (b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)):
+        s.set_table(i, tab)
+    s.set_host_scalar(6, b.max_seqlen)
+    s.set_host_scalar(7, b.max_kvlen)
+    s.set_device_tensor(8, cache)
+    s.set_device_tensor(9, scale)
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    key, value = s.output(0, np.float16), s.output(1, np.float16)
+    assert key.shape == ko.shape  # dim 0 = kvstarts[B], read back like reshape_dynamic_batching_key_value_cache.cc:43-53
+    assert np.array_equal(key.view(np.uint16), ko.view(np.uint16)) and np.array_equal(value.view(np.uint16), vo.view(np.uint16))
+    s.close()
