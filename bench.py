@@ -35,6 +35,7 @@ def parse():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--split-k", type=int, default=1)
+    ap.add_argument("--no-churn", action="store_true", help="skip the cfg4 continuous-batching churn run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy (the reference point for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this same command)")
@@ -192,6 +193,107 @@ def copy_calibration():
     torch.cuda.synchronize()
 
 
+def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
+    """Continuous-batching churn (Llama-2-13B shape, H = KVH = 40): 256 slots, every step the tables are rebuilt on
+    the GPU by pplhip_pack_tables from the slot state, one mixed MultiHeadCacheAttention call runs on them, and
+    pplhip_advance_slots grows the slots. The host only supplies the sizes its scheduler knows anyway (batch,
+    decoding_batches, maxima), precomputed for the seeded schedule; no table is uploaded and nothing is read back."""
+    import torch
+    from ppl_nn_amd import cabi, workloads
+    sch = workloads.ChurnSchedule(seed=2)
+    n, H, KVH, Dh = sch.num_slots, sch.num_heads, sch.num_kv_heads, sch.head_dim
+    dev = "cuda"
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    max_tokens = n * sch.region
+    cache = torch.zeros((max_tokens, 1, 2, KVH, Dh), dtype=torch.int8, device=dev)
+    scale = torch.zeros((max_tokens, 1, 2, KVH, Dh // 8), dtype=torch.float16, device=dev)
+    plans, host = [], []
+    for _ in range(steps + warm_steps):
+        kv, nl = sch.next_step()
+        is_dec = (nl == 1) & (kv > 0)
+        host.append(dict(kv=kv, nl=nl, nd=int(is_dec.sum()), batch=int((nl > 0).sum()), S=int(nl.sum()),
+                         max_seqlen=int(nl.max()), max_kvlen=int((kv + nl).max()),
+                         dec_kv=int((kv + nl)[is_dec].sum()),
+                         prefill_flops=int(sum(4 * H * Dh * (int(l) * (int(l) + 1) // 2) for l in nl[~is_dec & (nl > 0)]))))
+    max_S = max(h["S"] for h in host)
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    q = torch.randn((max_S, H, Dh), generator=g, dtype=torch.float16, device=dev)
+    k = torch.randn((max_S, KVH, Dh), generator=g, dtype=torch.float16, device=dev)
+    v = torch.randn((max_S, KVH, Dh), generator=g, dtype=torch.float16, device=dev)
+    out = torch.zeros((max_S, H, Dh), dtype=torch.float16, device=dev)
+    i64 = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(dev)
+    slot_kv = i64(np.zeros(n))
+    slot_cs = i64(sch.cachestart)
+    # per-step new-token counts are the scheduler's decision: staged on the device before the timed loop
+    slot_nl = [i64(h["nl"]) for h in host]
+    slot_kv_reset = [i64(h["kv"]) for h in host]  # retirements reset a slot to 0 (the scheduler's decision too)
+    seqstarts = torch.zeros(n + 1, dtype=torch.int64, device=dev)
+    kvstarts = torch.zeros(n + 1, dtype=torch.int64, device=dev)
+    cachestarts = torch.zeros(n, dtype=torch.int64, device=dev)
+    start_pos = torch.zeros(n, dtype=torch.int64, device=dev)
+    batch_slots = torch.zeros(n, dtype=torch.int64, device=dev)
+    header = torch.zeros(6, dtype=torch.int64, device=dev)
+    st = cabi.cache_strides_layout0(1, KVH, Dh)
+    calls = []
+    ws_bytes = 256
+    for i, h in enumerate(host):
+        pa = cabi.PackArgs()
+        pa.d_slot_kvlen, pa.d_slot_newlen, pa.d_slot_cachestart = ptr(slot_kv), ptr(slot_nl[i]), ptr(slot_cs)
+        pa.num_slots = n
+        pa.d_seqstarts, pa.d_kvstarts, pa.d_cachestarts = ptr(seqstarts), ptr(kvstarts), ptr(cachestarts)
+        pa.d_start_pos, pa.d_batch_slots, pa.d_header = ptr(start_pos), ptr(batch_slots), ptr(header)
+        a = cabi.MhcaArgs()
+        a.d_query, a.d_current_key, a.d_current_value = ptr(q), ptr(k), ptr(v)
+        a.d_seqstarts, a.d_kvstarts, a.d_cachestarts, a.d_start_pos = ptr(seqstarts), ptr(kvstarts), ptr(cachestarts), ptr(start_pos)
+        a.is_causal, a.batch, a.decoding_batches = 1, h["batch"], h["nd"]
+        a.max_seqlen, a.max_kvlen = h["max_seqlen"], h["max_kvlen"]
+        a.layer_idx, a.num_layer, a.num_heads, a.num_kv_heads, a.head_dim = 0, 1, H, KVH, Dh
+        a.cache_mode, a.page_size = 0, 128
+        for kk, vv in st.items():
+            setattr(a, kk, vv)
+        a.specify_decoding_attn_split_k = 1
+        a.d_cache, a.d_scale, a.d_output = ptr(cache), ptr(scale), ptr(out)
+        a.total_new_tokens = h["S"]
+        plan = cabi.MhcaPlan()
+        pkg.check(lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)), "prepare(churn)")
+        ws_bytes = max(ws_bytes, int(plan.workspace_bytes))
+        calls.append((pa, a, plan))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    def step(i):
+        pa, a, plan = calls[i]
+        slot_kv.copy_(slot_kv_reset[i])  # device-to-device: applies the scheduler's retirements
+        rc = lib.pplhip_pack_tables(C.byref(pa), stream)
+        rc = rc or lib.pplhip_mhca_forward(C.byref(a), C.byref(plan), ptr(ws), stream)
+        rc = rc or lib.pplhip_advance_slots(ptr(slot_kv), ptr(slot_nl[i]), n, stream)
+        if rc:
+            pkg.check(rc, "churn step")
+
+    for i in range(warm_steps):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(warm_steps, warm_steps + steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    timed = host[warm_steps:]
+    dec_tokens = sum(h["nd"] for h in timed)
+    dec_bytes = sum(h["dec_kv"] for h in timed) * 2.5 * KVH * Dh
+    flops = sum(h["prefill_flops"] for h in timed)
+    # check the on-device state against the host mirror once, after the timed region
+    assert np.array_equal(slot_kv.cpu().numpy(), host[-1]["kv"] + host[-1]["nl"]), "slot state diverged"
+    return {"workload": "cfg4 churn: 256 slots x %d steps, H=KVH=40, Dh 128, retire p=0.02, prompts U[32,512], tables "
+                        "rebuilt on the GPU every step" % steps,
+            "ms_per_step": ms, "decode_tokens_per_s": dec_tokens / (ms * steps * 1e-3),
+            "decode_kv_GB_per_step": dec_bytes / steps / 1e9, "prefill_GFLOP_per_step": flops / steps / 1e9,
+            "decode_GBps_if_step_were_decode_only": dec_bytes / (ms * steps * 1e-3) / 1e9}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -259,6 +361,10 @@ def main():
         _, mix_ms = timed(mixed, max(args.steps // 2, 10), max(args.warmup // 2, 3))
         result["fused_mixed_call_ms"] = mix_ms
         del mixed
+    if args.workload == "cfg2" and not args.no_churn:
+        del dec.slabs[1:], dec.args[1:]
+        torch.cuda.empty_cache()
+        result["churn_cfg4"] = churn_cfg4(pkg, lib)
     if args.copy_calibration:
         copy_calibration()
     if not args.no_cpu_baseline:

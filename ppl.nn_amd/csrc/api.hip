@@ -133,12 +133,12 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     // ---- decode: the kernel cuts the decode sequences' cached tokens, laid end to end, into S equal ranges on the
     // device; the host only picks S from the chip size. One workgroup (4 waves) per range and group of <= 4 kv heads,
     // two resident workgroups per CU.
-    plan->decode_waves_per_block = 4;
+    plan->decode_waves_per_block = decode_waves_per_block();
     const int64_t nd = a->decoding_batches;
     if (nd > 0) {
         const int hpb = decode_heads_per_block(a->num_kv_heads);
         const int64_t groups = a->num_kv_heads / hpb;
-        const int64_t slots = (int64_t)device_cu_count() * 2;
+        const int64_t slots = (int64_t)device_cu_count() * decode_blocks_per_cu();
         // halves of a slot: every workgroup streams the same number of bytes, so one workgroup per slot (a single,
         // perfectly filled round) measures best; the knob moves it to half or twice that
         int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;

@@ -66,6 +66,8 @@ inline int ceil_div(int64_t a, int64_t b) {
 pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream);
 pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream_t stream);
 int decode_heads_per_block(int kv_heads);
+int decode_blocks_per_cu();
+int decode_waves_per_block();
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
 pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, hipStream_t stream);
 pplhip_retcode launch_pack_tables(const pplhip_pack_args* a, hipStream_t stream);

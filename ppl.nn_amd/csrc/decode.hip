@@ -43,7 +43,10 @@
 namespace pplhip {
 
 constexpr int kDh = 128; // head_dim this kernel is specialised for
-constexpr int kDecodeWaves = 4;
+#ifndef PPLHIP_DECODE_WAVES
+#define PPLHIP_DECODE_WAVES 4
+#endif
+constexpr int kDecodeWaves = PPLHIP_DECODE_WAVES; // waves per workgroup; each owns a 20 KiB double-buffered LDS region
 constexpr int kStageTokens = 32; // tokens per pipeline stage (2 MFMA sub-blocks of 16)
 constexpr int kSubBlocks = kStageTokens / 16;
 // LDS bytes of one stage of one wave, and where its four arrays start
@@ -460,6 +463,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                     PPLHIP_WAIT_VMCNT(0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+#ifdef PPLHIP_X_NOCOMPUTE
+                if (it == 0)
+#endif
                 compute_stage(wave_lds_addr + (it & 1) * kStageBytes, ro, ss, qB, kq,
                               it + 1 == n_stages ? tail_rows_valid : kStageTokens, p.score_scale);
                 __builtin_amdgcn_sched_barrier(0);
@@ -561,6 +567,14 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
         }
         p.out[(p.seqstarts[b] * p.num_heads + head) * kDh + d] = (half_t)(a / L);
     }
+}
+
+int decode_blocks_per_cu() {
+    return (160 * 1024) / kDecodeLdsBytes; // LDS-limited
+}
+
+int decode_waves_per_block() {
+    return kDecodeWaves;
 }
 
 int decode_heads_per_block(int kv_heads) {
