@@ -463,9 +463,6 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                     PPLHIP_WAIT_VMCNT(0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-#ifdef PPLHIP_X_NOCOMPUTE
-                if (it == 0)
-#endif
                 compute_stage(wave_lds_addr + (it & 1) * kStageBytes, ro, ss, qB, kq,
                               it + 1 == n_stages ? tail_rows_valid : kStageTokens, p.score_scale);
                 __builtin_amdgcn_sched_barrier(0);

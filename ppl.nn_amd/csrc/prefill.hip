@@ -1,18 +1,24 @@
 // Causal prefill attention over ragged packed sequences (flash-attention style, fp16 MFMA, fp32 online softmax).
 //
 // Roofline: fp16 MFMA. One workgroup (4 wavefronts) owns 128 query rows of one (sequence, query head); each wave
-// owns 32 of them. K/V tiles of 64 tokens are staged in LDS once per workgroup and shared by the 4 waves, with the
-// next tile's global loads in flight (held in registers) while the current tile is computed; grouped query heads map
-// to their kv head by integer division. Everything is computed transposed so that probabilities never leave registers:
+// owns 32 of them. K/V tiles of 64 tokens are staged in LDS once per workgroup and shared by the 4 waves (two buffers,
+// one barrier per tile), with the next tile's global loads in flight (held in registers) while the current tile is
+// computed; grouped query heads map to their kv head by integer division. Everything is computed transposed so that
+// probabilities never leave registers:
 //   S^T = K * Q^T    v_mfma_f32_32x32x16_f16, A = K tile from LDS (16 B per lane per MFMA), B = Q^T held in registers
 //                    -> lane (n = lane & 31, hb = lane >> 5) owns query row n and kv tokens {8*(r/4) + 4*hb + r%4}
-//   O^T += V^T * P^T A = V^T: a lane reads 8 tokens x 4 channels from LDS (row-major, conflict-free) and transposes
-//                    them in registers with v_perm; B = P^T is exactly the layout the score registers already have.
+//   O^T += V^T * P^T A = V^T from LDS: the tile is transposed ONCE per workgroup on its way into LDS (4 tokens x 8
+//                    channels per thread, v_perm), laid out [channel][token position] with the positions permuted so
+//                    that the 8 tokens a lane owns in P^T are one 16-byte read; B = P^T is exactly the layout the score
+//                    registers already have.
 // Softmax statistics are per lane column, so rescaling O^T needs no cross-lane traffic; one shuffle per tile
-// combines the two half-waves' maxima. Tiles entirely above the causal diagonal are skipped. Workgroups are numbered
-// heaviest query tile first across ALL sequences and heads (longest-processing-time order, which keeps the tail of
-// the launch short for causal work), and the query heads of one kv head are spaced 8 apart so that they run on the
-// same XCD and share its L2 copy of the K/V rows. The output tile goes through LDS so that global stores are full rows.
+// combines the two half-waves' maxima. The reference maximum of a row is only moved when the running maximum has
+// outgrown it by more than 2^kRescaleLog2 (probabilities then stay below that factor, well inside fp16), which
+// removes the accumulator rescale from almost every tile. Tiles entirely above the causal diagonal are skipped.
+// Workgroups are numbered heaviest query tile first across ALL sequences and heads (longest-processing-time order,
+// which keeps the tail of the launch short for causal work), and the query heads of one kv head are spaced 8 apart so
+// that they run on the same XCD and share its L2 copy of the K/V rows. The output tile goes through LDS so that global
+// stores are full rows.
 //
 // K/V source: the fp16 current_key/current_value of the sequence (default), or the int8 slab dequantised on the way
 // into LDS (cache-prefill: supports start_pos > 0, i.e. chunked prefill / prompt cache).
@@ -23,8 +29,13 @@ namespace pplhip {
 constexpr int kPDh = 128;
 constexpr int kBM = 128; // query rows per workgroup
 constexpr int kBN = 64; // kv tokens per tile
-constexpr int kLdsRow = kPDh * 2 + 16; // bytes per LDS row: 256 B of fp16 + 16 B pad -> 16-byte reads of 8 consecutive
-                                       // rows hit distinct banks
+constexpr int kLdsRow = kPDh * 2 + 16; // bytes per K row in LDS: 256 B of fp16 + 16 B pad -> 16-byte reads of 16
+                                       // consecutive rows hit distinct banks
+constexpr int kVtRow = kBN * 2 + 16; // bytes per V^T row (one channel, 64 token positions) + 16 B pad
+constexpr int kLdsKBytes = kBN * kLdsRow; // 17408
+constexpr int kLdsVBytes = kPDh * kVtRow; // 18432
+constexpr int kLdsBufBytes = kLdsKBytes + kLdsVBytes; // one K/V tile
+constexpr float kRescaleLog2 = 8.0f;
 
 struct PrefillParams {
     const half_t* q;
@@ -45,89 +56,200 @@ struct PrefillParams {
     float score_scale; // log2(e) / sqrt(Dh)
 };
 
-// One thread's share of a 64-token K/V tile on its way from global memory to LDS.
+// A thread's share of a 64-token K/V tile: channels 8*col .. 8*col+7 (col = tid & 15) of the four consecutive tokens
+// 4*r0 .. 4*r0+3 (r0 = tid >> 4). A wave's load instruction covers four full 256-byte rows.
 template <bool FROM_CACHE>
 struct TileRegs;
 
 template <>
-struct TileRegs<false> { // fp16 source: 4 rows x 16 B of K and of V per thread
+struct TileRegs<false> { // fp16 source
     uint4 k[4], v[4];
 };
 template <>
-struct TileRegs<true> { // int8 slab: 32 channels (+4 scales) of one row of K and of V per thread
-    uint4 q[2][2];
-    uint2 s[2];
+struct TileRegs<true> { // int8 slab: 8 bytes + one fp16 scale per token for K and for V (8 channels = one quant group)
+    uint2 kq[4], vq[4];
+    uint16_t ks[4], vs[4];
 };
 
-__device__ inline void fetch_tile(TileRegs<false>& t, const PrefillParams& p, int64_t j0, int64_t kvlen, int64_t s0,
-                                  int64_t, int kvh) {
-    const int tid = threadIdx.x, col = tid & 15;
-#pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const int64_t j = j0 + (tid >> 4) + 16 * pass;
-        t.k[pass] = t.v[pass] = make_uint4(0, 0, 0, 0);
-        if (j < kvlen) {
-            const int64_t off = ((s0 + j) * p.kv_heads + kvh) * kPDh + col * 8;
-            t.k[pass] = *reinterpret_cast<const uint4*>(p.k + off);
-            t.v[pass] = *reinterpret_cast<const uint4*>(p.v + off);
-        }
-    }
+// Pins a pointer that is wave-uniform by construction into scalar registers, so that memory instructions take the
+// "scalar base + 32-bit lane offset" addressing form.
+__device__ inline const char* uniform_ptr(const char* p) {
+    const uint64_t u = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
 }
-__device__ inline void store_tile(const TileRegs<false>& t, char* lds_k, char* lds_v) {
-    const int tid = threadIdx.x, col = tid & 15;
+
+// Where a workgroup's K/V rows come from. Token j of the sequence is at (uniform base) + j * row_bytes, and a
+// thread's piece of the row it fetches in pass p of tile j0 is at base + (j0 + p) * row_bytes + voff, voff fixed for
+// the whole kernel: all per-tile address arithmetic is scalar.
+template <bool FROM_CACHE>
+struct TileSrc;
+template <>
+struct TileSrc<false> {
+    const char* k; // current_key / current_value row of token 0 of the sequence, this kv head
+    const char* v;
+    uint32_t row_bytes;
+    uint32_t voff; // 4 * r0 rows + 16 * col bytes
+};
+template <>
+struct TileSrc<true> {
+    const char* k; // slab rows of token 0 of the sequence (this layer, K / V, this kv head)
+    const char* v;
+    const char* ks; // their scale rows
+    const char* vs;
+    uint32_t row_bytes, srow_bytes;
+    uint32_t voff, svoff;
+};
+
+__device__ inline void fetch_tile(TileRegs<false>& t, const TileSrc<false>& src, int64_t j0, int64_t kvlen) {
+    const int r0 = threadIdx.x >> 4;
+    if (j0 + kBN <= kvlen) { // whole tile inside the sequence (wave-uniform)
+        const char* kb = uniform_ptr(src.k + j0 * src.row_bytes);
+        const char* vb = uniform_ptr(src.v + j0 * src.row_bytes);
 #pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const int row = (tid >> 4) + 16 * pass;
-        *reinterpret_cast<uint4*>(lds_k + row * kLdsRow + col * 16) = t.k[pass];
-        *reinterpret_cast<uint4*>(lds_v + row * kLdsRow + col * 16) = t.v[pass];
+        for (int pass = 0; pass < 4; ++pass) {
+            t.k[pass] = *reinterpret_cast<const uint4*>(kb + pass * src.row_bytes + src.voff);
+            t.v[pass] = *reinterpret_cast<const uint4*>(vb + pass * src.row_bytes + src.voff);
+        }
+    } else { // last, partial tile: rows past the end read as zero
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int64_t j = j0 + 4 * r0 + pass;
+            t.k[pass] = t.v[pass] = make_uint4(0, 0, 0, 0);
+            if (j < kvlen) {
+                const int64_t off = (j0 + pass) * src.row_bytes + src.voff;
+                t.k[pass] = *reinterpret_cast<const uint4*>(src.k + off);
+                t.v[pass] = *reinterpret_cast<const uint4*>(src.v + off);
+            }
+        }
     }
 }
 
-__device__ inline void fetch_tile(TileRegs<true>& t, const PrefillParams& p, int64_t j0, int64_t kvlen, int64_t,
-                                  int64_t tok0, int kvh) {
-    const int tid = threadIdx.x, row = tid >> 2, quarter = tid & 3;
-    const int64_t j = j0 + row;
+__device__ inline void fetch_tile(TileRegs<true>& t, const TileSrc<true>& src, int64_t j0, int64_t kvlen) {
+    const int r0 = threadIdx.x >> 4;
+    if (j0 + kBN <= kvlen) {
+        const char* kb = uniform_ptr(src.k + j0 * src.row_bytes);
+        const char* vb = uniform_ptr(src.v + j0 * src.row_bytes);
+        const char* ksb = uniform_ptr(src.ks + j0 * src.srow_bytes);
+        const char* vsb = uniform_ptr(src.vs + j0 * src.srow_bytes);
 #pragma unroll
-    for (int kv = 0; kv < 2; ++kv) {
-        t.q[kv][0] = t.q[kv][1] = make_uint4(0, 0, 0, 0);
-        t.s[kv] = make_uint2(0, 0);
-        if (j < kvlen) {
-            const int64_t r = p.addr.row(tok0 + j, kv, kvh);
-            t.q[kv][0] = *reinterpret_cast<const uint4*>(p.cache + r + quarter * 32);
-            t.q[kv][1] = *reinterpret_cast<const uint4*>(p.cache + r + quarter * 32 + 16);
-            t.s[kv] = *reinterpret_cast<const uint2*>(p.scale + r / kQuantGroup + quarter * 4);
+        for (int pass = 0; pass < 4; ++pass) {
+            t.kq[pass] = *reinterpret_cast<const uint2*>(kb + pass * src.row_bytes + src.voff);
+            t.vq[pass] = *reinterpret_cast<const uint2*>(vb + pass * src.row_bytes + src.voff);
+            t.ks[pass] = *reinterpret_cast<const uint16_t*>(ksb + pass * src.srow_bytes + src.svoff);
+            t.vs[pass] = *reinterpret_cast<const uint16_t*>(vsb + pass * src.srow_bytes + src.svoff);
+        }
+    } else {
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int64_t j = j0 + 4 * r0 + pass;
+            t.kq[pass] = t.vq[pass] = make_uint2(0, 0);
+            t.ks[pass] = t.vs[pass] = 0;
+            if (j < kvlen) {
+                const int64_t off = (j0 + pass) * src.row_bytes + src.voff;
+                const int64_t soff = (j0 + pass) * src.srow_bytes + src.svoff;
+                t.kq[pass] = *reinterpret_cast<const uint2*>(src.k + off);
+                t.vq[pass] = *reinterpret_cast<const uint2*>(src.v + off);
+                t.ks[pass] = *reinterpret_cast<const uint16_t*>(src.ks + soff);
+                t.vs[pass] = *reinterpret_cast<const uint16_t*>(src.vs + soff);
+            }
         }
     }
 }
-__device__ inline void store_tile(const TileRegs<true>& t, char* lds_k, char* lds_v) {
-    const int tid = threadIdx.x, row = tid >> 2, quarter = tid & 3;
+
+__device__ inline TileSrc<false> make_tile_src_f16(const PrefillParams& p, int64_t s0, int kvh) {
+    TileSrc<false> src;
+    const int tid = threadIdx.x, col = tid & 15, r0 = tid >> 4;
+    src.row_bytes = (uint32_t)p.kv_heads * kPDh * 2;
+    const int64_t first = (s0 * p.kv_heads + kvh) * kPDh * 2;
+    src.k = reinterpret_cast<const char*>(p.k) + first;
+    src.v = reinterpret_cast<const char*>(p.v) + first;
+    src.voff = 4 * r0 * src.row_bytes + col * 16;
+    return src;
+}
+__device__ inline TileSrc<true> make_tile_src_cache(const PrefillParams& p, int64_t tok0, int kvh) {
+    TileSrc<true> src;
+    const int tid = threadIdx.x, col = tid & 15, r0 = tid >> 4;
+    const int64_t rk = p.addr.row(tok0, 0, kvh), rv = p.addr.row(tok0, 1, kvh);
+    src.row_bytes = (uint32_t)p.addr.stride_s; // int8: one byte per element
+    src.srow_bytes = src.row_bytes / kQuantGroup * 2;
+    src.k = reinterpret_cast<const char*>(p.cache) + rk;
+    src.v = reinterpret_cast<const char*>(p.cache) + rv;
+    src.ks = reinterpret_cast<const char*>(p.scale) + rk / kQuantGroup * 2;
+    src.vs = reinterpret_cast<const char*>(p.scale) + rv / kQuantGroup * 2;
+    src.voff = 4 * r0 * src.row_bytes + col * 8;
+    src.svoff = 4 * r0 * src.srow_bytes + col * 2;
+    return src;
+}
+
+// 8 int8 values times one fp16 scale -> 8 fp16 values (the product is rounded once, as in the decode kernel's
+// dequantisation: |q| <= 128 is exact in fp16 and so is the fp32 product before the final rounding)
+__device__ inline uint4 dequant8(uint2 q, uint16_t scale_bits) {
+    half_t sc;
+    __builtin_memcpy(&sc, &scale_bits, 2);
+    const float sf = (float)sc;
+    const uint32_t w[2] = {q.x, q.y};
+    half_t o[8];
 #pragma unroll
-    for (int kv = 0; kv < 2; ++kv) {
-        char* dst = (kv ? lds_v : lds_k) + row * kLdsRow + quarter * 64;
-        const uint32_t w[8] = {t.q[kv][0].x, t.q[kv][0].y, t.q[kv][0].z, t.q[kv][0].w,
-                               t.q[kv][1].x, t.q[kv][1].y, t.q[kv][1].z, t.q[kv][1].w};
-        half_t sc[4];
-        __builtin_memcpy(sc, &t.s[kv], 8);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            half_t o[8];
-            const float sf = (float)sc[g];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int qi = (int)(int8_t)((w[2 * g + (i >> 2)] >> (8 * (i & 3))) & 0xff);
-                o[i] = (half_t)((float)qi * sf);
-            }
-            uint4 packed;
-            __builtin_memcpy(&packed, o, 16);
-            *reinterpret_cast<uint4*>(dst + g * 16) = packed;
-        }
+    for (int i = 0; i < 8; ++i) {
+        const int qi = (int)(int8_t)((w[i >> 2] >> (8 * (i & 3))) & 0xff);
+        o[i] = (half_t)((float)qi * sf);
     }
+    uint4 packed;
+    __builtin_memcpy(&packed, o, 16);
+    return packed;
+}
+
+// K rows go to LDS as they are; V is transposed: row = channel, and token t of the tile sits at position
+// (t with bits 2 and 3 swapped), 16-byte chunks XOR-swizzled by row / 16 so that both these 8-byte writes and the
+// 16-byte reads of the PV step spread over all banks.
+__device__ inline void store_kv(const uint4 (&kr)[4], const uint4 (&vr)[4], char* lds_k, char* lds_vt) {
+    const int tid = threadIdx.x, col = tid & 15, r0 = tid >> 4;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass)
+        *reinterpret_cast<uint4*>(lds_k + (4 * r0 + pass) * kLdsRow + col * 16) = kr[pass];
+    const int chunk = (2 * (r0 >> 2) + (r0 & 1)) ^ (col >> 1); // (position * 2 / 16) ^ (row / 16), row / 16 = col / 2
+    char* dst = lds_vt + (8 * col) * kVtRow + chunk * 16 + 8 * ((r0 >> 1) & 1);
+    const uint32_t a[4][4] = {{vr[0].x, vr[0].y, vr[0].z, vr[0].w},
+                              {vr[1].x, vr[1].y, vr[1].z, vr[1].w},
+                              {vr[2].x, vr[2].y, vr[2].z, vr[2].w},
+                              {vr[3].x, vr[3].y, vr[3].z, vr[3].w}};
+#pragma unroll
+    for (int m = 0; m < 4; ++m) { // dword m of a token = channels 2m, 2m+1
+        uint2 lo, hi;
+        lo.x = __builtin_amdgcn_perm(a[1][m], a[0][m], 0x05040100u);
+        lo.y = __builtin_amdgcn_perm(a[3][m], a[2][m], 0x05040100u);
+        hi.x = __builtin_amdgcn_perm(a[1][m], a[0][m], 0x07060302u);
+        hi.y = __builtin_amdgcn_perm(a[3][m], a[2][m], 0x07060302u);
+        *reinterpret_cast<uint2*>(dst + (2 * m) * kVtRow) = lo;
+        *reinterpret_cast<uint2*>(dst + (2 * m + 1) * kVtRow) = hi;
+    }
+}
+__device__ inline void store_tile(const TileRegs<false>& t, char* lds_k, char* lds_vt) {
+    store_kv(t.k, t.v, lds_k, lds_vt);
+}
+__device__ inline void store_tile(const TileRegs<true>& t, char* lds_k, char* lds_vt) {
+    uint4 kr[4], vr[4];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        kr[pass] = dequant8(t.kq[pass], t.ks[pass]);
+        vr[pass] = dequant8(t.vq[pass], t.vs[pass]);
+    }
+    store_kv(kr, vr, lds_k, lds_vt);
+}
+
+// the value the lane 32 positions away holds (the two half-waves of a query column exchange partial results)
+__device__ inline float other_half(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    // lower lanes: r[1] holds the upper half's value; upper lanes: r[0] holds the lower half's value
+    return (threadIdx.x & 32) ? __uint_as_float(r[0]) : __uint_as_float(r[1]);
 }
 
 template <bool FROM_CACHE>
 __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) char lds_k[kBN * kLdsRow];
-    __shared__ __attribute__((aligned(16))) char lds_v[kBN * kLdsRow];
+    // two K/V tile buffers: tile t+1 is written while tile t is read, one workgroup barrier per tile
+    __shared__ __attribute__((aligned(16))) char lds[2 * kLdsBufBytes];
 
     // ---- which (query tile, sequence, head): heaviest tiles of every sequence and head first
     const int per_tile = p.num_seqs * p.num_heads;
@@ -161,7 +283,10 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     if (kv_end > kvlen) kv_end = kvlen;
 
     TileRegs<FROM_CACHE> regs;
-    fetch_tile(regs, p, 0, kvlen, s0, tok0, kvh);
+    TileSrc<FROM_CACHE> src;
+    if constexpr (FROM_CACHE) src = make_tile_src_cache(p, tok0, kvh);
+    else src = make_tile_src_f16(p, s0, kvh);
+    fetch_tile(regs, src, 0, kvlen);
 
     // Q^T as the B operand: qB[kk] = Q[row][16*kk + 8*hb .. +7]
     half8_t qB[8];
@@ -175,124 +300,138 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
         }
     }
 
-    float16_t oT[4];
+    float16_t oT[4]; // O^T accumulators: oT[i][r] = channel 32*i + 8*(r/4) + 4*hb + r%4 of query row n
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oT[i][r] = 0.f;
-    float m_run = -INFINITY, l_part = 0.f; // m_run is the running max of the RAW scores (before the exp2 scaling)
+    // m_ref: reference maximum of the RAW scores (before the exp2 scaling) that the probabilities are taken against
+    float m_ref = -INFINITY, l_part = 0.f;
 
     const int64_t wave_last_vis = p.is_causal ? sp + q0 + 32 * wave + 31 : kvlen; // last key any row of this wave sees
     const int64_t wave_first_vis = p.is_causal ? sp + q0 + 32 * wave : kvlen; // keys <= this are seen by all its rows
     const int64_t vis = p.is_causal ? sp + row : kvlen; // last visible key of this lane's row
+    const int64_t last_key = vis < kvlen - 1 ? vis : kvlen - 1; // last key this lane's row may attend to
     const float c = p.score_scale;
 
-    for (int64_t j0 = 0; j0 < kv_end; j0 += kBN) {
-        __syncthreads(); // every wave is done reading the previous tile
-        store_tile(regs, lds_k, lds_v);
-        __syncthreads();
-        if (j0 + kBN < kv_end) fetch_tile(regs, p, j0 + kBN, kvlen, s0, tok0, kvh); // in flight during the compute
-        if (j0 > wave_last_vis) continue; // the whole tile is above this wave's diagonal (wave-uniform)
+    // per-lane LDS offsets that do not depend on the tile
+    const int k_off = n * kLdsRow + 16 * hb;
+    int vt_off[4]; // V^T row n of channel block 0 with 16-byte chunk (2*pr + hb) ^ (n >> 4); channel block i adds 32
+                   // rows and, through the row / 16 swizzle, flips the pair index pr by i
+#pragma unroll
+    for (int pr = 0; pr < 4; ++pr) vt_off[pr] = kLdsKBytes + n * kVtRow + (((2 * pr + hb) ^ (n >> 4)) << 4);
 
-        // ---- S^T tiles: 2 x (32 kv tokens x 32 query rows)
-        float16_t sT[2];
+    // pipeline: registers hold tile t+1 (in flight from global memory) while tile t is computed out of LDS buffer t & 1;
+    // after the compute the registers are parked in the other buffer and the loads of tile t+2 are issued
+    store_tile(regs, lds, lds + kLdsKBytes);
+    if (kBN < kv_end) fetch_tile(regs, src, kBN, kvlen);
+    __syncthreads();
+    int buf = 0;
+    for (int64_t j0 = 0; j0 < kv_end; j0 += kBN, buf ^= 1) {
+        const char* tile = lds + buf * kLdsBufBytes;
+        if (j0 <= wave_last_vis) { // else the whole tile is above this wave's diagonal (wave-uniform)
+            // ---- S^T tiles: 2 x (32 kv tokens x 32 query rows)
+            float16_t sT[2];
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            float16_t acc;
+            for (int blk = 0; blk < 2; ++blk) {
+                float16_t acc;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-            const char* kr = lds_k + (32 * blk + n) * kLdsRow + 16 * hb;
+                for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+                const char* kr = tile + 32 * blk * kLdsRow + k_off;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) {
-                half8_t a;
-                const uint4 x = *reinterpret_cast<const uint4*>(kr + 32 * kk);
-                __builtin_memcpy(&a, &x, 16);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qB[kk], acc, 0, 0, 0);
+                for (int kk = 0; kk < 8; ++kk) {
+                    half8_t a;
+                    const uint4 x = *reinterpret_cast<const uint4*>(kr + 32 * kk);
+                    __builtin_memcpy(&a, &x, 16);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qB[kk], acc, 0, 0, 0);
+                }
+                sT[blk] = acc;
             }
-            sT[blk] = acc;
-        }
-        const bool need_mask = (j0 + kBN - 1 > wave_first_vis) || (j0 + kBN > kvlen);
-        if (need_mask) {
+            const bool need_mask = (j0 + kBN - 1 > wave_first_vis) || (j0 + kBN > kvlen);
+            if (need_mask) {
+                // last visible token of this row, relative to the tile, clamped to [-1, 63]
+                const int64_t lim64 = last_key - j0;
+                const int lim = (int)(lim64 < -1 ? -1 : (lim64 > kBN - 1 ? kBN - 1 : lim64));
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (32 * blk + 8 * (r >> 2) + 4 * hb + (r & 3) > lim) sT[blk][r] = -INFINITY;
+            }
+
+            // ---- online softmax for this lane's query row: p = exp2(s*c - m*c), one fma + one exp2 per score
+            float mx = -INFINITY;
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int64_t j = j0 + 32 * blk + 8 * (r >> 2) + 4 * hb + (r & 3);
-                    if (j > vis || j >= kvlen) sT[blk][r] = -INFINITY;
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sT[blk][r]);
+            mx = fmaxf(mx, other_half(mx));
+            // key 0 is visible to every row, so the first tile gives every row a finite maximum (m_ref = -inf forces
+            // the update); rows past the sequence end have all-zero queries and stay finite as well
+            const bool moved = (mx - m_ref) * c > kRescaleLog2;
+            if (__any(moved)) { // a row's result depends on its own scores only: rows that did not move keep theirs
+                const float m_new = moved ? mx : m_ref;
+                const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
+                m_ref = m_new;
+                l_part *= alpha;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) oT[i] *= alpha;
+            }
+            const float neg_mc = -m_ref * c;
+            float psum = 0.f;
+            half8_t pB[4]; // pB[2*blk + J]: k-slot e8 <-> token 32*blk + 16*J + 8*(e8/4) + 4*hb + e8%4
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int J = 0; J < 2; ++J) {
+                    float pe[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sT[blk][8 * J + e], c, neg_mc));
+                        psum += pe[e];
+                    }
+                    pB[2 * blk + J] = half8_t{(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3],
+                                              (half_t)pe[4], (half_t)pe[5], (half_t)pe[6], (half_t)pe[7]};
+                }
+            l_part += psum;
+
+            // ---- O^T += V^T * P^T: channel block i (32 channels), 16 tokens per MFMA k-block
+#pragma unroll
+            for (int J = 0; J < 4; ++J)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    half8_t a;
+                    const uint4 x = *reinterpret_cast<const uint4*>(tile + vt_off[J ^ i] + i * 32 * kVtRow);
+                    __builtin_memcpy(&a, &x, 16);
+                    oT[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pB[J], oT[i], 0, 0, 0);
                 }
         }
-
-        // ---- online softmax for this lane's query row: p = exp2(s*c - m*c), one fma + one exp2 per score
-        float mx = -INFINITY;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sT[blk][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // key 0 is visible to every row, so m_new is finite from the first tile on; rows past the sequence end have
-        // all-zero queries and stay finite as well
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
-        m_run = m_new;
-        const float neg_mc = -m_new * c;
-        float psum = 0.f;
-        half8_t pB[4]; // pB[2*blk + J]: k-slot e8 <-> token 32*blk + 16*J + 8*(e8/4) + 4*hb + e8%4
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int J = 0; J < 2; ++J) {
-                float pe[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sT[blk][8 * J + e], c, neg_mc));
-                    psum += pe[e];
-                }
-                pB[2 * blk + J] = half8_t{(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3],
-                                          (half_t)pe[4], (half_t)pe[5], (half_t)pe[6], (half_t)pe[7]};
-            }
-        l_part = l_part * alpha + psum;
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) oT[i] *= alpha;
+        if (j0 + kBN < kv_end) {
+            // the other buffer was last read during the previous iteration, which every wave left through the barrier
+            char* next = lds + (buf ^ 1) * kLdsBufBytes;
+            store_tile(regs, next, next + kLdsKBytes);
+            if (j0 + 2 * kBN < kv_end) fetch_tile(regs, src, j0 + 2 * kBN, kvlen);
         }
-
-        // ---- O^T += V^T * P^T, 16 tokens per MFMA k-block
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
-            uint2 vr[8]; // vr[e8]: channels 4n .. 4n+3 of token 16*kb + 8*(e8/4) + 4*hb + e8%4
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                vr[e] = *reinterpret_cast<const uint2*>(lds_v + (16 * kb + 8 * (e >> 2) + 4 * hb + (e & 3)) * kLdsRow + 8 * n);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-                uint32_t t[4];
-#pragma unroll
-                for (int pr = 0; pr < 4; ++pr)
-                    t[pr] = __builtin_amdgcn_perm((i < 2) ? vr[2 * pr + 1].x : vr[2 * pr + 1].y,
-                                                  (i < 2) ? vr[2 * pr].x : vr[2 * pr].y, sel);
-                half8_t a;
-                __builtin_memcpy(&a, t, 16);
-                oT[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pB[kb], oT[i], 0, 0, 0);
-            }
-        }
+        __syncthreads();
     }
 
-    const float l_tot = l_part + __shfl_xor(l_part, 32);
+    const float l_tot = l_part + other_half(l_part);
     const float inv = 1.0f / l_tot;
-    // ---- output through LDS: each wave parks its 32 x 128 fp16 tile in its own 32 rows, then writes full rows
-    __syncthreads(); // all waves are done with the last K/V tile
-    char* otile = (wave < 2 ? lds_k : lds_v) + (wave & 1) * 32 * kLdsRow;
-    // lane (row n, hb) holds, in oT[i][r], channel 4 * (8*(r/4) + 4*hb + r%4) + i
+    // ---- output through LDS (the loop's last barrier freed it): each wave parks its 32 x 128 fp16 tile in its own
+    // 32 rows, then writes full rows
+    char* otile = lds + wave * 32 * kLdsRow;
+    // lane (query row n, hb) holds, in oT[i][r], channel 32*i + 8*(r/4) + 4*hb + r%4
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int ch = 4 * (8 * (r >> 2) + 4 * hb + (r & 3));
-        const half4_t o = {(half_t)(oT[0][r] * inv), (half_t)(oT[1][r] * inv), (half_t)(oT[2][r] * inv),
-                           (half_t)(oT[3][r] * inv)};
-        uint2 packed;
-        __builtin_memcpy(&packed, &o, 8);
-        *reinterpret_cast<uint2*>(otile + n * kLdsRow + ch * 2) = packed;
-    }
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int ch = 32 * i + 8 * g + 4 * hb;
+            const half4_t o = {(half_t)(oT[i][4 * g] * inv), (half_t)(oT[i][4 * g + 1] * inv),
+                               (half_t)(oT[i][4 * g + 2] * inv), (half_t)(oT[i][4 * g + 3] * inv)};
+            uint2 packed;
+            __builtin_memcpy(&packed, &o, 8);
+            *reinterpret_cast<uint2*>(otile + n * kLdsRow + ch * 2) = packed;
+        }
     // (same wave wrote and reads: no workgroup barrier needed, the compiler orders the LDS accesses)
 #pragma unroll
     for (int pass = 0; pass < 8; ++pass) {
