@@ -181,6 +181,98 @@ typedef struct pplhip_kv_cache_args {
 pplhip_retcode pplhip_kv_cache_forward(const pplhip_kv_cache_args* args, void* stream);
 
 /*
+ * opmx.dynamic_batching::MultiHeadAttention (no cache): the argument list of
+ * `ppl::kernel::llm::cuda::pmx::dynamic_batching_multi_head_attention` as called from
+ * src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/multi_head_attention_kernel.cc:105-127.
+ *   query  fp16 [seqstarts[batch], num_heads, head_dim]
+ *   key    fp16 [kvstarts[batch], num_kv_heads, head_dim]   all keys of every sequence, packed in batch order
+ *   value  fp16 [kvstarts[batch], num_kv_heads, head_dim]
+ *   output fp16 [seqstarts[batch], num_heads, head_dim]
+ * The queries of a sequence are its LAST seqlen keys: with is_causal, query i of sequence b attends to keys
+ * 0 .. (kvlen_b - seqlen_b) + i; without, to all kvlen_b keys. kvlen_b >= seqlen_b >= 1 is required.
+ * MultiHeadCacheAttention == MultiHeadAttention applied to the outputs of KeyValueCache.
+ * Same limits as above: head_dim 128, at most 16 query heads per kv head, no attn_mask, no alibi.
+ */
+typedef struct pplhip_mha_args {
+    const void* d_query;
+    const void* d_key;
+    const void* d_value;
+    const void* d_attn_mask; /* must be NULL */
+    const int64_t* d_seqstarts; /* [batch+1] */
+    const int64_t* d_kvstarts; /* [batch+1] */
+    int32_t is_causal;
+    int32_t is_alibi; /* must be 0: RC_UNSUPPORTED otherwise (multi_head_attention_kernel.cc:71-74) */
+    int64_t batch;
+    int64_t decoding_batches; /* accepted for interface parity; every sequence takes the same path */
+    int64_t max_seqlen;
+    int64_t max_kvlen;
+    int32_t num_heads;
+    int32_t num_kv_heads;
+    int32_t head_dim;
+    int32_t reserved;
+    void* d_output;
+} pplhip_mha_args;
+
+pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* args, void* stream);
+
+/*
+ * opmx.dynamic_batching::RotaryPositionEmbedding: the argument list of
+ * `ppl::kernel::llm::cuda::pmx::dynamic_batching_rotary_position_embedding` as called from
+ * src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/rotary_position_embedding_kernel.cc:110-132.
+ *   query / rotated_query  fp16 [total_tokens, num_heads, head_dim]
+ *   key   / rotated_key    fp16 [total_tokens, num_key_heads, head_dim]     (outputs may alias the inputs)
+ * Token t of sequence b has position start_pos[b] + (t - seqstarts[b]); channel pair (2i, 2i+1), 2i < rotary_dim,
+ * is rotated by position * theta^(-2i / rotary_dim):
+ *     y[2i] = x[2i] cos - x[2i+1] sin,   y[2i+1] = x[2i+1] cos + x[2i] sin;
+ * channels >= rotary_dim are copied; `bypass_key` copies the key unrotated. rotary_dim 0 means head_dim.
+ * scaling_type: the values of RotaryPositionEmbeddingParam (src/ppl/nn/params/opmx/rotary_position_embedding_param.h:
+ * 12-16). LINEAR divides the position by scaling_factor. DYNAMIC, for a sequence whose total length
+ * T = start_pos + seqlen exceeds max_position_embeddings, replaces theta by
+ * theta * (scaling_factor * T / max_position_embeddings - (scaling_factor - 1)) ^ (rotary_dim / (rotary_dim - 2)).
+ * (The reference wrapper maps the three values through an inverted `!=` chain at
+ * rotary_position_embedding_kernel.cc:99-108, which sends NONE to LINEAR and everything else to NONE; this library
+ * takes the value at its name.)
+ * head_dim and rotary_dim must be multiples of 8, head_dim <= 2048.
+ */
+enum {
+    PPLHIP_ROPE_SCALING_NONE = 0,
+    PPLHIP_ROPE_SCALING_LINEAR = 1,
+    PPLHIP_ROPE_SCALING_DYNAMIC = 2
+};
+
+typedef struct pplhip_rope_args {
+    const void* d_query;
+    const void* d_key;
+    const int64_t* d_start_pos; /* [batch] */
+    const int64_t* d_seqstarts; /* [batch+1] */
+    float theta;
+    int32_t bypass_key;
+    int32_t rotary_dim;
+    int32_t reserved;
+    int64_t batch;
+    int64_t total_tokens; /* = seqstarts[batch] = dim 0 of query and key */
+    int32_t num_heads;
+    int32_t num_key_heads;
+    int32_t head_dim;
+    int32_t max_position_embeddings;
+    int64_t max_seqlen;
+    int32_t scaling_type;
+    float scaling_factor;
+    void* d_rotated_query;
+    void* d_rotated_key;
+} pplhip_rope_args;
+
+pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* args, void* stream);
+
+/*
+ * opmx.dynamic_batching::PositionIndex (`dynamic_batching_position_index` as called from
+ * src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/position_index_kernel.cc:60-67):
+ * position_idx[t] = start_pos[b] + (t - seqstarts[b]) for every packed token t of sequence b; i64 [total_tokens].
+ */
+pplhip_retcode pplhip_position_index(const int64_t* d_start_pos, const int64_t* d_seqstarts, int64_t batch,
+                                     int64_t total_tokens, int64_t max_seqlen, int64_t* d_position_idx, void* stream);
+
+/*
  * On-device rebuild of the ragged-batch tables, replacing the host loops of
  * tools/benchmark_llama/generation_state.cc:60-125 (FirstStep) and :127-192 (NextStep) plus the eight per-step
  * uploads of tools/benchmark_llama/text_generator.cc:233-291.

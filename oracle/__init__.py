@@ -31,6 +31,12 @@ def lib():
         L.oracle_kv_quantize_write.restype = C.c_int
         L.oracle_mhca_forward.argtypes = [vp, vp]
         L.oracle_mhca_forward.restype = C.c_int
+        L.oracle_mha_forward.argtypes = [vp, vp]
+        L.oracle_mha_forward.restype = C.c_int
+        L.oracle_rope_forward.argtypes = [vp]
+        L.oracle_rope_forward.restype = C.c_int
+        L.oracle_position_index.argtypes = [vp, vp, i64, vp]
+        L.oracle_position_index.restype = C.c_int
         L.oracle_kv_cache_forward.argtypes = [vp]
         L.oracle_kv_cache_forward.restype = C.c_int
         L.oracle_pack_tables.argtypes = [vp]

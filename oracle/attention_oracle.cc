@@ -18,6 +18,12 @@
 //                          Bit pattern of the absent CUDA kernel: parity unpinned.
 //   oracle_mhca_forward    pinned against a float64 numpy softmax(QK^T/sqrt(d)+mask)V, closed forms
 //                          (kvlen 1, equal keys, dominant key), GQA==MHA, decode == last prefill row, NaN poison.
+//   oracle_mha_forward     pinned against the same float64 textbook routine (explicit K/V, kvlen >= seqlen offsets)
+//                          and by the identity MHCA == MHA applied to KeyValueCache's outputs.
+//   oracle_rope_forward    pinned by rotation invariants (pair norms, position 0 = identity, R(p1+p2) = R(p1)R(p2),
+//                          q.k depends on the position difference only) and a numpy complex-multiply restatement;
+//                          pair convention and NTK formula of the absent kernel: parity unpinned.
+//   oracle_position_index  pinned by a Python loop.
 //   oracle_kv_cache_forward pinned by |dequant(quant(x)) - x| <= scale/2 and row-order checks.
 //   oracle_pack_tables     pinned against a brute-force Python loop written from generation_state.cc.
 //   oracle_x86_attention   pinned against the same float64 textbook routine.
@@ -223,6 +229,120 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
             }
         }
     }
+    return PPLHIP_RC_SUCCESS;
+}
+
+// MultiHeadAttention (no cache): explicit packed fp16 key/value rows indexed by kvstarts; the queries of a sequence
+// are its last seqlen keys. Argument meaning follows the call at
+// src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/multi_head_attention_kernel.cc:105-127.
+int oracle_mha_forward(const pplhip_mha_args* a, double* out_f64) {
+    const int H = a->num_heads, KVH = a->num_kv_heads, Dh = a->head_dim;
+    if (H <= 0 || KVH <= 0 || H % KVH) return PPLHIP_RC_INVALID_VALUE;
+    if (a->d_attn_mask || a->is_alibi) return PPLHIP_RC_UNSUPPORTED;
+    const uint16_t* Q = (const uint16_t*)a->d_query;
+    const uint16_t* Kp = (const uint16_t*)a->d_key;
+    const uint16_t* Vp = (const uint16_t*)a->d_value;
+    uint16_t* O = (uint16_t*)a->d_output;
+    const int rep = H / KVH;
+    const double sm_scale = 1.0 / sqrt((double)Dh);
+#pragma omp parallel for collapse(2) schedule(dynamic, 1)
+    for (int64_t b = 0; b < a->batch; ++b) {
+        for (int h = 0; h < H; ++h) {
+            const int kvh = h / rep;
+            const int64_t s0 = a->d_seqstarts[b], seqlen = a->d_seqstarts[b + 1] - s0;
+            const int64_t k0 = a->d_kvstarts[b], kvlen = a->d_kvstarts[b + 1] - k0;
+            const int64_t sp = kvlen - seqlen;
+            std::vector<double> p((size_t)kvlen), acc(Dh), q(Dh);
+            for (int64_t t = 0; t < seqlen; ++t) {
+                const uint16_t* qr = Q + ((s0 + t) * H + h) * Dh;
+                for (int d = 0; d < Dh; ++d) q[d] = half_to_float(qr[d]);
+                const int64_t last = a->is_causal ? std::min<int64_t>(sp + t, kvlen - 1) : kvlen - 1;
+                double m = -INFINITY;
+                for (int64_t j = 0; j <= last; ++j) {
+                    const uint16_t* kr = Kp + ((k0 + j) * KVH + kvh) * Dh;
+                    double s = 0;
+                    for (int d = 0; d < Dh; ++d) s += q[d] * (double)half_to_float(kr[d]);
+                    p[j] = s * sm_scale;
+                    m = std::max(m, p[j]);
+                }
+                double l = 0;
+                for (int64_t j = 0; j <= last; ++j) {
+                    p[j] = exp(p[j] - m);
+                    l += p[j];
+                }
+                std::fill(acc.begin(), acc.end(), 0.0);
+                for (int64_t j = 0; j <= last; ++j) {
+                    const uint16_t* vr = Vp + ((k0 + j) * KVH + kvh) * Dh;
+                    for (int d = 0; d < Dh; ++d) acc[d] += p[j] * (double)half_to_float(vr[d]);
+                }
+                for (int d = 0; d < Dh; ++d) {
+                    const double o = acc[d] / l;
+                    const int64_t idx = ((s0 + t) * H + h) * Dh + d;
+                    if (out_f64) out_f64[idx] = o;
+                    O[idx] = float_to_half((float)o);
+                }
+            }
+        }
+    }
+    return PPLHIP_RC_SUCCESS;
+}
+
+// RotaryPositionEmbedding over a ragged batch, float64 throughout, one rounding to binary16 at the end.
+// Argument meaning follows src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/
+// rotary_position_embedding_kernel.cc:110-132; the pair convention (consecutive channels rotate together, angle
+// position * theta^(-2i/rotary_dim)) and the linear / dynamic-NTK position scaling restate the published
+// algorithm of the absent kernel library: parity unpinned against its exact bits.
+int oracle_rope_forward(const pplhip_rope_args* a) {
+    const int Dh = a->head_dim, rd = a->rotary_dim == 0 ? Dh : a->rotary_dim;
+    if (Dh <= 0 || rd % 2 || rd > Dh) return PPLHIP_RC_INVALID_VALUE;
+    const uint16_t* Q = (const uint16_t*)a->d_query;
+    const uint16_t* K = (const uint16_t*)a->d_key;
+    uint16_t* QO = (uint16_t*)a->d_rotated_query;
+    uint16_t* KO = (uint16_t*)a->d_rotated_key;
+    for (int64_t b = 0; b < a->batch; ++b) {
+        const int64_t s0 = a->d_seqstarts[b], seqlen = a->d_seqstarts[b + 1] - s0, sp = a->d_start_pos[b];
+        double theta = (double)a->theta;
+        if (a->scaling_type == PPLHIP_ROPE_SCALING_DYNAMIC) {
+            const double total = (double)(sp + seqlen), maxp = (double)a->max_position_embeddings;
+            if (total > maxp) {
+                const double f = (double)a->scaling_factor;
+                theta *= pow(f * total / maxp - (f - 1.0), (double)rd / (double)(rd - 2));
+            }
+        }
+        for (int64_t t = 0; t < seqlen; ++t) {
+            double pos = (double)(sp + t);
+            if (a->scaling_type == PPLHIP_ROPE_SCALING_LINEAR) pos /= (double)a->scaling_factor;
+            for (int which = 0; which < 2; ++which) {
+                const int heads = which ? a->num_key_heads : a->num_heads;
+                const uint16_t* src = which ? K : Q;
+                uint16_t* dst = which ? KO : QO;
+                const bool bypass = which && a->bypass_key;
+                for (int h = 0; h < heads; ++h) {
+                    const int64_t off = ((s0 + t) * heads + h) * Dh;
+                    for (int i = 0; i < Dh / 2; ++i) {
+                        const uint16_t r0 = src[off + 2 * i], r1 = src[off + 2 * i + 1];
+                        if (bypass || 2 * i >= rd) {
+                            dst[off + 2 * i] = r0;
+                            dst[off + 2 * i + 1] = r1;
+                            continue;
+                        }
+                        const double ang = pos * pow(theta, -2.0 * i / (double)rd);
+                        const double c = cos(ang), sn = sin(ang);
+                        const double x0 = half_to_float(r0), x1 = half_to_float(r1);
+                        dst[off + 2 * i] = float_to_half((float)(x0 * c - x1 * sn));
+                        dst[off + 2 * i + 1] = float_to_half((float)(x1 * c + x0 * sn));
+                    }
+                }
+            }
+        }
+    }
+    return PPLHIP_RC_SUCCESS;
+}
+
+// PositionIndex: position of every packed token (position_index_kernel.cc:60-67 for the argument meaning).
+int oracle_position_index(const int64_t* start_pos, const int64_t* seqstarts, int64_t batch, int64_t* out) {
+    for (int64_t b = 0; b < batch; ++b)
+        for (int64_t t = seqstarts[b]; t < seqstarts[b + 1]; ++t) out[t] = start_pos[b] + (t - seqstarts[b]);
     return PPLHIP_RC_SUCCESS;
 }
 

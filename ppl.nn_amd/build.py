@@ -8,7 +8,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "decode.hip", "prefill.hip", "pack.hip"]
+KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "decode.hip", "prefill.hip", "pack.hip", "rope.hip"]
 
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",

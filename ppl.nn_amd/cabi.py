@@ -75,6 +75,32 @@ class KvCacheArgs(C.Structure):
     ]
 
 
+class MhaArgs(C.Structure):
+    _fields_ = [
+        ("d_query", _p), ("d_key", _p), ("d_value", _p), ("d_attn_mask", _p),
+        ("d_seqstarts", _p), ("d_kvstarts", _p),
+        ("is_causal", _i32), ("is_alibi", _i32),
+        ("batch", _i64), ("decoding_batches", _i64), ("max_seqlen", _i64), ("max_kvlen", _i64),
+        ("num_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32), ("reserved", _i32),
+        ("d_output", _p),
+    ]
+
+
+class RopeArgs(C.Structure):
+    _fields_ = [
+        ("d_query", _p), ("d_key", _p), ("d_start_pos", _p), ("d_seqstarts", _p),
+        ("theta", C.c_float), ("bypass_key", _i32), ("rotary_dim", _i32), ("reserved", _i32),
+        ("batch", _i64), ("total_tokens", _i64),
+        ("num_heads", _i32), ("num_key_heads", _i32), ("head_dim", _i32), ("max_position_embeddings", _i32),
+        ("max_seqlen", _i64),
+        ("scaling_type", _i32), ("scaling_factor", C.c_float),
+        ("d_rotated_query", _p), ("d_rotated_key", _p),
+    ]
+
+
+ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_DYNAMIC = 0, 1, 2
+
+
 class PackArgs(C.Structure):
     _fields_ = [
         ("d_slot_kvlen", _p), ("d_slot_newlen", _p), ("d_slot_cachestart", _p),
@@ -90,6 +116,9 @@ PROTOTYPES = {
     "pplhip_version": (_i32, []),
     "pplhip_mhca_prepare": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan)]),
     "pplhip_mhca_forward": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan), _p, _p]),
+    "pplhip_mha_forward": (_i32, [C.POINTER(MhaArgs), _p]),
+    "pplhip_rope_forward": (_i32, [C.POINTER(RopeArgs), _p]),
+    "pplhip_position_index": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
     "pplhip_kv_quantize_write": (_i32, [C.POINTER(KvWriteArgs), _p]),
     "pplhip_kv_cache_forward": (_i32, [C.POINTER(KvCacheArgs), _p]),
     "pplhip_pack_tables": (_i32, [C.POINTER(PackArgs), _p]),

@@ -183,6 +183,65 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     return launch_prefill(a, plan, s);
 }
 
+pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {
+    if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (a->is_alibi) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support is_alibi == false");
+    if (a->d_attn_mask) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "attn_mask is not supported");
+    if (a->head_dim != 128) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: only 128 is supported", a->head_dim);
+    if (a->num_heads <= 0 || a->num_kv_heads <= 0 || a->num_heads % a->num_kv_heads != 0)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d must be a positive multiple of num_kv_heads %d",
+                    a->num_heads, a->num_kv_heads);
+    if (a->num_heads / a->num_kv_heads > 16)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "more than 16 query heads per kv head");
+    if (a->batch < 0 || a->max_seqlen < 0 || a->max_kvlen < a->max_seqlen)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "inconsistent batch %lld / max_seqlen %lld / max_kvlen %lld",
+                    (long long)a->batch, (long long)a->max_seqlen, (long long)a->max_kvlen);
+    if (a->batch == 0) return PPLHIP_RC_SUCCESS;
+    if (!a->d_query || !a->d_key || !a->d_value || !a->d_seqstarts || !a->d_kvstarts || !a->d_output)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
+    if (((uintptr_t)a->d_query & 15) || ((uintptr_t)a->d_key & 15) || ((uintptr_t)a->d_value & 15) ||
+        ((uintptr_t)a->d_output & 15))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "query/key/value/output must be 16-byte aligned");
+    return launch_mha(a, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* a, void* stream) {
+    if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (a->scaling_type != PPLHIP_ROPE_SCALING_NONE && a->scaling_type != PPLHIP_ROPE_SCALING_LINEAR &&
+        a->scaling_type != PPLHIP_ROPE_SCALING_DYNAMIC)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "invalid scaling type: %d", a->scaling_type);
+    const int rotary_dim = a->rotary_dim == 0 ? a->head_dim : a->rotary_dim;
+    if (a->head_dim <= 0 || a->head_dim % 8 || a->head_dim > 2048)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 8, at most 2048", a->head_dim);
+    if (rotary_dim < 0 || rotary_dim % 8 || rotary_dim > a->head_dim)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "rotary_dim %d: must be a multiple of 8 within head_dim %d", rotary_dim,
+                    a->head_dim);
+    if (a->num_heads <= 0 || a->num_key_heads <= 0)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d / num_key_heads %d", a->num_heads, a->num_key_heads);
+    if (!(a->theta > 0.f)) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "theta must be positive");
+    if (a->scaling_type != PPLHIP_ROPE_SCALING_NONE && !(a->scaling_factor > 0.f))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "scaling_factor must be positive");
+    if (a->scaling_type == PPLHIP_ROPE_SCALING_DYNAMIC && (a->max_position_embeddings <= 0 || rotary_dim <= 2))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "dynamic scaling needs max_position_embeddings > 0 and rotary_dim > 2");
+    if (a->batch < 0 || a->total_tokens < 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "negative batch or token count");
+    if (a->batch == 0 || a->total_tokens == 0) return PPLHIP_RC_SUCCESS;
+    if (!a->d_query || !a->d_key || !a->d_seqstarts || !a->d_start_pos || !a->d_rotated_query || !a->d_rotated_key)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
+    if (((uintptr_t)a->d_query & 15) || ((uintptr_t)a->d_key & 15) || ((uintptr_t)a->d_rotated_query & 15) ||
+        ((uintptr_t)a->d_rotated_key & 15))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "query/key tensors must be 16-byte aligned");
+    return launch_rope(a, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_position_index(const int64_t* d_start_pos, const int64_t* d_seqstarts, int64_t batch,
+                                     int64_t total_tokens, int64_t max_seqlen, int64_t* d_position_idx, void* stream) {
+    (void)max_seqlen;
+    if (batch < 0 || total_tokens < 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "negative batch or token count");
+    if (batch == 0 || total_tokens == 0) return PPLHIP_RC_SUCCESS;
+    if (!d_start_pos || !d_seqstarts || !d_position_idx) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
+    return launch_position_index(d_seqstarts, d_start_pos, batch, total_tokens, d_position_idx, (hipStream_t)stream);
+}
+
 pplhip_retcode pplhip_kv_quantize_write(const pplhip_kv_write_args* a, void* stream) {
     pplhip_retcode rc = validate_write(a);
     if (rc != PPLHIP_RC_SUCCESS) return rc;

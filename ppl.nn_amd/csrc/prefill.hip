@@ -261,8 +261,13 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     const int head = kvh * p.rep + hl / p.kv_heads;
     const int64_t s0 = p.seqstarts[b];
     const int64_t L = p.seqstarts[b + 1] - s0;
-    const int64_t sp = FROM_CACHE ? p.start_pos[b] : 0;
-    const int64_t kvlen = FROM_CACHE ? (p.kvstarts[b + 1] - p.kvstarts[b]) : L;
+    // K/V rows of the sequence: slab tokens cachestarts[b] .. +kvlen (cache source), or rows kvstarts[b] .. +kvlen of
+    // the packed fp16 key/value tensors. The new tokens are the LAST L of the kvlen keys: query row i sees keys
+    // <= sp + i with sp = kvlen - L (= start_pos for the cache source). MultiHeadCacheAttention without cache-prefill
+    // passes kvstarts = seqstarts, i.e. kvlen = L and sp = 0.
+    const int64_t kv0 = p.kvstarts[b];
+    const int64_t kvlen = p.kvstarts[b + 1] - kv0;
+    const int64_t sp = FROM_CACHE ? p.start_pos[b] : (kvlen > L ? kvlen - L : 0);
     const int64_t tok0 = FROM_CACHE ? p.cachestarts[b] : 0;
     const int ntiles = (int)((L + kBM - 1) / kBM);
     const int ntiles_max = gridDim.x / per_tile;
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     TileRegs<FROM_CACHE> regs;
     TileSrc<FROM_CACHE> src;
     if constexpr (FROM_CACHE) src = make_tile_src_cache(p, tok0, kvh);
-    else src = make_tile_src_f16(p, s0, kvh);
+    else src = make_tile_src_f16(p, kv0, kvh);
     fetch_tile(regs, src, 0, kvlen);
 
     // Q^T as the B operand: qB[kk] = Q[row][16*kk + 8*hb .. +7]
@@ -453,7 +458,8 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     p.cache = (const int8_t*)a->d_cache;
     p.scale = (const half_t*)a->d_scale;
     p.seqstarts = a->d_seqstarts;
-    p.kvstarts = a->d_kvstarts;
+    // fp16 source: the keys of a prefill sequence are its own new tokens, packed like the queries
+    p.kvstarts = a->enable_cache_prefill ? a->d_kvstarts : a->d_seqstarts;
     p.cachestarts = a->d_cachestarts;
     p.start_pos = a->d_start_pos;
     p.out = (half_t*)a->d_output;
@@ -473,6 +479,37 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     else
         hipLaunchKernelGGL(prefill_attention_kernel<false>, grid, dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("prefill_attention");
+    return PPLHIP_RC_SUCCESS;
+}
+
+// opmx.dynamic_batching::MultiHeadAttention: the same kernel over explicit packed fp16 key/value tensors; every
+// sequence (decode ones included) is a set of query tiles.
+pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
+    if (a->batch <= 0 || a->max_seqlen <= 0) return PPLHIP_RC_SUCCESS;
+    PrefillParams p;
+    p.q = (const half_t*)a->d_query;
+    p.k = (const half_t*)a->d_key;
+    p.v = (const half_t*)a->d_value;
+    p.cache = nullptr;
+    p.scale = nullptr;
+    p.seqstarts = a->d_seqstarts;
+    p.kvstarts = a->d_kvstarts;
+    p.cachestarts = nullptr;
+    p.start_pos = nullptr;
+    p.out = (half_t*)a->d_output;
+    p.addr = CacheAddr{0, 0, 0, 0, 0};
+    p.first_seq = 0;
+    p.num_heads = a->num_heads;
+    p.kv_heads = a->num_kv_heads;
+    p.rep = a->num_heads / a->num_kv_heads;
+    p.is_causal = a->is_causal;
+    p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
+    p.num_seqs = (int32_t)a->batch;
+    const int64_t q_tiles = (a->max_seqlen + kBM - 1) / kBM;
+    const int64_t blocks = q_tiles * a->batch * a->num_heads;
+    if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many query tiles in one call");
+    hipLaunchKernelGGL(prefill_attention_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    PPLHIP_CHECK_LAUNCH("multi_head_attention");
     return PPLHIP_RC_SUCCESS;
 }
 

@@ -1,0 +1,135 @@
+// opmx.dynamic_batching::RotaryPositionEmbedding and ::PositionIndex over ragged packed batches: the step that
+// precedes attention and uses the same seqstarts / start_pos tables.
+//
+// Both are streaming kernels (HBM roofline): RotaryPositionEmbedding reads and writes every query and key element
+// once, 16 bytes per lane; the angle of a (position, channel pair) is formed in float64 (position * theta^(-2i/d),
+// reduced mod 2*pi before it is narrowed), because a float32 product loses the low bits of a 100k-token position.
+// Pair convention: consecutive channels (x[2i], x[2i+1]) rotate together by position * theta^(-2i / rotary_dim);
+// channels >= rotary_dim pass through.
+#include "common.h"
+
+namespace pplhip {
+
+struct RopeParams {
+    const half_t* q;
+    const half_t* k;
+    half_t* q_out;
+    half_t* k_out;
+    const int64_t* seqstarts;
+    const int64_t* start_pos;
+    int32_t batch;
+    int32_t num_heads, num_key_heads;
+    int32_t head_dim, rotary_dim;
+    int32_t bypass_key;
+    int32_t scaling_type;
+    int32_t max_position_embeddings;
+    double log2_theta;
+    double scaling_factor;
+};
+
+constexpr double kTwoPi = 6.283185307179586476925286766559;
+
+__global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
+    const int64_t t = blockIdx.x; // packed token
+    const int cpr = p.head_dim / 8; // 16-byte chunks per head row
+    const int rows_per_pass = 256 / cpr;
+    const int slot = threadIdx.x / cpr;
+    const int chunk = threadIdx.x - slot * cpr;
+    if (slot >= rows_per_pass) return;
+
+    const int b = find_sequence(p.seqstarts, p.batch, t);
+    const int64_t s0 = p.seqstarts[b];
+    const int64_t sp = p.start_pos[b];
+    double pos = (double)(sp + (t - s0));
+    double log2_theta = p.log2_theta;
+    if (p.scaling_type == PPLHIP_ROPE_SCALING_LINEAR) {
+        pos /= p.scaling_factor;
+    } else if (p.scaling_type == PPLHIP_ROPE_SCALING_DYNAMIC) {
+        const double total = (double)(sp + (p.seqstarts[b + 1] - s0));
+        if (total > (double)p.max_position_embeddings) {
+            const double grow = p.scaling_factor * total / (double)p.max_position_embeddings - (p.scaling_factor - 1.0);
+            log2_theta += log2(grow) * ((double)p.rotary_dim / (double)(p.rotary_dim - 2));
+        }
+    }
+    // this lane's 4 channel pairs: 4*chunk .. 4*chunk+3
+    float cs[4], sn[4];
+    const bool rotate = 8 * chunk < p.rotary_dim; // rotary_dim is a multiple of 8: a chunk is rotated whole or not at all
+    if (rotate) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int pair = 4 * chunk + j;
+            const double inv_freq = exp2(-(2.0 * pair / (double)p.rotary_dim) * log2_theta);
+            double a = pos * inv_freq;
+            a -= kTwoPi * rint(a / kTwoPi);
+            cs[j] = cosf((float)a);
+            sn[j] = sinf((float)a);
+        }
+    }
+    const int rows = p.num_heads + p.num_key_heads;
+    for (int r = slot; r < rows; r += rows_per_pass) {
+        const bool is_key = r >= p.num_heads;
+        const int head = is_key ? r - p.num_heads : r;
+        const int64_t off = ((t * (is_key ? p.num_key_heads : p.num_heads) + head) * (int64_t)p.head_dim) + 8 * chunk;
+        const uint4 raw = *reinterpret_cast<const uint4*>((is_key ? p.k : p.q) + off);
+        uint4 res = raw;
+        if (rotate && !(is_key && p.bypass_key)) {
+            half_t x[8], y[8];
+            __builtin_memcpy(x, &raw, 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float x0 = (float)x[2 * j], x1 = (float)x[2 * j + 1];
+                y[2 * j] = (half_t)(x0 * cs[j] - x1 * sn[j]);
+                y[2 * j + 1] = (half_t)(x1 * cs[j] + x0 * sn[j]);
+            }
+            __builtin_memcpy(&res, y, 16);
+        }
+        *reinterpret_cast<uint4*>((is_key ? p.k_out : p.q_out) + off) = res;
+    }
+}
+
+__global__ __launch_bounds__(256) void position_index_kernel(const int64_t* __restrict__ seqstarts,
+                                                             const int64_t* __restrict__ start_pos, int batch,
+                                                             int64_t total, int64_t* __restrict__ out) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    const int b = find_sequence(seqstarts, batch, t);
+    out[t] = start_pos[b] + (t - seqstarts[b]);
+}
+
+pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream) {
+    if (a->total_tokens == 0 || a->batch == 0) return PPLHIP_RC_SUCCESS;
+    RopeParams p;
+    p.q = (const half_t*)a->d_query;
+    p.k = (const half_t*)a->d_key;
+    p.q_out = (half_t*)a->d_rotated_query;
+    p.k_out = (half_t*)a->d_rotated_key;
+    p.seqstarts = a->d_seqstarts;
+    p.start_pos = a->d_start_pos;
+    p.batch = (int32_t)a->batch;
+    p.num_heads = a->num_heads;
+    p.num_key_heads = a->num_key_heads;
+    p.head_dim = a->head_dim;
+    p.rotary_dim = a->rotary_dim == 0 ? a->head_dim : a->rotary_dim;
+    p.bypass_key = a->bypass_key;
+    p.scaling_type = a->scaling_type;
+    p.max_position_embeddings = a->max_position_embeddings;
+    p.log2_theta = log2((double)a->theta);
+    p.scaling_factor = (double)a->scaling_factor;
+    if (a->total_tokens > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "rotary embedding: too many tokens");
+    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a->total_tokens), dim3(256), 0, stream, p);
+    PPLHIP_CHECK_LAUNCH("rotary_position_embedding");
+    return PPLHIP_RC_SUCCESS;
+}
+
+pplhip_retcode launch_position_index(const int64_t* d_seqstarts, const int64_t* d_start_pos, int64_t batch,
+                                     int64_t total_tokens, int64_t* d_out, hipStream_t stream) {
+    if (total_tokens == 0 || batch == 0) return PPLHIP_RC_SUCCESS;
+    const int64_t blocks = (total_tokens + 255) / 256;
+    if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "position index: too many tokens");
+    hipLaunchKernelGGL(position_index_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, d_seqstarts, d_start_pos,
+                       (int)batch, total_tokens, d_out);
+    PPLHIP_CHECK_LAUNCH("position_index");
+    return PPLHIP_RC_SUCCESS;
+}
+
+} // namespace pplhip

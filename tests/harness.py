@@ -134,6 +134,73 @@ def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None):
                 output=out.cpu().view(torch.int16).numpy().view(np.float16))
 
 
+def mha_inputs(b, t):
+    """Packed fp16 key/value of every sequence (history rows then new rows) for MultiHeadAttention."""
+    hs, ss = b.histstarts, b.seqstarts
+    keys, values = [], []
+    for i in range(b.batch):
+        keys += [t["hist_key"][hs[i]:hs[i + 1]], t["current_key"][ss[i]:ss[i + 1]]]
+        values += [t["hist_value"][hs[i]:hs[i + 1]], t["current_value"][ss[i]:ss[i + 1]]]
+    shape = (0, b.num_kv_heads, b.head_dim)
+    cat = lambda xs: np.ascontiguousarray(np.concatenate(xs)) if xs else np.zeros(shape, np.float16)
+    return cat(keys), cat(values)
+
+
+def fill_mha_args(a, b, q, key, value, seqstarts, kvstarts, out, ptr=_ptr):
+    a.d_query, a.d_key, a.d_value, a.d_attn_mask = ptr(q), ptr(key), ptr(value), None
+    a.d_seqstarts, a.d_kvstarts = ptr(seqstarts), ptr(kvstarts)
+    a.is_causal, a.is_alibi = b.is_causal, 0
+    a.batch, a.decoding_batches = b.batch, b.decoding_batches
+    a.max_seqlen, a.max_kvlen = b.max_seqlen, b.max_kvlen
+    a.num_heads, a.num_kv_heads, a.head_dim = b.num_heads, b.num_kv_heads, b.head_dim
+    a.d_output = ptr(out)
+    a._refs = [q, key, value, seqstarts, kvstarts, out]
+    return a
+
+
+def run_oracle_mha(b, q, key, value):
+    import oracle
+    out = np.zeros((b.total_new_tokens, b.num_heads, b.head_dim), np.float16)
+    out64 = np.zeros(out.shape, np.float64)
+    a = fill_mha_args(cabi.MhaArgs(), b, q, key, value, b.seqstarts, b.kvstarts, out)
+    rc = oracle.lib().oracle_mha_forward(C.byref(a), _ptr(out64))
+    assert rc == 0, rc
+    return dict(output=out, output_f64=out64)
+
+
+def run_device_mha(b, q, key, value):
+    import torch
+    lib = pkg.load_library()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    dq, dk, dv = to_dev(q), to_dev(key), to_dev(value)
+    ss, ks = to_dev(b.seqstarts), to_dev(b.kvstarts)
+    out = torch.zeros((b.total_new_tokens, b.num_heads, b.head_dim), dtype=torch.float16, device="cuda")
+    a = fill_mha_args(cabi.MhaArgs(), b, dq, dk, dv, ss, ks, out, ptr=dev_ptr)
+    pkg.check(lib.pplhip_mha_forward(C.byref(a), stream), "mha_forward")
+    torch.cuda.synchronize()
+    return dict(output=out.cpu().view(torch.int16).numpy().view(np.float16))
+
+
+def fill_rope_args(a, q, k, seqlens, start_pos, q_out, k_out, theta=10000.0, rotary_dim=0, bypass_key=0,
+                   scaling_type=0, scaling_factor=1.0, max_pos=2048, ptr=_ptr, tables=None):
+    seqlens = np.asarray(seqlens, np.int64)
+    ss = np.concatenate([[0], np.cumsum(seqlens)]).astype(np.int64)
+    sp = np.asarray(start_pos, np.int64)
+    if tables is not None:  # device copies supplied by the caller
+        ss_arg, sp_arg = tables
+    else:
+        ss_arg, sp_arg = ss, sp
+    a.d_query, a.d_key, a.d_start_pos, a.d_seqstarts = ptr(q), ptr(k), ptr(sp_arg), ptr(ss_arg)
+    a.theta, a.bypass_key, a.rotary_dim = theta, bypass_key, rotary_dim
+    a.batch, a.total_tokens = len(seqlens), int(ss[-1])
+    a.num_heads, a.num_key_heads, a.head_dim = int(q.shape[1]), int(k.shape[1]), int(q.shape[2])
+    a.max_position_embeddings, a.max_seqlen = max_pos, int(seqlens.max()) if len(seqlens) else 0
+    a.scaling_type, a.scaling_factor = scaling_type, scaling_factor
+    a.d_rotated_query, a.d_rotated_key = ptr(q_out), ptr(k_out)
+    a._refs = [q, k, ss_arg, sp_arg, q_out, k_out]
+    return a
+
+
 def assert_attn_close(got_f16, ref_f64, abs_tol=ABS_TOL, rel_tol=REL_TOL, what="attention output"):
     got = got_f16.astype(np.float64)
     assert np.isfinite(got).all(), f"{what}: non-finite values"

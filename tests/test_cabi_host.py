@@ -29,7 +29,8 @@ def test_library_exports_every_declared_symbol(hiplib):
 
 @pytest.mark.parametrize("cname,cls", [("pplhip_mhca_args", cabi.MhcaArgs), ("pplhip_mhca_plan", cabi.MhcaPlan),
                                        ("pplhip_kv_write_args", cabi.KvWriteArgs),
-                                       ("pplhip_kv_cache_args", cabi.KvCacheArgs), ("pplhip_pack_args", cabi.PackArgs)])
+                                       ("pplhip_kv_cache_args", cabi.KvCacheArgs), ("pplhip_pack_args", cabi.PackArgs),
+                                       ("pplhip_mha_args", cabi.MhaArgs), ("pplhip_rope_args", cabi.RopeArgs)])
 def test_ctypes_mirror_matches_header(cname, cls):
     txt = re.sub(r"/\*.*?\*/", "", header_text(), flags=re.S)
     body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), txt, flags=re.S).group(1)
@@ -95,6 +96,55 @@ def test_kv_cache_rejects_like_the_reference_stub(hiplib):
         a.num_repeat = 1
         setattr(a, field, 3)
         assert hiplib.pplhip_kv_cache_forward(C.byref(a), None) == cabi.RC_UNSUPPORTED
+
+
+def test_mha_rejects_like_the_reference_wrapper(hiplib):
+    def args(**kw):
+        a = cabi.MhaArgs()
+        for f in ("d_query", "d_key", "d_value", "d_seqstarts", "d_kvstarts", "d_output"):
+            setattr(a, f, 0x1000)
+        a.is_causal, a.batch, a.max_seqlen, a.max_kvlen = 1, 0, 0, 0  # batch 0: validation only, nothing launched
+        a.num_heads, a.num_kv_heads, a.head_dim = 8, 2, 128
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    assert hiplib.pplhip_mha_forward(C.byref(args()), None) == cabi.RC_SUCCESS
+    # multi_head_attention_kernel.cc:71-74
+    assert hiplib.pplhip_mha_forward(C.byref(args(is_alibi=1)), None) == cabi.RC_UNSUPPORTED
+    assert b"is_alibi" in hiplib.pplhip_last_error()
+    assert hiplib.pplhip_mha_forward(C.byref(args(d_attn_mask=0x1000)), None) == cabi.RC_UNSUPPORTED
+    assert hiplib.pplhip_mha_forward(C.byref(args(head_dim=64)), None) == cabi.RC_UNSUPPORTED
+    assert hiplib.pplhip_mha_forward(C.byref(args(num_kv_heads=3)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_mha_forward(C.byref(args(batch=1, max_seqlen=4, max_kvlen=2)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_mha_forward(C.byref(args(batch=1, max_seqlen=1, max_kvlen=2, d_key=0)), None) == \
+        cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_mha_forward(None, None) == cabi.RC_INVALID_VALUE
+
+
+def test_rope_rejects(hiplib):
+    def args(**kw):
+        a = cabi.RopeArgs()
+        for f in ("d_query", "d_key", "d_start_pos", "d_seqstarts", "d_rotated_query", "d_rotated_key"):
+            setattr(a, f, 0x1000)
+        a.theta, a.batch, a.total_tokens = 10000.0, 0, 0  # batch 0: validation only, nothing launched
+        a.num_heads, a.num_key_heads, a.head_dim, a.scaling_factor = 8, 2, 128, 1.0
+        a.max_position_embeddings = 2048
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    assert hiplib.pplhip_rope_forward(C.byref(args()), None) == cabi.RC_SUCCESS
+    # rotary_position_embedding_kernel.cc:105-108: "invalid scaling type"
+    assert hiplib.pplhip_rope_forward(C.byref(args(scaling_type=3)), None) == cabi.RC_INVALID_VALUE
+    assert b"invalid scaling type" in hiplib.pplhip_last_error()
+    assert hiplib.pplhip_rope_forward(C.byref(args(rotary_dim=12)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_rope_forward(C.byref(args(rotary_dim=256)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_rope_forward(C.byref(args(head_dim=100)), None) == cabi.RC_UNSUPPORTED
+    assert hiplib.pplhip_rope_forward(C.byref(args(theta=0.0)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_rope_forward(C.byref(args(scaling_type=1, scaling_factor=0.0)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_rope_forward(C.byref(args(batch=1, total_tokens=1, d_key=0)), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_position_index(0x1000, 0x1000, -1, 0, 0, 0x1000, None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_position_index(0x1000, 0x1000, 1, 1, 1, None, None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_position_index(0x1000, 0x1000, 0, 0, 0, None, None) == cabi.RC_SUCCESS
 
 
 def test_pack_rejects_bad_slot_count(hiplib):

@@ -204,3 +204,51 @@ def test_pack_tables_random_and_churn(hiplib, olib):
         harness.pkg.check(hiplib.pplhip_advance_slots(dkv.data_ptr(), dnl.data_ptr(), len(kv), None), "advance")
         torch.cuda.synchronize()
         assert np.array_equal(dkv.cpu().numpy(), kv + nl)
+
+
+@pytest.mark.parametrize("causal", [1, 0])
+def test_multi_head_attention_vs_oracle(causal):
+    # decode rows (1 query, long history), chunked rows (kvlen > seqlen), fresh prompts; tiles that straddle 64/128
+    b = workloads.Batch(8, 2, 128, [1, 1, 7, 130, 64, 257], [300, 0, 0, 70, 64, 0], 2, is_causal=causal,
+                        name="mha_mixed")
+    t = workloads.make_tensors(b, seed=31)
+    key, value = harness.mha_inputs(b, t)
+    print(f"case {b.name} causal={causal} S={b.total_new_tokens} KV={int(b.kvstarts[-1])}", flush=True)
+    ref = harness.run_oracle_mha(b, t["query"], key, value)
+    got = harness.run_device_mha(b, t["query"], key, value)
+    harness.assert_attn_close(got["output"], ref["output_f64"], what="MultiHeadAttention output")
+
+
+def test_mhca_equals_mha_over_kv_cache_outputs(hiplib):
+    """The operator identity MultiHeadCacheAttention == MultiHeadAttention o KeyValueCache, all on the device."""
+    import torch
+    b = workloads.Batch(8, 2, 128, [1, 1, 40, 200], [99, 7, 0, 0], 2, name="mhca_identity")
+    t = workloads.make_tensors(b, seed=32)
+    print(f"case {b.name}", flush=True)
+    mhca = harness.run_device(b, t, cache_prefill=1)
+    # KeyValueCache on a fresh slab with the same history, then MultiHeadAttention over its fp16 outputs
+    cache, scale = (harness.to_dev(x) for x in harness.new_slab(b))
+    d = {k: harness.to_dev(v) for k, v in t.items()}
+    tabs = {k: harness.to_dev(v) for k, v in dict(hs=b.histstarts, z=np.zeros(b.batch, np.int64), cs=b.cachestarts,
+                                                  ss=b.seqstarts, ks=b.kvstarts, sp=b.start_pos).items()}
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, d["hist_key"], d["hist_value"], tabs["hs"], tabs["z"],
+                                tabs["cs"], cache, scale, ptr=harness.dev_ptr)
+    harness.pkg.check(hiplib.pplhip_kv_quantize_write(C.byref(w), None), "history write")
+    a = cabi.KvCacheArgs()
+    harness.fill_write_args(a.write, b, d["current_key"], d["current_value"], tabs["ss"], tabs["sp"], tabs["cs"],
+                            cache, scale, ptr=harness.dev_ptr)
+    total_kv = int(b.kvstarts[-1])
+    a.d_kvstarts = harness.dev_ptr(tabs["ks"])
+    a.total_kv_tokens, a.max_kvlen = total_kv, b.max_kvlen
+    a.num_repeat, a.cache_mode, a.cache_layout = 1, 0, 0
+    ko = torch.zeros((total_kv, 2, 128), dtype=torch.float16, device="cuda")
+    vo = torch.zeros_like(ko)
+    a.d_key_out, a.d_value_out = harness.dev_ptr(ko), harness.dev_ptr(vo)
+    harness.pkg.check(hiplib.pplhip_kv_cache_forward(C.byref(a), None), "kv_cache_forward")
+    out = torch.zeros((b.total_new_tokens, 8, 128), dtype=torch.float16, device="cuda")
+    m = harness.fill_mha_args(cabi.MhaArgs(), b, d["query"], ko, vo, tabs["ss"], tabs["ks"], out, ptr=harness.dev_ptr)
+    harness.pkg.check(hiplib.pplhip_mha_forward(C.byref(m), None), "mha_forward")
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), mhca["cache"])
+    via = out.cpu().view(torch.int16).numpy().view(np.float16).astype(np.float64)
+    assert np.abs(via - mhca["output"].astype(np.float64)).max() < 2e-3

@@ -195,3 +195,34 @@ def test_x86_baseline_vs_textbook(olib):
         for h in range(8):
             want = harness.textbook_attention(q[h], k[h], v[h], causal_offset=0)
             assert np.abs(out[h] - want).max() < 2e-5
+
+
+@pytest.mark.parametrize("causal", [1, 0])
+def test_mha_vs_textbook_and_mhca_identity(causal):
+    # explicit K/V with kvlen > seqlen (decode rows, chunked rows) and kvlen == seqlen (fresh prompts)
+    b = workloads.Batch(8, 2, 128, [1, 1, 7, 33, 5], [12, 0, 0, 20, 64], 2, is_causal=causal, name="mha_mixed")
+    t = workloads.make_tensors(b, seed=21)
+    key, value = harness.mha_inputs(b, t)
+    got = harness.run_oracle_mha(b, t["query"], key, value)
+    ss, ks = b.seqstarts, b.kvstarts
+    for i in range(b.batch):
+        L, kv = int(ss[i + 1] - ss[i]), int(ks[i + 1] - ks[i])
+        for h in range(b.num_heads):
+            ref = harness.textbook_attention(t["query"][ss[i]:ss[i + 1], h], key[ks[i]:ks[i + 1], h // 4],
+                                             value[ks[i]:ks[i + 1], h // 4], causal_offset=(kv - L) if causal else None)
+            assert np.abs(got["output_f64"][ss[i]:ss[i + 1], h] - ref).max() < 1e-9
+    # MultiHeadCacheAttention == MultiHeadAttention over the KeyValueCache outputs: feed MHA the de-quantised cache
+    # rows the cache path attends to (cache-prefill on, so every sequence reads the slab)
+    mhca = harness.run_oracle(b, t, cache_prefill=1)
+    import oracle
+    n = int(ks[-1])
+    deq = lambda kv_idx: np.concatenate([
+        (mhca["cache"][b.cachestarts[i]:b.cachestarts[i] + (ks[i + 1] - ks[i]), 0, kv_idx].astype(np.float32).reshape(-1, 2, 16, 8)
+         * mhca["scale"][b.cachestarts[i]:b.cachestarts[i] + (ks[i + 1] - ks[i]), 0, kv_idx].astype(np.float32)[..., None]
+         ).reshape(-1, 2, 128) for i in range(b.batch)]).astype(np.float16)
+    kd, vd = deq(0), deq(1)
+    assert kd.shape == (n, 2, 128)
+    via_mha = harness.run_oracle_mha(b, t["query"], kd, vd)
+    # int8 * fp16 scale is exact in fp32 and, with |q| <= 127, needs at most 18 significant bits: rounding it to
+    # fp16 here is the KeyValueCache op's output rounding, which the cache path does not apply -> small difference
+    assert np.abs(via_mha["output_f64"] - mhca["output_f64"]).max() < 2e-3
