@@ -226,6 +226,16 @@ public:
     BufferDesc& GetBufferDesc() { return buffer_; }
     const BufferDesc& GetBufferDesc() const { return buffer_; }
     bool IsBufferOwner() const { return is_buffer_owner_; }
+    // takes over src's buffer, device and ownership; src is left empty
+    void MoveFrom(BufferInfo* src) {
+        if (src == this) return;
+        FreeBuffer();
+        buffer_ = src->buffer_;
+        device_ = src->device_;
+        is_buffer_owner_ = src->is_buffer_owner_;
+        src->buffer_ = BufferDesc();
+        src->is_buffer_owner_ = false;
+    }
 
 private:
     BufferDesc buffer_;
@@ -262,6 +272,9 @@ public:
         return info_.ReallocBuffer(shape_);
     }
     BufferInfo& GetBufferInfo() { return info_; }
+    // in-place ops hand their input's buffer to the output when they are its last consumer
+    // (TensorImpl::TransferBufferFrom, used at rotary_position_embedding_kernel.cc:66-76)
+    void TransferBufferFrom(TensorImpl* src) { info_.MoveFrom(&src->info_); }
 
 private:
     std::string name_;

@@ -491,6 +491,211 @@ private:
     const opmx::KeyValueCacheParam* param_;
 };
 
+// ---------------------------------------------------------------- MultiHeadAttention (no cache)
+class DynamicBatchingMultiHeadAttentionKernel final : public LlmHipKernel {
+public:
+    DynamicBatchingMultiHeadAttentionKernel(const ir::Node* node, const EngineConfig* cfg,
+                                            const opmx::MultiHeadAttentionParam* p)
+        : LlmHipKernel(node, cfg), param_(p) {}
+    RetCode Reshape(InputOutputInfo* info) const override { return GenericInferDims(info); }
+
+protected:
+    // inputs, checks and argument order of multi_head_attention_kernel.cc:24-128
+    RetCode DoExecute(KernelExecContext* ctx) override {
+        REQUIRED_INPUT(query, 0);
+        REQUIRED_INPUT(key, 1);
+        REQUIRED_INPUT(value, 2);
+        REQUIRED_INPUT(seqstarts, 3);
+        REQUIRED_INPUT(kvstarts, 4);
+        REQUIRED_INPUT(decoding_batches, 5);
+        REQUIRED_INPUT(max_seqlen, 6);
+        REQUIRED_INPUT(max_kvlen, 7);
+        OPTIONAL_INPUT(attn_mask, 8);
+        REQUIRED_OUTPUT(attn_output, 0);
+
+        auto rc = Reshape(ctx);
+        if (rc != RC_SUCCESS) return rc;
+        REALLOC_TENSOR_BUFFER(attn_output);
+        if (param_->is_alibi) {
+            LOG(ERROR) << "currently only support is_alibi == false";
+            return RC_UNSUPPORTED;
+        }
+        int64_t decoding_batches_val = 0, max_seqlen_val = 0, max_kvlen_val = 0;
+        if (ReadScalar(decoding_batches, &decoding_batches_val) != RC_SUCCESS) {
+            LOG(ERROR) << "decoding_batches->CopyToHost() failed";
+            return RC_DEVICE_MEMORY_ERROR;
+        }
+        if (ReadScalar(max_seqlen, &max_seqlen_val) != RC_SUCCESS) {
+            LOG(ERROR) << "max_seqlen->CopyToHost() failed";
+            return RC_DEVICE_MEMORY_ERROR;
+        }
+        if (ReadScalar(max_kvlen, &max_kvlen_val) != RC_SUCCESS) {
+            LOG(ERROR) << "max_kvlen->CopyToHost() failed";
+            return RC_DEVICE_MEMORY_ERROR;
+        }
+        void* attn_mask_data = nullptr;
+        if (attn_mask && attn_mask->GetShape()->CalcElementsExcludingPadding() > 0) attn_mask_data = attn_mask->GetBufferPtr();
+
+        pplhip_mha_args a;
+        memset(&a, 0, sizeof(a));
+        a.d_query = query->GetBufferPtr();
+        a.d_key = key->GetBufferPtr();
+        a.d_value = value->GetBufferPtr();
+        a.d_attn_mask = attn_mask_data;
+        a.d_seqstarts = seqstarts->GetBufferPtr<int64_t>();
+        a.d_kvstarts = kvstarts->GetBufferPtr<int64_t>();
+        a.is_causal = param_->is_causal;
+        a.is_alibi = param_->is_alibi;
+        a.batch = (int64_t)seqstarts->GetShape()->GetDim(0) - 1;
+        a.decoding_batches = decoding_batches_val;
+        a.max_seqlen = max_seqlen_val;
+        a.max_kvlen = max_kvlen_val;
+        a.num_heads = param_->num_heads;
+        a.num_kv_heads = param_->num_kv_heads;
+        a.head_dim = param_->head_dim;
+        a.d_output = attn_output->GetBufferPtr();
+        return (RetCode)CheckKernelRc(pplhip_mha_forward(&a, GetStream()), GetName());
+    }
+
+private:
+    const opmx::MultiHeadAttentionParam* param_;
+};
+
+// ---------------------------------------------------------------- RotaryPositionEmbedding
+class DynamicBatchingRotaryPositionEmbeddingKernel final : public LlmHipKernel {
+public:
+    DynamicBatchingRotaryPositionEmbeddingKernel(const ir::Node* node, const EngineConfig* cfg,
+                                                 const opmx::RotaryPositionEmbeddingParam* p)
+        : LlmHipKernel(node, cfg), param_(p) {}
+    // oputils/opmx/reshape_rotary_position_embedding.cc:26-35
+    RetCode Reshape(InputOutputInfo* info) const override {
+        for (uint32_t i = 0; i < 2; ++i) {
+            auto in = info->GetInput<TensorImpl>(i);
+            auto out = info->GetOutput<TensorImpl>(i);
+            if (!in || !out) return RC_NOT_FOUND;
+            out->GetShape()->Reshape(in->GetShape()->GetDims(), in->GetShape()->GetDimCount());
+            out->GetShape()->SetDataType(in->GetShape()->GetDataType());
+        }
+        return RC_SUCCESS;
+    }
+
+protected:
+    // rotary_position_embedding_kernel.cc:24-133
+    RetCode DoExecute(KernelExecContext* ctx) override {
+        REQUIRED_INPUT(query, 0);
+        REQUIRED_INPUT(key, 1);
+        REQUIRED_INPUT(seqstarts, 2);
+        REQUIRED_INPUT(start_pos, 3);
+        REQUIRED_INPUT(max_seqlen, 4);
+        REQUIRED_OUTPUT(rotated_query, 0);
+        REQUIRED_OUTPUT(rotated_key, 1);
+
+        auto rc = Reshape(ctx);
+        if (rc != RC_SUCCESS) return rc;
+        // an input this kernel is the last consumer of gives its buffer to the output (the rotation is in place)
+        void* query_data = query->GetBufferPtr();
+        void* key_data = key->GetBufferPtr();
+        if (ctx->IsLastConsumerOfInput(0) && query->GetBufferInfo().IsBufferOwner()) {
+            rotated_query->TransferBufferFrom(query);
+        } else {
+            REALLOC_TENSOR_BUFFER(rotated_query);
+        }
+        if (ctx->IsLastConsumerOfInput(1) && key->GetBufferInfo().IsBufferOwner()) {
+            rotated_key->TransferBufferFrom(key);
+        } else {
+            REALLOC_TENSOR_BUFFER(rotated_key);
+        }
+        auto query_shape = rotated_query->GetShape();
+        auto key_shape = rotated_key->GetShape();
+        if (DATATYPE_FLOAT16 != query_shape->GetDataType()) {
+            LOG(ERROR) << "currently only support fp16";
+            return RC_UNSUPPORTED;
+        }
+        int64_t max_seqlen_val = 0;
+        if (ReadScalar(max_seqlen, &max_seqlen_val) != RC_SUCCESS) {
+            LOG(ERROR) << "max_seqlen->CopyToHost() failed";
+            return RC_DEVICE_MEMORY_ERROR;
+        }
+        // The reference maps the parameter through `!=` tests (rotary_position_embedding_kernel.cc:99-108), which
+        // turns NONE into LINEAR and LINEAR / DYNAMIC into NONE; the value is taken at its name here.
+        int32_t scaling_type;
+        if (param_->scaling_type == param_->SCALING_TYPE_NONE) {
+            scaling_type = PPLHIP_ROPE_SCALING_NONE;
+        } else if (param_->scaling_type == param_->SCALING_TYPE_LINEAR) {
+            scaling_type = PPLHIP_ROPE_SCALING_LINEAR;
+        } else if (param_->scaling_type == param_->SCALING_TYPE_DYNAMIC) {
+            scaling_type = PPLHIP_ROPE_SCALING_DYNAMIC;
+        } else {
+            LOG(ERROR) << "invalid scaling type: " << param_->scaling_type;
+            return RC_INVALID_VALUE;
+        }
+        pplhip_rope_args a;
+        memset(&a, 0, sizeof(a));
+        a.d_query = query_data;
+        a.d_key = key_data;
+        a.d_start_pos = start_pos->GetBufferPtr<int64_t>();
+        a.d_seqstarts = seqstarts->GetBufferPtr<int64_t>();
+        a.theta = param_->theta;
+        a.bypass_key = param_->bypass_key;
+        a.head_dim = (int32_t)query_shape->GetDim(2);
+        a.rotary_dim = param_->rotary_dim == 0 ? a.head_dim : param_->rotary_dim;
+        a.batch = start_pos->GetShape()->GetDim(0);
+        a.total_tokens = query_shape->GetDim(0);
+        a.num_heads = (int32_t)query_shape->GetDim(1);
+        a.num_key_heads = (int32_t)key_shape->GetDim(1);
+        a.max_position_embeddings = param_->max_position_embeddings;
+        a.max_seqlen = max_seqlen_val;
+        a.scaling_type = scaling_type;
+        a.scaling_factor = param_->scaling_factor;
+        a.d_rotated_query = rotated_query->GetBufferPtr();
+        a.d_rotated_key = rotated_key->GetBufferPtr();
+        return (RetCode)CheckKernelRc(pplhip_rope_forward(&a, GetStream()), GetName());
+    }
+
+private:
+    const opmx::RotaryPositionEmbeddingParam* param_;
+};
+
+// ---------------------------------------------------------------- PositionIndex
+class DynamicBatchingPositionIndexKernel final : public LlmHipKernel {
+public:
+    DynamicBatchingPositionIndexKernel(const ir::Node* node, const EngineConfig* cfg) : LlmHipKernel(node, cfg) {}
+    RetCode Reshape(InputOutputInfo* info) const override { return GenericInferDims(info); }
+
+protected:
+    // position_index_kernel.cc:24-70
+    RetCode DoExecute(KernelExecContext* ctx) override {
+        REQUIRED_INPUT(sequence, 0);
+        REQUIRED_INPUT(seqstarts, 1);
+        REQUIRED_INPUT(start_pos, 2);
+        REQUIRED_INPUT(max_seqlen, 3);
+        REQUIRED_OUTPUT(position_idx, 0);
+
+        auto rc = Reshape(ctx);
+        if (rc != RC_SUCCESS) return rc;
+        if (ctx->IsLastConsumerOfInput(0) && sequence->GetBufferInfo().IsBufferOwner()) {
+            position_idx->TransferBufferFrom(sequence);
+        } else {
+            REALLOC_TENSOR_BUFFER(position_idx);
+        }
+        if (DATATYPE_INT64 != position_idx->GetShape()->GetDataType()) {
+            LOG(ERROR) << "position_idx takes the type of the token sequence, which must be int64";
+            return RC_UNSUPPORTED;
+        }
+        int64_t max_seqlen_val = 0;
+        if (ReadScalar(max_seqlen, &max_seqlen_val) != RC_SUCCESS) {
+            LOG(ERROR) << "max_seqlen->CopyToHost() failed";
+            return RC_DEVICE_MEMORY_ERROR;
+        }
+        const int64_t batch = start_pos->GetShape()->GetDim(0);
+        const int64_t total = (int64_t)position_idx->GetShape()->CalcElementsExcludingPadding();
+        return (RetCode)CheckKernelRc(
+            pplhip_position_index(start_pos->GetBufferPtr<int64_t>(), seqstarts->GetBufferPtr<int64_t>(), batch, total,
+                                  max_seqlen_val, position_idx->GetBufferPtr<int64_t>(), GetStream()),
+            GetName());
+    }
+};
+
 // ---------------------------------------------------------------- ops + registry
 class LlmHipOptKernel : public OptKernel {
 public:
@@ -541,6 +746,46 @@ private:
     std::shared_ptr<opmx::KeyValueCacheParam> param_;
 };
 
+class DynamicBatchingMultiHeadAttentionOp final : public LlmHipOptKernel {
+public:
+    using LlmHipOptKernel::LlmHipOptKernel;
+    RetCode Init(const ir::Graph* graph, const EngineConfig* cfg) override {
+        cfg_ = cfg;
+        return GenericLoadParam(graph, &param_);
+    }
+    KernelImpl* CreateKernelImpl() const override {
+        return new DynamicBatchingMultiHeadAttentionKernel(GetNode(), cfg_, param_.get());
+    }
+
+private:
+    std::shared_ptr<opmx::MultiHeadAttentionParam> param_;
+};
+
+class DynamicBatchingRotaryPositionEmbeddingOp final : public LlmHipOptKernel {
+public:
+    using LlmHipOptKernel::LlmHipOptKernel;
+    RetCode Init(const ir::Graph* graph, const EngineConfig* cfg) override {
+        cfg_ = cfg;
+        return GenericLoadParam(graph, &param_);
+    }
+    KernelImpl* CreateKernelImpl() const override {
+        return new DynamicBatchingRotaryPositionEmbeddingKernel(GetNode(), cfg_, param_.get());
+    }
+
+private:
+    std::shared_ptr<opmx::RotaryPositionEmbeddingParam> param_;
+};
+
+class DynamicBatchingPositionIndexOp final : public LlmHipOptKernel { // no attributes (position_index_op.cc:29-41)
+public:
+    using LlmHipOptKernel::LlmHipOptKernel;
+    RetCode Init(const ir::Graph*, const EngineConfig* cfg) override {
+        cfg_ = cfg;
+        return RC_SUCCESS;
+    }
+    KernelImpl* CreateKernelImpl() const override { return new DynamicBatchingPositionIndexKernel(GetNode(), cfg_); }
+};
+
 typedef LlmHipOptKernel* (*OptKernelCreator)(const ir::Node*);
 
 utils::OpInfoManager<OptKernelCreator>& OptKernelCreatorManager() {
@@ -568,6 +813,9 @@ static void RegisterResourcesOnce() { // default_register_resources.cc:28-34
     std::call_once(once, [] {
         RegisterOptKernelCreator<DynamicBatchingKeyValueCacheOp>("opmx.dynamic_batching", "KeyValueCache", 1, 1);
         RegisterOptKernelCreator<DynamicBatchingMultiHeadCacheAttentionOp>("opmx.dynamic_batching", "MultiHeadCacheAttention", 1, 1);
+        RegisterOptKernelCreator<DynamicBatchingMultiHeadAttentionOp>("opmx.dynamic_batching", "MultiHeadAttention", 1, 1);
+        RegisterOptKernelCreator<DynamicBatchingPositionIndexOp>("opmx.dynamic_batching", "PositionIndex", 1, 1);
+        RegisterOptKernelCreator<DynamicBatchingRotaryPositionEmbeddingOp>("opmx.dynamic_batching", "RotaryPositionEmbedding", 1, 1);
     });
 }
 

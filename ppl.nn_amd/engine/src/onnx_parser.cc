@@ -270,6 +270,44 @@ RetCode ParseKeyValueCacheParam(const PbNode& pb, const std::string& node_name, 
     return RC_SUCCESS;
 }
 
+// models/onnx/parsers/opmx/parse_multi_head_attention_param.cc:10-31
+RetCode ParseMultiHeadAttentionParam(const PbNode& pb, const std::string& node_name, ir::Attr* arg) {
+    auto param = static_cast<opmx::MultiHeadAttentionParam*>(arg);
+    if (!GetNodeAttr(pb, "num_heads", &param->num_heads, -1)) { LOG(ERROR) << node_name << ": missing num_heads"; return RC_INVALID_VALUE; }
+    if (!GetNodeAttr(pb, "head_dim", &param->head_dim, -1)) { LOG(ERROR) << node_name << ": missing head_dim"; return RC_INVALID_VALUE; }
+    int32_t is_causal, is_alibi;
+    GetNodeAttr(pb, "is_causal", &is_causal, 1);
+    param->is_causal = is_causal;
+    GetNodeAttr(pb, "is_alibi", &is_alibi, 0);
+    param->is_alibi = is_alibi;
+    GetNodeAttr(pb, "num_kv_heads", &param->num_kv_heads, param->num_heads);
+    return RC_SUCCESS;
+}
+
+// models/onnx/parsers/opmx/parse_rotary_position_embedding_param.cc:10-41
+RetCode ParseRotaryPositionEmbeddingParam(const PbNode& pb, const std::string& node_name, ir::Attr* arg) {
+    auto param = static_cast<opmx::RotaryPositionEmbeddingParam*>(arg);
+    if (!GetNodeAttr(pb, "theta", &param->theta, -1.0f)) { LOG(ERROR) << node_name << ": missing theta"; return RC_INVALID_VALUE; }
+    GetNodeAttr(pb, "bypass_key", &param->bypass_key, 0);
+    GetNodeAttr(pb, "rotary_dim", &param->rotary_dim, 0);
+    GetNodeAttr(pb, "scaling_factor", &param->scaling_factor, 1.0f);
+    GetNodeAttr(pb, "max_position_embeddings", &param->max_position_embeddings, 2048);
+    std::string scaling_type;
+    for (auto& a : pb.attrs)
+        if (a.name == "scaling_type") scaling_type = a.s;
+    if (scaling_type == "") {
+        param->scaling_type = opmx::RotaryPositionEmbeddingParam::SCALING_TYPE_NONE;
+    } else if (scaling_type == "linear") {
+        param->scaling_type = opmx::RotaryPositionEmbeddingParam::SCALING_TYPE_LINEAR;
+    } else if (scaling_type == "dynamic") {
+        param->scaling_type = opmx::RotaryPositionEmbeddingParam::SCALING_TYPE_DYNAMIC;
+    } else {
+        LOG(ERROR) << "unsupported scaling_type: " << scaling_type;
+        return RC_UNSUPPORTED;
+    }
+    return RC_SUCCESS;
+}
+
 utils::OpInfoManager<ParserInfo>& ParamParserManager() {
     static utils::OpInfoManager<ParserInfo> mgr;
     static std::once_flag once;
@@ -285,6 +323,11 @@ utils::OpInfoManager<ParserInfo>& ParamParserManager() {
             {[] { return std::make_shared<opmx::MultiHeadCacheAttentionParam>(); }, ParseMultiHeadCacheAttentionParam});
         reg("opmx.dynamic_batching", "KeyValueCache", 1, 1,
             {[] { return std::make_shared<opmx::KeyValueCacheParam>(); }, ParseKeyValueCacheParam});
+        reg("opmx.dynamic_batching", "MultiHeadAttention", 1, 1,
+            {[] { return std::make_shared<opmx::MultiHeadAttentionParam>(); }, ParseMultiHeadAttentionParam});
+        reg("opmx.dynamic_batching", "RotaryPositionEmbedding", 1, 1,
+            {[] { return std::make_shared<opmx::RotaryPositionEmbeddingParam>(); }, ParseRotaryPositionEmbeddingParam});
+        reg("opmx.dynamic_batching", "PositionIndex", 1, 1, {nullptr, nullptr}); // no attributes
     });
     return mgr;
 }

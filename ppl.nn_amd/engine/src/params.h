@@ -1,10 +1,14 @@
 // Op parameter structs, field for field as in the reference:
 //   src/ppl/nn/params/opmx/multi_head_cache_attention_param.h:10-38
 //   src/ppl/nn/params/opmx/key_value_cache_param.h:10-30
+//   src/ppl/nn/params/opmx/multi_head_attention_param.h:10-26
+//   src/ppl/nn/params/opmx/rotary_position_embedding_param.h:10-36
 #ifndef PPLNN_LLM_HIP_PARAMS_H_
 #define PPLNN_LLM_HIP_PARAMS_H_
 
 #include "core.h"
+
+#include <cmath>
 
 namespace ppl { namespace nn { namespace opmx {
 
@@ -42,6 +46,34 @@ struct KeyValueCacheParam final : public ir::Attr {
         return num_layer == p.num_layer && layer_idx == p.layer_idx && quant_bit == p.quant_bit &&
             quant_group == p.quant_group && num_repeat == p.num_repeat && cache_mode == p.cache_mode &&
             cache_layout == p.cache_layout && (cache_mode == 0 || page_size == p.page_size);
+    }
+};
+
+struct MultiHeadAttentionParam final : public ir::Attr {
+    int32_t num_heads = 0;
+    int32_t num_kv_heads = 0;
+    int32_t head_dim = 0;
+    bool is_causal = true;
+    bool is_alibi = false;
+    bool operator==(const MultiHeadAttentionParam& p) const {
+        return num_heads == p.num_heads && num_kv_heads == p.num_kv_heads && head_dim == p.head_dim &&
+            is_causal == p.is_causal && is_alibi == p.is_alibi;
+    }
+};
+
+struct RotaryPositionEmbeddingParam final : public ir::Attr {
+    enum { SCALING_TYPE_NONE = 0, SCALING_TYPE_LINEAR = 1, SCALING_TYPE_DYNAMIC = 2 };
+    int32_t bypass_key = 0;
+    int32_t rotary_dim = 0;
+    float theta = 10000.0f;
+    int32_t max_position_embeddings = 2048;
+    int32_t scaling_type = SCALING_TYPE_NONE;
+    float scaling_factor = 1.0f;
+    bool operator==(const RotaryPositionEmbeddingParam& p) const {
+        return bypass_key == p.bypass_key && fabs(theta - p.theta) <= 1e-05 && rotary_dim == p.rotary_dim &&
+            scaling_type == p.scaling_type &&
+            (scaling_type == SCALING_TYPE_NONE || max_position_embeddings == p.max_position_embeddings) &&
+            (scaling_type == SCALING_TYPE_NONE || fabs(scaling_factor - p.scaling_factor) <= 1e-05);
     }
 };
 

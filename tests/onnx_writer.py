@@ -105,3 +105,82 @@ def kv_cache_model(num_layer, layer_idx, extra_attrs=()):
     ins = [value_info(x, types.get(x, INT64), ["d%d" % i for i in range(ranks[x])]) for x in KVC_INPUTS]
     outs = [value_info("key", FLOAT16, ["t", "h", "d"]), value_info("value", FLOAT16, ["t", "h", "d"])]
     return model([n], ins, outs, [("", 11), ("opmx.dynamic_batching", 1)])
+
+
+def attr_string(name, v):
+    return _str(1, name) + _ld(4, v.encode()) + _int(20, 3)
+
+
+DB = "opmx.dynamic_batching"
+_TYPES = {"query": FLOAT16, "key": FLOAT16, "value": FLOAT16, "current_key": FLOAT16, "current_value": FLOAT16,
+          "cache": INT8, "scale": FLOAT16}
+_RANKS = {"query": 3, "key": 3, "value": 3, "current_key": 3, "current_value": 3, "seqstarts": 1, "kvstarts": 1,
+          "cachestarts": 1, "start_pos": 1, "decoding_batches": 0, "max_seqlen": 0, "max_kvlen": 0, "cache": 5,
+          "scale": 5, "sequence": 1}
+
+
+def _inputs(names):
+    return [value_info(x, _TYPES.get(x, INT64), ["d%d" % i for i in range(_RANKS[x])]) for x in names]
+
+
+def rope_attrs(theta=10000.0, drop_theta=False, scaling_type=None, **ints):
+    attrs = [] if drop_theta else [attr_float("theta", theta)]
+    attrs += [attr_float(k, v) if isinstance(v, float) else attr_int(k, v) for k, v in ints.items()]
+    if scaling_type is not None:
+        attrs.append(attr_string("scaling_type", scaling_type))
+    return attrs
+
+
+def rope_model(attrs):
+    names = ["query", "key", "seqstarts", "start_pos", "max_seqlen"]
+    n = node("RotaryPositionEmbedding", names, ["rotated_query", "rotated_key"], name="rope", domain=DB, attrs=attrs)
+    outs = [value_info("rotated_query", FLOAT16, ["s", "h", "d"]), value_info("rotated_key", FLOAT16, ["s", "h", "d"])]
+    return model([n], _inputs(names), outs, [("", 11), (DB, 1)])
+
+
+ROPE_MHCA_INPUTS = ["query", "key", "current_value", "seqstarts", "kvstarts", "cachestarts", "start_pos",
+                    "decoding_batches", "max_seqlen", "max_kvlen", "cache", "scale"]
+
+
+def rope_mhca_model(num_heads, num_kv_heads, head_dim, num_layer, layer_idx, theta):
+    """RotaryPositionEmbedding feeding MultiHeadCacheAttention: rotated_query / rotated_key are intermediate tensors."""
+    rope = node("RotaryPositionEmbedding", ["query", "key", "seqstarts", "start_pos", "max_seqlen"],
+                ["rotated_query", "rotated_key"], name="rope", domain=DB, attrs=rope_attrs(theta))
+    attrs = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, num_layer=num_layer,
+                 layer_idx=layer_idx, quant_bit=8, quant_group=8)
+    attn = node("MultiHeadCacheAttention",
+                ["rotated_query", "rotated_key"] + ROPE_MHCA_INPUTS[2:], ["attn_output"], name="attn", domain=DB,
+                attrs=[attr_int(k, v) for k, v in attrs.items()])
+    outs = [value_info("attn_output", FLOAT16, ["s", "h", "d"])]
+    return model([rope, attn], _inputs(ROPE_MHCA_INPUTS), outs, [("", 11), (DB, 1)])
+
+
+KVC_MHA_INPUTS = ["query", "current_key", "current_value", "seqstarts", "kvstarts", "cachestarts", "start_pos",
+                  "decoding_batches", "max_seqlen", "max_kvlen", "cache", "scale"]
+
+
+def kv_cache_mha_model(num_heads, num_kv_heads, head_dim, num_layer, layer_idx, mha_extra=()):
+    """KeyValueCache feeding MultiHeadAttention: the two-op spelling of MultiHeadCacheAttention."""
+    kvc = node("KeyValueCache", KVC_INPUTS, ["key", "value"], name="kvcache", domain=DB,
+               attrs=[attr_int(k, v) for k, v in dict(num_layer=num_layer, layer_idx=layer_idx, quant_bit=8,
+                                                      quant_group=8).items()])
+    attrs = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim)
+    attrs.update(dict(mha_extra))
+    mha = node("MultiHeadAttention", ["query", "key", "value", "seqstarts", "kvstarts", "decoding_batches", "max_seqlen",
+                                      "max_kvlen"], ["attn_output"], name="mha", domain=DB,
+               attrs=[attr_int(k, v) for k, v in attrs.items()])
+    outs = [value_info("attn_output", FLOAT16, ["s", "h", "d"])]
+    return model([kvc, mha], _inputs(KVC_MHA_INPUTS), outs, [("", 11), (DB, 1)])
+
+
+def mha_model(attrs):
+    names = ["query", "key", "value", "seqstarts", "kvstarts", "decoding_batches", "max_seqlen", "max_kvlen"]
+    n = node("MultiHeadAttention", names, ["attn_output"], name="mha", domain=DB,
+             attrs=[attr_int(k, v) for k, v in attrs.items()])
+    return model([n], _inputs(names), [value_info("attn_output", FLOAT16, ["s", "h", "d"])], [("", 11), (DB, 1)])
+
+
+def position_index_model():
+    names = ["sequence", "seqstarts", "start_pos", "max_seqlen"]
+    n = node("PositionIndex", names, ["position_idx"], name="posidx", domain=DB)
+    return model([n], _inputs(names), [value_info("position_idx", INT64, ["s"])], [("", 11), (DB, 1)])

@@ -124,3 +124,38 @@ def test_engine_configure_like_the_reference(eng):
     assert eng.pplnn_hip_engine_configure_u32(e, 1006, 0) == cabi.RC_INVALID_VALUE
     eng.pplnn_hip_engine_destroy(e)
     assert not eng.pplnn_hip_engine_create(0, 99)  # unknown mm_policy: factories return nullptr on failure
+
+
+def test_new_ops_load_and_preprocess(eng):
+    e = eng.pplnn_hip_engine_create(0, 1)
+    for m in (ow.rope_model(ow.rope_attrs(500000.0, rotary_dim=64, bypass_key=1, scaling_type="linear",
+                                          scaling_factor=2.0)),
+              ow.rope_model(ow.rope_attrs(10000.0, scaling_type="dynamic", max_position_embeddings=4096)),
+              ow.mha_model(dict(num_heads=32, head_dim=128, num_kv_heads=8)),
+              ow.position_index_model(),
+              ow.rope_mhca_model(32, 8, 128, 2, 1, 10000.0),
+              ow.kv_cache_mha_model(32, 8, 128, 2, 1)):
+        b, rc = _load(eng, m)
+        assert rc == 0, eng.pplnn_hip_last_error()
+        assert eng.pplnn_hip_builder_set_engine(b, e) == 0
+        assert eng.pplnn_hip_builder_preprocess(b) == 0, eng.pplnn_hip_last_error()
+        eng.pplnn_hip_builder_destroy(b)
+    eng.pplnn_hip_engine_destroy(e)
+
+
+def test_rope_and_mha_attr_errors(eng):
+    # parse_rotary_position_embedding_param.cc:13-16: theta is required
+    b, rc = _load(eng, ow.rope_model(ow.rope_attrs(drop_theta=True)))
+    assert rc == cabi.RC_INVALID_VALUE and b"theta" in eng.pplnn_hip_last_error()
+    eng.pplnn_hip_builder_destroy(b)
+    # :26-37: unknown scaling_type string
+    b, rc = _load(eng, ow.rope_model(ow.rope_attrs(10000.0, scaling_type="yarn")))
+    assert rc == cabi.RC_UNSUPPORTED and b"scaling_type" in eng.pplnn_hip_last_error()
+    eng.pplnn_hip_builder_destroy(b)
+    # parse_multi_head_attention_param.cc:13-21
+    for missing in ("num_heads", "head_dim"):
+        attrs = dict(num_heads=8, head_dim=128)
+        attrs.pop(missing)
+        b, rc = _load(eng, ow.mha_model(attrs))
+        assert rc == cabi.RC_INVALID_VALUE and missing.encode() in eng.pplnn_hip_last_error()
+        eng.pplnn_hip_builder_destroy(b)

@@ -187,3 +187,87 @@ def test_kv_cache_graph_through_the_engine(hiplib, olib):
     assert key.shape == ko.shape  # dim 0 = kvstarts[B], read back like reshape_dynamic_batching_key_value_cache.cc:43-53
     assert np.array_equal(key.view(np.uint16), ko.view(np.uint16)) and np.array_equal(value.view(np.uint16), vo.view(np.uint16))
     s.close()
+
+
+def _rope_on_oracle(olib, q, k, b, theta):
+    qo, ko = np.zeros_like(q), np.zeros_like(k)
+    a = harness.fill_rope_args(cabi.RopeArgs(), q, k, b.seqlens, b.start_pos, qo, ko, theta=theta)
+    assert olib.oracle_rope_forward(C.byref(a)) == 0
+    return qo, ko
+
+
+def test_rope_then_mhca_graph(hiplib, olib):
+    """Two nodes: RotaryPositionEmbedding -> MultiHeadCacheAttention; rotated_query / rotated_key are intermediate
+    tensors of the runtime (allocated from the engine's arena, released after the attention node)."""
+    import torch
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(8, 2, 128, [1, 1, 50, 131], [700, 12, 0, 0], 2, num_layer=1, layer_idx=0, name="engine_rope_mhca")
+    t = workloads.make_tensors(b, seed=41)
+    theta = 500000.0
+    # oracle: rotate, then attend (the rotated fp16 tensors are what the attention node sees)
+    rq, rk = _rope_on_oracle(olib, t["query"], t["current_key"], b, theta)
+    t_rot = dict(t, query=rq, current_key=rk)
+    ref = harness.run_oracle(b, t_rot)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    s = Session(eng, ow.rope_mhca_model(8, 2, 128, 1, 0, theta))
+    assert eng.pplnn_hip_runtime_input_count(s.rt) == 12
+    s.set_device_tensor(0, harness.to_dev(t["query"]))
+    s.set_device_tensor(1, harness.to_dev(t["current_key"]))
+    s.set_device_tensor(2, harness.to_dev(t["current_value"]))
+    for i, tab in zip(range(3, 7), (b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)):
+        s.set_table(i, tab)
+    for i, v in zip(range(7, 10), (b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+        s.set_host_scalar(i, v)
+    s.set_device_tensor(10, cache)
+    s.set_device_tensor(11, scale)
+    for _ in range(2):
+        assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+        out = s.output(0, np.float16)
+        # the rotated inputs may differ from the oracle's by one fp16 ulp -> same attention tolerance still holds
+        harness.assert_attn_close(out, ref["output_f64"], abs_tol=3e-3)
+    torch.cuda.synchronize()
+    # the K rows written to the slab are the ROTATED keys
+    cache_h = cache.cpu().numpy()
+    diff = np.abs(cache_h.astype(np.int32) - ref["cache"].astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.02  # one-ulp differences of the rotation move few int8 codes
+    s.close()
+
+
+def test_kv_cache_then_mha_graph_equals_mhca(hiplib):
+    import torch
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(8, 2, 128, [1, 1, 40, 200], [99, 7, 0, 0], 2, num_layer=2, layer_idx=1, name="engine_kvc_mha")
+    t = workloads.make_tensors(b, seed=42)
+    mhca = harness.run_device(b, t, cache_prefill=1)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    s = Session(eng, ow.kv_cache_mha_model(8, 2, 128, 2, 1))
+    s.set_device_tensor(0, harness.to_dev(t["query"]))
+    s.set_device_tensor(1, harness.to_dev(t["current_key"]))
+    s.set_device_tensor(2, harness.to_dev(t["current_value"]))
+    for i, tab in zip(range(3, 7), (b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)):
+        s.set_table(i, tab)
+    for i, v in zip(range(7, 10), (b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+        s.set_host_scalar(i, v)
+    s.set_device_tensor(10, cache)
+    s.set_device_tensor(11, scale)
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    out = s.output(0, np.float16)
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), mhca["cache"])
+    assert np.abs(out.astype(np.float64) - mhca["output"].astype(np.float64)).max() < 2e-3
+    s.close()
+
+
+def test_position_index_graph(hiplib):
+    eng = harness.pkg.load_engine_library()
+    seqlens, start = np.array([1, 9, 1, 30], np.int64), np.array([70, 0, 5, 100], np.int64)
+    ss = np.concatenate([[0], np.cumsum(seqlens)]).astype(np.int64)
+    s = Session(eng, ow.position_index_model())
+    s.set_table(0, np.arange(int(ss[-1]), dtype=np.int64))  # token ids: only the shape and type matter
+    s.set_table(1, ss)
+    s.set_table(2, start)
+    s.set_host_scalar(3, int(seqlens.max()))
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    out = s.output(0, np.int64)
+    assert np.array_equal(out, np.concatenate([p + np.arange(n) for n, p in zip(seqlens, start)]))
+    s.close()
