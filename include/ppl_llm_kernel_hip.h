@@ -55,7 +55,11 @@ int32_t pplhip_version(void);
  *   current_value fp16 [S, num_kv_heads, head_dim]
  *   seqstarts     i64  [batch+1]   prefix sums of new-token counts, seqstarts[0] = 0
  *   kvstarts      i64  [batch+1]   prefix sums of kv lengths (start_pos + seqlen), kvstarts[0] = 0
- *   cachestarts   i64  [batch]     first slab token of each sequence (cache_mode 0)
+ *   cachestarts   i64  [batch]     first slab token of each sequence (cache_mode 0), or
+ *                      [batch, cachestart_stride_b] first slab token of every PAGE of each sequence (cache_mode 1):
+ *                      token j of sequence b lives at slab token cachestarts[b][j / page_size] + j % page_size
+ *                      (page table laid out as in tools/benchmark_llama/generation_state.cc:111-117);
+ *                      page_size must be a power of two >= 64
  *   start_pos     i64  [batch]     tokens already cached before this call
  *   cache         i8   element (tok, layer, kv, head, d) at
  *                      tok*cache_stride_s + layer*cache_stride_l + kv*cache_stride_kv + head*cache_stride_h + d
@@ -85,7 +89,7 @@ typedef struct pplhip_mhca_args {
     int32_t num_heads;
     int32_t num_kv_heads;
     int32_t head_dim;
-    int32_t cache_mode; /* 0 = contiguous region per sequence; 1 (paged) is rejected for now */
+    int32_t cache_mode; /* 0 = contiguous region per sequence; 1 = paged (see cachestarts above) */
     int32_t page_size;
     int64_t cache_stride_s;
     int64_t cache_stride_l;
@@ -153,6 +157,9 @@ typedef struct pplhip_kv_write_args {
     int64_t cache_stride_kv;
     void* d_cache;
     void* d_scale;
+    int32_t cache_mode; /* as in pplhip_mhca_args */
+    int32_t page_size;
+    int64_t cachestart_stride_b;
 } pplhip_kv_write_args;
 
 pplhip_retcode pplhip_kv_quantize_write(const pplhip_kv_write_args* args, void* stream);

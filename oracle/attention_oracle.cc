@@ -87,6 +87,14 @@ struct CacheView {
     }
 };
 
+// Slab token of token j of sequence b: contiguous region (cache_mode 0) or page table (cache_mode 1) laid out as
+// tools/benchmark_llama/generation_state.cc:111-117 fills it: cachestarts[b][p] = first slab token of page p.
+inline int64_t slab_token(const int64_t* cachestarts, int cache_mode, int page_size, int64_t stride_b, int64_t b,
+                          int64_t j) {
+    if (cache_mode == 0) return cachestarts[b] + j;
+    return cachestarts[b * stride_b + j / page_size] + j % page_size;
+}
+
 void write_new_tokens(const pplhip_kv_write_args* a) {
     CacheView cv{(int8_t*)a->d_cache, (uint16_t*)a->d_scale, a->cache_stride_s, a->cache_stride_l,
                  a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
@@ -95,7 +103,8 @@ void write_new_tokens(const pplhip_kv_write_args* a) {
     for (int64_t b = 0; b < a->batch; ++b) {
         const int64_t s0 = a->d_seqstarts[b], s1 = a->d_seqstarts[b + 1];
         for (int64_t t = s0; t < s1; ++t) {
-            const int64_t tok = a->d_cachestarts[b] + a->d_start_pos[b] + (t - s0);
+            const int64_t tok = slab_token(a->d_cachestarts, a->cache_mode, a->page_size, a->cachestart_stride_b, b,
+                                           a->d_start_pos[b] + (t - s0));
             for (int kv = 0; kv < 2; ++kv)
                 for (int h = 0; h < KVH; ++h) {
                     const uint16_t* x = src[kv] + (t * KVH + h) * Dh;
@@ -144,7 +153,7 @@ int oracle_kv_quantize_write(const pplhip_kv_write_args* a) {
 int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
     const int H = a->num_heads, KVH = a->num_kv_heads, Dh = a->head_dim;
     if (H <= 0 || KVH <= 0 || H % KVH || Dh % kGroup) return PPLHIP_RC_INVALID_VALUE;
-    if (a->d_attn_mask || a->d_alibi_slopes || a->cache_mode != 0) return PPLHIP_RC_UNSUPPORTED;
+    if (a->d_attn_mask || a->d_alibi_slopes || (a->cache_mode != 0 && a->cache_mode != 1)) return PPLHIP_RC_UNSUPPORTED;
     pplhip_kv_write_args w;
     memset(&w, 0, sizeof(w));
     w.d_current_key = a->d_current_key;
@@ -164,6 +173,9 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
     w.cache_stride_kv = a->cache_stride_kv;
     w.d_cache = a->d_cache;
     w.d_scale = a->d_scale;
+    w.cache_mode = a->cache_mode;
+    w.page_size = a->page_size;
+    w.cachestart_stride_b = a->cachestart_stride_b;
     write_new_tokens(&w);
 
     CacheView cv{(int8_t*)a->d_cache, (uint16_t*)a->d_scale, a->cache_stride_s, a->cache_stride_l,
@@ -187,7 +199,8 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
             std::vector<double> K((size_t)kvlen * Dh), V((size_t)kvlen * Dh);
             for (int64_t j = 0; j < kvlen; ++j) {
                 if (from_cache) {
-                    const int64_t tok = a->d_cachestarts[b] + j;
+                    const int64_t tok =
+                        slab_token(a->d_cachestarts, a->cache_mode, a->page_size, a->cachestart_stride_b, b, j);
                     dequant_row(cv.row(tok, 0, kvh), cv.srow(tok, 0, kvh), Dh, &K[j * Dh]);
                     dequant_row(cv.row(tok, 1, kvh), cv.srow(tok, 1, kvh), Dh, &V[j * Dh]);
                 } else {

@@ -62,6 +62,7 @@ class KvWriteArgs(C.Structure):
         ("layer_idx", _i32), ("num_layer", _i32), ("num_kv_heads", _i32), ("head_dim", _i32),
         ("cache_stride_s", _i64), ("cache_stride_l", _i64), ("cache_stride_h", _i64), ("cache_stride_kv", _i64),
         ("d_cache", _p), ("d_scale", _p),
+        ("cache_mode", _i32), ("page_size", _i32), ("cachestart_stride_b", _i64),
     ]
 
 

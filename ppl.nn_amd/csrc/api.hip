@@ -66,6 +66,22 @@ static void write_args_from_mhca(const pplhip_mhca_args* a, pplhip_kv_write_args
     w->cache_stride_kv = a->cache_stride_kv;
     w->d_cache = a->d_cache;
     w->d_scale = a->d_scale;
+    w->cache_mode = a->cache_mode;
+    w->page_size = a->page_size;
+    w->cachestart_stride_b = a->cachestart_stride_b;
+}
+
+// cache_mode 0 (one contiguous slab region per sequence) or 1 (paged; multi_head_cache_attention_kernel.cc:161-168
+// requires the 2-D page table, whose second extent arrives here as cachestart_stride_b)
+static pplhip_retcode validate_cache_mode(int cache_mode, int page_size, int64_t cachestart_stride_b) {
+    if (cache_mode != 0 && cache_mode != 1) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "unknown cache_mode %d", cache_mode);
+    if (cache_mode == 1) {
+        if (cachestart_stride_b <= 0)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cachestarts must be a 2d tensor in cache_mode 1");
+        if (page_size < 64 || (page_size & (page_size - 1)))
+            PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "page_size %d: must be a power of two, at least 64", page_size);
+    }
+    return PPLHIP_RC_SUCCESS;
 }
 
 static pplhip_retcode validate_write(const pplhip_kv_write_args* a) {
@@ -73,6 +89,8 @@ static pplhip_retcode validate_write(const pplhip_kv_write_args* a) {
     if (a->batch < 0 || a->total_new_tokens < 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "negative batch or token count");
     pplhip_retcode rc = validate_common(a->num_kv_heads, a->head_dim, a->num_layer, a->layer_idx, a->cache_stride_s,
                                         a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->d_cache, a->d_scale);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    rc = validate_cache_mode(a->cache_mode, a->page_size, a->cachestart_stride_b);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
     if (a->batch > 0 && a->total_new_tokens > 0) {
         if (!a->d_current_key || !a->d_current_value || !a->d_seqstarts || !a->d_cachestarts || !a->d_start_pos)
@@ -102,7 +120,10 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     memset(plan, 0, sizeof(*plan));
     if (a->d_alibi_slopes) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support is_alibi == false");
     if (a->d_attn_mask) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "attn_mask is not supported");
-    if (a->cache_mode != 0) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support cache_mode == 0");
+    {
+        pplhip_retcode rcm = validate_cache_mode(a->cache_mode, a->page_size, a->cachestart_stride_b);
+        if (rcm != PPLHIP_RC_SUCCESS) return rcm;
+    }
     if (a->num_heads <= 0 || a->num_kv_heads <= 0 || a->num_heads % a->num_kv_heads)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d is not a multiple of num_kv_heads %d", a->num_heads,
                     a->num_kv_heads);

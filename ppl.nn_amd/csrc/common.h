@@ -45,6 +45,24 @@ struct CacheAddr {
     }
 };
 
+// Where token j of sequence b lives in the slab: a contiguous region per sequence (cache_mode 0, page_shift == 0) or
+// pages of 2^page_shift tokens listed per sequence in a [batch, stride_b] table (cache_mode 1).
+struct PageMap {
+    const int64_t* cachestarts;
+    int64_t stride_b;
+    int32_t page_shift;
+    __device__ inline int64_t token(int64_t b, int64_t j) const {
+        if (page_shift == 0) return cachestarts[b] + j;
+        return cachestarts[b * stride_b + (j >> page_shift)] + (j & ((int64_t(1) << page_shift) - 1));
+    }
+};
+inline int page_shift_of(int cache_mode, int page_size) { // host: 0 for the contiguous mode
+    if (cache_mode == 0) return 0;
+    int s = 0;
+    while ((1 << s) < page_size) ++s;
+    return s;
+}
+
 // first index b in [0, n) with starts[b+1] > x  (starts is a non-decreasing prefix-sum table with n+1 entries)
 __device__ inline int find_sequence(const int64_t* __restrict__ starts, int n, int64_t x) {
     int lo = 0, hi = n;

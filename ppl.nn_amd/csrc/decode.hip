@@ -64,7 +64,9 @@ struct DecodeParams {
     const half_t* scale;
     const int64_t* seqstarts;
     const int64_t* kvstarts;
-    const int64_t* cachestarts;
+    const int64_t* cachestarts; // [nd], or the [nd, cs_stride_b] page table when page_shift > 0
+    int64_t cs_stride_b;
+    int32_t page_shift; // 0: contiguous region per sequence; else pages of 2^page_shift tokens
     half_t* out; // [S, H, Dh]
     float* part_acc; // [slots, H, Dh], slots = num_ranges + nd
     float* part_ml; // [slots, H, 2]
@@ -174,6 +176,7 @@ constexpr int kDmaPerStage = 2 * (kStageTokens / 8) + 2; // 4 K + 4 V + K scales
 struct DmaOffsets {
     uint32_t kv[kStageTokens / 8]; // rows 8*i + lane/8: row * stride + swizzled piece * 16
     uint32_t sc; // row lane/2: row * scale stride + (lane & 1) * 16
+    uint8_t kv_row[kStageTokens / 8], sc_row; // the (clamped) rows themselves: the paged path picks a page per row
 };
 
 // rows_mem: rows of the stage that exist in the chunk (1..32); later rows are clamped onto the last one
@@ -185,10 +188,12 @@ __device__ inline void make_dma_offsets(DmaOffsets& o, int lane, uint32_t stride
         r = r < rows_mem ? r : rows_mem - 1;
         // the swizzle key is the LDS row (8*i + lane/8) & 7 = lane >> 3, whatever row the bytes come from
         o.kv[i] = (uint32_t)r * stride + 16u * piece;
+        o.kv_row[i] = (uint8_t)r;
     }
     int rs = lane >> 1;
     rs = rs < rows_mem ? rs : rows_mem - 1;
     o.sc = (uint32_t)rs * sstride_b + 16u * (lane & 1);
+    o.sc_row = (uint8_t)rs;
 }
 
 // Enqueues the 10 global->LDS transfers of one stage. cbase/sbase: K row 0 of the stage in the cache / scale tensors;
@@ -203,6 +208,24 @@ __device__ inline void dma_stage(char* lds_stage, const char* cbase, const char*
     }
     __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + o.sc), (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
     __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + kv_off_s + o.sc), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
+}
+
+// The same 10 transfers when a stage may straddle two pages of a paged slab: rows below `split` come from page A
+// (cbase_a / sbase_a address row 0 of the stage), the others from page B (cbase_b / sbase_b address the row that
+// would precede page B's first row by `split` rows, so the same per-row offsets apply). The base is then per lane,
+// so these transfers take the 64-bit vector-address form.
+__device__ inline void dma_stage_paged(char* lds_stage, const char* cbase_a, const char* cbase_b, const char* sbase_a,
+                                       const char* sbase_b, int split, const DmaOffsets& o, uint32_t kv_off,
+                                       uint32_t kv_off_s) {
+#pragma unroll
+    for (int i = 0; i < kStageTokens / 8; ++i) {
+        const char* cb = (o.kv_row[i] < split ? cbase_a : cbase_b) + o.kv[i];
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)cb, (lds_ptr_t)(lds_stage + kLdsK + 1024 * i), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cb + kv_off), (lds_ptr_t)(lds_stage + kLdsV + 1024 * i), 16, 0, 0);
+    }
+    const char* sb = (o.sc_row < split ? sbase_a : sbase_b) + o.sc;
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)sb, (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sb + kv_off_s), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
 }
 
 // Per-lane LDS read offsets inside a stage (they are the same for every stage).
@@ -345,6 +368,7 @@ __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, 
     }
 }
 
+template <bool PAGED>
 __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63;
@@ -398,7 +422,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         const int64_t seg_end = ((r1 < seq_hi) ? r1 : seq_hi) - seq_lo;
         pos = seq_lo + seg_end;
         const bool whole_sequence = seg_begin == 0 && seg_end == seq_hi - seq_lo;
-        const int64_t tok0 = p.cachestarts[b];
+        // contiguous slab region of the sequence, or its row of the page table
+        const int64_t tok0 = PAGED ? 0 : p.cachestarts[b];
+        const int64_t* page_row = PAGED ? p.cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
         const int64_t qrow = p.seqstarts[b];
         int64_t sub = (seg_end - seg_begin + tsplits - 1) / tsplits;
         sub = (sub + kStageTokens - 1) / kStageTokens * kStageTokens;
@@ -427,6 +453,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         ss.l_part = 0.f;
 
         if (t_begin < t_end) {
+            const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
             const int64_t row0 = p.addr.row(tok0 + t_begin, 0, kvh);
             const char* cbase = reinterpret_cast<const char*>(p.cache) + row0;
             const char* sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
@@ -437,16 +464,37 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
             const int tail_rows_mem =
                 (int)((seg_end - last_stage_t0) < kStageTokens ? (seg_end - last_stage_t0) : kStageTokens);
             const int tail_rows_valid = (int)(t_end - last_stage_t0);
-            auto issue = [&](int idx) {
+            auto issue_with = [&](int idx, const DmaOffsets& off, int rows_mem) {
                 char* dst = wave_lds + (idx & 1) * kStageBytes;
-                const char* cb = make_uniform(cbase + idx * step_c);
-                const char* sb = make_uniform(sbase + idx * step_s);
+                if (PAGED) {
+                    // a stage of 32 tokens touches at most two pages (pages hold >= 64 tokens)
+                    const int64_t t0 = t_begin + (int64_t)idx * kStageTokens;
+                    const int64_t in_page = t0 & ((int64_t(1) << p.page_shift) - 1);
+                    const int64_t left = (int64_t(1) << p.page_shift) - in_page; // rows of the stage in its first page
+                    const int split = left < kStageTokens ? (int)left : kStageTokens;
+                    const int64_t pa = page_row[t0 >> p.page_shift];
+                    // the second page exists whenever one of the stage's (clamped) rows lies in it
+                    const int64_t pb = split < rows_mem ? page_row[(t0 >> p.page_shift) + 1] : pa;
+                    const int64_t ra = (pa + in_page) * (int64_t)stride + head_off;
+                    const int64_t rb = (pb - split) * (int64_t)stride + head_off;
+                    const char* ca = make_uniform(reinterpret_cast<const char*>(p.cache) + ra);
+                    const char* cb = make_uniform(reinterpret_cast<const char*>(p.cache) + rb);
+                    const char* sa = make_uniform(reinterpret_cast<const char*>(p.scale) + (ra / kQuantGroup) * 2);
+                    const char* sb = make_uniform(reinterpret_cast<const char*>(p.scale) + (rb / kQuantGroup) * 2);
+                    dma_stage_paged(dst, ca, cb, sa, sb, split, off, kv_off, kv_off_s);
+                } else {
+                    const char* cb = make_uniform(cbase + idx * step_c);
+                    const char* sb = make_uniform(sbase + idx * step_s);
+                    dma_stage(dst, cb, sb, off, kv_off, kv_off_s);
+                }
+            };
+            auto issue = [&](int idx) {
                 if (idx == n_stages - 1 && tail_rows_mem < kStageTokens) { // wave-uniform, at most once per segment
                     DmaOffsets tail;
                     make_dma_offsets(tail, lane, stride, sstride_b, tail_rows_mem);
-                    dma_stage(dst, cb, sb, tail, kv_off, kv_off_s);
+                    issue_with(idx, tail, tail_rows_mem);
                 } else {
-                    dma_stage(dst, cb, sb, full, kv_off, kv_off_s);
+                    issue_with(idx, full, kStageTokens);
                 }
             };
 
@@ -590,6 +638,8 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     p.seqstarts = a->d_seqstarts;
     p.kvstarts = a->d_kvstarts;
     p.cachestarts = a->d_cachestarts;
+    p.cs_stride_b = a->cachestart_stride_b;
+    p.page_shift = page_shift_of(a->cache_mode, a->page_size);
     p.out = (half_t*)a->d_output;
     p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
     p.nd = nd;
@@ -610,14 +660,21 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
     static bool lds_opt_in = false; // more than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in
     if (!lds_opt_in) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_int8kv_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess)
-            PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
-                        lds_bytes, hipGetErrorString(e));
+        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true>)}) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess)
+                PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
+                            lds_bytes, hipGetErrorString(e));
+        }
         lds_opt_in = true;
     }
-    hipLaunchKernelGGL(decode_int8kv_kernel, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes, stream, p);
+    if (p.page_shift)
+        hipLaunchKernelGGL(decode_int8kv_kernel<true>, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes,
+                           stream, p);
+    else
+        hipLaunchKernelGGL(decode_int8kv_kernel<false>, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes,
+                           stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
     hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_merge");

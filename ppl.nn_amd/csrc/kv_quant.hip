@@ -13,7 +13,7 @@ struct QuantWriteParams {
     const half_t* key;
     const half_t* value;
     const int64_t* seqstarts;
-    const int64_t* cachestarts;
+    PageMap pages;
     const int64_t* start_pos;
     int8_t* cache;
     half_t* scale;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     const int head = r2 / gph;
     const int grp = r2 - head * gph;
     const int b = find_sequence(p.seqstarts, p.batch, t);
-    const int64_t tok = p.cachestarts[b] + p.start_pos[b] + (t - p.seqstarts[b]);
+    const int64_t tok = p.pages.token(b, p.start_pos[b] + (t - p.seqstarts[b]));
     const half_t* src = (kv ? p.value : p.key) + ((t * p.kv_heads + head) * gph + grp) * 8;
     const uint4 raw = *reinterpret_cast<const uint4*>(src);
     uint2 q;
@@ -77,7 +77,7 @@ pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream
     p.key = (const half_t*)a->d_current_key;
     p.value = (const half_t*)a->d_current_value;
     p.seqstarts = a->d_seqstarts;
-    p.cachestarts = a->d_cachestarts;
+    p.pages = PageMap{a->d_cachestarts, a->cachestart_stride_b, page_shift_of(a->cache_mode, a->page_size)};
     p.start_pos = a->d_start_pos;
     p.cache = (int8_t*)a->d_cache;
     p.scale = (half_t*)a->d_scale;

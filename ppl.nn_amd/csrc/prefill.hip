@@ -45,7 +45,7 @@ struct PrefillParams {
     const half_t* scale;
     const int64_t* seqstarts;
     const int64_t* kvstarts;
-    const int64_t* cachestarts;
+    PageMap pages; // cache source only
     const int64_t* start_pos;
     half_t* out;
     CacheAddr addr;
@@ -94,12 +94,21 @@ struct TileSrc<false> {
 };
 template <>
 struct TileSrc<true> {
-    const char* k; // slab rows of token 0 of the sequence (this layer, K / V, this kv head)
+    const char* k; // slab rows of slab token 0 (this layer, K / V, this kv head)
     const char* v;
     const char* ks; // their scale rows
     const char* vs;
+    const int64_t* page_row; // cache_mode 1: the sequence's row of the page table; cache_mode 0: null
+    int64_t tok0; // cache_mode 0: first slab token of the sequence
+    int32_t page_shift;
     uint32_t row_bytes, srow_bytes;
     uint32_t voff, svoff;
+    // slab token of sequence token j0, the first of a 64-token tile: tiles never straddle a page (pages are powers of
+    // two >= 64 tokens and tiles start at multiples of 64)
+    __device__ inline int64_t tile_token(int64_t j0) const {
+        if (page_shift == 0) return tok0 + j0;
+        return page_row[j0 >> page_shift] + (j0 & ((int64_t(1) << page_shift) - 1));
+    }
 };
 
 __device__ inline void fetch_tile(TileRegs<false>& t, const TileSrc<false>& src, int64_t j0, int64_t kvlen) {
@@ -128,11 +137,12 @@ __device__ inline void fetch_tile(TileRegs<false>& t, const TileSrc<false>& src,
 
 __device__ inline void fetch_tile(TileRegs<true>& t, const TileSrc<true>& src, int64_t j0, int64_t kvlen) {
     const int r0 = threadIdx.x >> 4;
+    const int64_t tok = src.tile_token(j0);
+    const char* kb = uniform_ptr(src.k + tok * src.row_bytes);
+    const char* vb = uniform_ptr(src.v + tok * src.row_bytes);
+    const char* ksb = uniform_ptr(src.ks + tok * src.srow_bytes);
+    const char* vsb = uniform_ptr(src.vs + tok * src.srow_bytes);
     if (j0 + kBN <= kvlen) {
-        const char* kb = uniform_ptr(src.k + j0 * src.row_bytes);
-        const char* vb = uniform_ptr(src.v + j0 * src.row_bytes);
-        const char* ksb = uniform_ptr(src.ks + j0 * src.srow_bytes);
-        const char* vsb = uniform_ptr(src.vs + j0 * src.srow_bytes);
 #pragma unroll
         for (int pass = 0; pass < 4; ++pass) {
             t.kq[pass] = *reinterpret_cast<const uint2*>(kb + pass * src.row_bytes + src.voff);
@@ -147,12 +157,10 @@ __device__ inline void fetch_tile(TileRegs<true>& t, const TileSrc<true>& src, i
             t.kq[pass] = t.vq[pass] = make_uint2(0, 0);
             t.ks[pass] = t.vs[pass] = 0;
             if (j < kvlen) {
-                const int64_t off = (j0 + pass) * src.row_bytes + src.voff;
-                const int64_t soff = (j0 + pass) * src.srow_bytes + src.svoff;
-                t.kq[pass] = *reinterpret_cast<const uint2*>(src.k + off);
-                t.vq[pass] = *reinterpret_cast<const uint2*>(src.v + off);
-                t.ks[pass] = *reinterpret_cast<const uint16_t*>(src.ks + soff);
-                t.vs[pass] = *reinterpret_cast<const uint16_t*>(src.vs + soff);
+                t.kq[pass] = *reinterpret_cast<const uint2*>(kb + pass * src.row_bytes + src.voff);
+                t.vq[pass] = *reinterpret_cast<const uint2*>(vb + pass * src.row_bytes + src.voff);
+                t.ks[pass] = *reinterpret_cast<const uint16_t*>(ksb + pass * src.srow_bytes + src.svoff);
+                t.vs[pass] = *reinterpret_cast<const uint16_t*>(vsb + pass * src.srow_bytes + src.svoff);
             }
         }
     }
@@ -168,16 +176,19 @@ __device__ inline TileSrc<false> make_tile_src_f16(const PrefillParams& p, int64
     src.voff = 4 * r0 * src.row_bytes + col * 16;
     return src;
 }
-__device__ inline TileSrc<true> make_tile_src_cache(const PrefillParams& p, int64_t tok0, int kvh) {
+__device__ inline TileSrc<true> make_tile_src_cache(const PrefillParams& p, int b, int kvh) {
     TileSrc<true> src;
     const int tid = threadIdx.x, col = tid & 15, r0 = tid >> 4;
-    const int64_t rk = p.addr.row(tok0, 0, kvh), rv = p.addr.row(tok0, 1, kvh);
+    const int64_t rk = p.addr.row(0, 0, kvh), rv = p.addr.row(0, 1, kvh);
     src.row_bytes = (uint32_t)p.addr.stride_s; // int8: one byte per element
     src.srow_bytes = src.row_bytes / kQuantGroup * 2;
     src.k = reinterpret_cast<const char*>(p.cache) + rk;
     src.v = reinterpret_cast<const char*>(p.cache) + rv;
     src.ks = reinterpret_cast<const char*>(p.scale) + rk / kQuantGroup * 2;
     src.vs = reinterpret_cast<const char*>(p.scale) + rv / kQuantGroup * 2;
+    src.page_shift = p.pages.page_shift;
+    src.page_row = p.pages.page_shift ? p.pages.cachestarts + (int64_t)b * p.pages.stride_b : nullptr;
+    src.tok0 = p.pages.page_shift ? 0 : p.pages.cachestarts[b];
     src.voff = 4 * r0 * src.row_bytes + col * 8;
     src.svoff = 4 * r0 * src.srow_bytes + col * 2;
     return src;
@@ -268,7 +279,6 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     const int64_t kv0 = p.kvstarts[b];
     const int64_t kvlen = p.kvstarts[b + 1] - kv0;
     const int64_t sp = FROM_CACHE ? p.start_pos[b] : (kvlen > L ? kvlen - L : 0);
-    const int64_t tok0 = FROM_CACHE ? p.cachestarts[b] : 0;
     const int ntiles = (int)((L + kBM - 1) / kBM);
     const int ntiles_max = gridDim.x / per_tile;
     const int qt = ntiles_max - 1 - qt_rev; // tile index counted from the start of the sequence
@@ -289,7 +299,7 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
 
     TileRegs<FROM_CACHE> regs;
     TileSrc<FROM_CACHE> src;
-    if constexpr (FROM_CACHE) src = make_tile_src_cache(p, tok0, kvh);
+    if constexpr (FROM_CACHE) src = make_tile_src_cache(p, b, kvh);
     else src = make_tile_src_f16(p, kv0, kvh);
     fetch_tile(regs, src, 0, kvlen);
 
@@ -460,7 +470,7 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     p.seqstarts = a->d_seqstarts;
     // fp16 source: the keys of a prefill sequence are its own new tokens, packed like the queries
     p.kvstarts = a->enable_cache_prefill ? a->d_kvstarts : a->d_seqstarts;
-    p.cachestarts = a->d_cachestarts;
+    p.pages = PageMap{a->d_cachestarts, a->cachestart_stride_b, page_shift_of(a->cache_mode, a->page_size)};
     p.start_pos = a->d_start_pos;
     p.out = (half_t*)a->d_output;
     p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
@@ -494,7 +504,7 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
     p.scale = nullptr;
     p.seqstarts = a->d_seqstarts;
     p.kvstarts = a->d_kvstarts;
-    p.cachestarts = nullptr;
+    p.pages = PageMap{nullptr, 0, 0};
     p.start_pos = nullptr;
     p.out = (half_t*)a->d_output;
     p.addr = CacheAddr{0, 0, 0, 0, 0};

@@ -25,14 +25,41 @@ def _ptr(a):
     return a.ctypes.data_as(C.c_void_p) if a is not None else None
 
 
-def new_slab(b):
-    shape = (b.max_tokens, b.num_layer, 2, b.num_kv_heads, b.head_dim)
+class PagedLayout:
+    """cache_mode 1: every sequence owns ceil(kvlen / page_size) pages scattered over the slab in a seeded random
+    order; table[b, p] = first slab token of page p of sequence b (unused entries -1)."""
+
+    def __init__(self, b, page_size=128, seed=0):
+        kv = b.kvlens
+        pages = (kv + page_size - 1) // page_size
+        self.page_size = page_size
+        self.max_pages = int(max(1, pages.max())) if len(pages) else 1
+        total = int(pages.sum())
+        order = np.random.default_rng(seed).permutation(total + 3)  # a few pages stay unused
+        self.slab_tokens = (total + 3) * page_size
+        self.table = np.full((b.batch, self.max_pages), -1, np.int64)
+        k = 0
+        for i, n in enumerate(pages):
+            self.table[i, :n] = order[k:k + n] * page_size
+            k += int(n)
+
+    def token(self, i, j):
+        return int(self.table[i, j // self.page_size] + j % self.page_size)
+
+
+def _set_cache_mode(a, paged):
+    a.cache_mode, a.page_size = (1, paged.page_size) if paged else (0, 128)
+    a.cachestart_stride_b = paged.max_pages if paged else 0
+
+
+def new_slab(b, paged=None):
+    shape = ((paged.slab_tokens if paged else b.max_tokens), b.num_layer, 2, b.num_kv_heads, b.head_dim)
     cache = np.full(shape, CACHE_FILL, dtype=np.int8)
     scale = np.full(shape[:-1] + (b.head_dim // 8,), SCALE_FILL, dtype=np.uint16).view(np.float16)
     return cache, scale
 
 
-def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, scale, ptr=_ptr):
+def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, scale, ptr=_ptr, paged=None):
     st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
     w.d_current_key, w.d_current_value = ptr(key), ptr(value)
     w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(seqstarts), ptr(cachestarts), ptr(start_pos)
@@ -41,13 +68,14 @@ def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, 
     for k, v in st.items():
         setattr(w, k, v)
     w.d_cache, w.d_scale = ptr(cache), ptr(scale)
+    _set_cache_mode(w, paged)
     # the struct only holds raw addresses: keep the arrays (often temporaries such as b.histstarts) alive with it
     w._refs = getattr(w, "_refs", []) + [key, value, seqstarts, start_pos, cachestarts, cache, scale]
     return w
 
 
 def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out, ptr=_ptr,
-                   cache_prefill=0, split_k=1):
+                   cache_prefill=0, split_k=1, paged=None):
     st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
     a.d_query, a.d_current_key, a.d_current_value = ptr(q), ptr(k), ptr(v)
     a.d_attn_mask = None
@@ -59,10 +87,9 @@ def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, c
     a.max_seqlen, a.max_kvlen = b.max_seqlen, b.max_kvlen
     a.layer_idx, a.num_layer = b.layer_idx, b.num_layer
     a.num_heads, a.num_kv_heads, a.head_dim = b.num_heads, b.num_kv_heads, b.head_dim
-    a.cache_mode, a.page_size = 0, 128
     for kk, vv in st.items():
         setattr(a, kk, vv)
-    a.cachestart_stride_b = 0
+    _set_cache_mode(a, paged)
     a.enable_cache_prefill = cache_prefill
     a.enable_decoding_sharemem_mhca = a.enable_decoding_infinity_mhca = a.enable_decoding_infinity_gqca = 1
     a.specify_decoding_attn_split_k = split_k
@@ -73,21 +100,22 @@ def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, c
     return a
 
 
-def run_oracle(b, t, cache_prefill=0, want_f64=True):
+def run_oracle(b, t, cache_prefill=0, want_f64=True, paged=None):
     """History write + MHCA on the CPU oracle. Returns cache (int8), scale (fp16), output (fp16), output_f64."""
     import oracle
     L = oracle.lib()
-    cache, scale = new_slab(b)
+    cache, scale = new_slab(b, paged)
     zeros = np.zeros(b.batch, np.int64)
+    cs = np.ascontiguousarray(paged.table) if paged else b.cachestarts
     if b.total_hist_tokens:
         w = fill_write_args(cabi.KvWriteArgs(), b, t["hist_key"], t["hist_value"], b.histstarts, zeros,
-                            b.cachestarts, cache, scale)
+                            cs, cache, scale, paged=paged)
         assert L.oracle_kv_quantize_write(C.byref(w)) == 0
     out = np.zeros((b.total_new_tokens, b.num_heads, b.head_dim), np.float16)
     out64 = np.zeros(out.shape, np.float64) if want_f64 else None
     seqstarts, kvstarts, sp = b.seqstarts, b.kvstarts, b.start_pos.copy()
     a = fill_mhca_args(cabi.MhcaArgs(), b, t["query"], t["current_key"], t["current_value"], seqstarts, kvstarts,
-                       b.cachestarts, sp, cache, scale, out, cache_prefill=cache_prefill)
+                       cs, sp, cache, scale, out, cache_prefill=cache_prefill, paged=paged)
     rc = L.oracle_mhca_forward(C.byref(a), _ptr(out64))
     assert rc == 0, rc
     return dict(cache=cache, scale=scale, output=out, output_f64=out64)
@@ -104,25 +132,26 @@ def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None):
+def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None):
     """Same call through the C ABI on cuda:0."""
     import torch
     lib = pkg.load_library()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cache_h, scale_h = new_slab(b)
+    cache_h, scale_h = new_slab(b, paged)
     cache, scale = to_dev(cache_h), to_dev(scale_h)
     d = {k: to_dev(v) for k, v in t.items()}
-    tabs = dict(seqstarts=b.seqstarts, kvstarts=b.kvstarts, cachestarts=b.cachestarts, start_pos=b.start_pos,
+    tabs = dict(seqstarts=b.seqstarts, kvstarts=b.kvstarts,
+                cachestarts=np.ascontiguousarray(paged.table) if paged else b.cachestarts, start_pos=b.start_pos,
                 histstarts=b.histstarts, zeros=np.zeros(max(b.batch, 1), np.int64))
     dt = {k: to_dev(v) for k, v in tabs.items()}
     if b.total_hist_tokens:
         w = fill_write_args(cabi.KvWriteArgs(), b, d["hist_key"], d["hist_value"], dt["histstarts"], dt["zeros"],
-                            dt["cachestarts"], cache, scale, ptr=dev_ptr)
+                            dt["cachestarts"], cache, scale, ptr=dev_ptr, paged=paged)
         pkg.check(lib.pplhip_kv_quantize_write(C.byref(w), stream), "kv_quantize_write(history)")
     out = torch.zeros((b.total_new_tokens, b.num_heads, b.head_dim), dtype=torch.float16, device="cuda")
     a = fill_mhca_args(cabi.MhcaArgs(), b, d["query"], d["current_key"], d["current_value"], dt["seqstarts"],
                        dt["kvstarts"], dt["cachestarts"], dt["start_pos"], cache, scale, out, ptr=dev_ptr,
-                       cache_prefill=cache_prefill, split_k=split_k)
+                       cache_prefill=cache_prefill, split_k=split_k, paged=paged)
     plan = cabi.MhcaPlan()
     pkg.check(lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)), "mhca_prepare")
     ws = torch.empty(max(int(plan.workspace_bytes), 256), dtype=torch.uint8, device="cuda")

@@ -72,7 +72,12 @@ def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
     (lambda a: setattr(a, "d_alibi_slopes", 0x10), cabi.RC_UNSUPPORTED),  # …_kernel.cc:95-98
     (lambda a: setattr(a, "d_scale", None), cabi.RC_UNSUPPORTED),  # …_kernel.cc:100-103
     (lambda a: setattr(a, "d_attn_mask", 0x10), cabi.RC_UNSUPPORTED),
-    (lambda a: setattr(a, "cache_mode", 1), cabi.RC_UNSUPPORTED),
+    (lambda a: setattr(a, "cache_mode", 1), cabi.RC_INVALID_VALUE),  # no 2-d page table: …_kernel.cc:162-166
+    (lambda a: setattr(a, "cache_mode", 2), cabi.RC_UNSUPPORTED),
+    (lambda a: (setattr(a, "cache_mode", 1), setattr(a, "cachestart_stride_b", 4), setattr(a, "page_size", 96)),
+     cabi.RC_UNSUPPORTED),
+    (lambda a: (setattr(a, "cache_mode", 1), setattr(a, "cachestart_stride_b", 4), setattr(a, "page_size", 32)),
+     cabi.RC_UNSUPPORTED),
     (lambda a: setattr(a, "head_dim", 64), cabi.RC_UNSUPPORTED),
     (lambda a: setattr(a, "num_kv_heads", 3), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "layer_idx", 5), cabi.RC_INVALID_VALUE),
@@ -87,6 +92,12 @@ def test_prepare_rejects(hiplib, mutate, rc):
     mutate(a)
     assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == rc
     assert len(hiplib.pplhip_last_error()) > 0
+
+
+def test_prepare_accepts_paged_cache(hiplib):
+    a, plan = _valid_args(), cabi.MhcaPlan()
+    a.cache_mode, a.cachestart_stride_b, a.page_size = 1, 4, 128
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
 
 
 def test_kv_cache_rejects_like_the_reference_stub(hiplib):

@@ -271,3 +271,38 @@ def test_position_index_graph(hiplib):
     out = s.output(0, np.int64)
     assert np.array_equal(out, np.concatenate([p + np.arange(n) for n, p in zip(seqlens, start)]))
     s.close()
+
+
+def test_paged_mhca_graph_through_the_engine(hiplib):
+    """cache_mode 1 through the op: the 2-d cachestarts tensor is the page table, its second extent the table stride."""
+    import torch
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(8, 2, 128, [1, 1, 90], [700, 12, 0], 2, num_layer=1, layer_idx=0, name="engine_paged")
+    t = workloads.make_tensors(b, seed=61)
+    paged = harness.PagedLayout(b, page_size=128, seed=4)
+    ref = harness.run_oracle(b, t, paged=paged)
+    # history through the C ABI into the paged slab
+    cache_h, scale_h = harness.new_slab(b, paged)
+    cache, scale = harness.to_dev(cache_h), harness.to_dev(scale_h)
+    hk, hv = harness.to_dev(t["hist_key"]), harness.to_dev(t["hist_value"])
+    hs, z, tab = harness.to_dev(b.histstarts), harness.to_dev(np.zeros(b.batch, np.int64)), harness.to_dev(paged.table)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, hk, hv, hs, z, tab, cache, scale, ptr=harness.dev_ptr, paged=paged)
+    harness.pkg.check(hiplib.pplhip_kv_quantize_write(C.byref(w), None), "history")
+    torch.cuda.synchronize()
+    s = Session(eng, ow.mhca_model(8, 2, 128, 1, 0, extra_attrs={"cache_mode": 1, "page_size": 128}))
+    s.set_device_tensor(0, harness.to_dev(t["query"]))
+    s.set_device_tensor(1, harness.to_dev(t["current_key"]))
+    s.set_device_tensor(2, harness.to_dev(t["current_value"]))
+    s.set_table(3, b.seqstarts)
+    s.set_table(4, b.kvstarts)
+    s.set_table(5, paged.table)
+    s.set_table(6, b.start_pos)
+    for i, v in zip(range(7, 10), (b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+        s.set_host_scalar(i, v)
+    s.set_device_tensor(10, cache)
+    s.set_device_tensor(11, scale)
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    harness.assert_attn_close(s.output(0, np.float16), ref["output_f64"])
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), ref["cache"])
+    s.close()

@@ -252,3 +252,34 @@ def test_mhca_equals_mha_over_kv_cache_outputs(hiplib):
     assert np.array_equal(cache.cpu().numpy(), mhca["cache"])
     via = out.cpu().view(torch.int16).numpy().view(np.float16).astype(np.float64)
     assert np.abs(via - mhca["output"].astype(np.float64)).max() < 2e-3
+
+
+@pytest.mark.parametrize("page_size", [64, 128, 256])
+def test_paged_cache_mode(page_size):
+    """cache_mode 1 on the device: bit-identical slab rows and outputs to the contiguous mode, parity with the oracle.
+    Long decode sequences make 32-token stages straddle page boundaries at every offset."""
+    for cache_prefill in (0, 1):
+        # without cache-prefill the prompts start at position 0; with it one of them is a chunk at position 64
+        b = workloads.Batch(8, 2, 128, [1, 1, 1, 1, 70, 300], [130, 5, 1000, 2047, 0, 64 * cache_prefill], 4,
+                            num_layer=2, layer_idx=1, name="paged_mixed")
+        t = workloads.make_tensors(b, seed=52)
+        paged = harness.PagedLayout(b, page_size=page_size, seed=page_size)
+        print(f"case {b.name} page_size={page_size} max_pages={paged.max_pages} cache_prefill={cache_prefill}",
+              flush=True)
+        ref = harness.run_oracle(b, t, cache_prefill=cache_prefill, paged=paged)
+        got = harness.run_device(b, t, cache_prefill=cache_prefill, paged=paged)
+        flat = harness.run_device(b, t, cache_prefill=cache_prefill)
+        assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
+        assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
+        harness.assert_attn_close(got["output"], ref["output_f64"])
+        assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
+
+
+def test_paged_cache_full_size_decode():
+    b = workloads.cfg2_decode_part()
+    t = workloads.make_tensors(b, seed=53)
+    paged = harness.PagedLayout(b, page_size=128, seed=9)
+    print(f"case {b.name} paged full size: {int(b.kvstarts[-1])} cached tokens, {paged.max_pages} pages max", flush=True)
+    got = harness.run_device(b, t, paged=paged)
+    flat = harness.run_device(b, t)
+    assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))

@@ -226,3 +226,27 @@ def test_mha_vs_textbook_and_mhca_identity(causal):
     # int8 * fp16 scale is exact in fp32 and, with |q| <= 127, needs at most 18 significant bits: rounding it to
     # fp16 here is the KeyValueCache op's output rounding, which the cache path does not apply -> small difference
     assert np.abs(via_mha["output_f64"] - mhca["output_f64"]).max() < 2e-3
+
+
+def test_paged_cache_equals_contiguous_cache():
+    """cache_mode 1: the same tokens reached through a scattered page table give the same bytes and the same outputs."""
+    b = workloads.Batch(8, 2, 128, [1, 1, 1, 70, 300], [130, 5, 1000, 0, 64], 3, num_layer=2, layer_idx=1,
+                        name="paged_mixed")
+    t = workloads.make_tensors(b, seed=51)
+    for page_size in (64, 128):
+        paged = harness.PagedLayout(b, page_size=page_size, seed=page_size)
+        flat = harness.run_oracle(b, t, cache_prefill=1)
+        pg = harness.run_oracle(b, t, cache_prefill=1, paged=paged)
+        assert np.array_equal(flat["output_f64"], pg["output_f64"])
+        kv = b.kvlens
+        for i in range(b.batch):
+            for j in (0, int(kv[i]) // 2, int(kv[i]) - 1):
+                a, c = int(b.cachestarts[i]) + j, paged.token(i, j)
+                assert np.array_equal(flat["cache"][a], pg["cache"][c])
+                assert np.array_equal(flat["scale"][a].view(np.uint16), pg["scale"][c].view(np.uint16))
+        # untouched pages keep the fill pattern
+        used = set()
+        for i in range(b.batch):
+            used |= {int(x) // page_size for x in paged.table[i] if x >= 0}
+        free = sorted(set(range(paged.slab_tokens // page_size)) - used)
+        assert free and (pg["cache"][free[0] * page_size:(free[0] + 1) * page_size] == harness.CACHE_FILL).all()
