@@ -52,15 +52,24 @@ def _set_cache_mode(a, paged):
     a.cachestart_stride_b = paged.max_pages if paged else 0
 
 
-def new_slab(b, paged=None):
-    shape = ((paged.slab_tokens if paged else b.max_tokens), b.num_layer, 2, b.num_kv_heads, b.head_dim)
+def _strides(b, paged, layout):
+    tokens = paged.slab_tokens if paged else b.max_tokens
+    if layout == 3:
+        return cabi.cache_strides_layout3(b.num_layer, b.num_kv_heads, b.head_dim, tokens)
+    return cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
+
+
+def new_slab(b, paged=None, layout=0):
+    tokens = paged.slab_tokens if paged else b.max_tokens
+    shape = (tokens, b.num_layer, 2, b.num_kv_heads, b.head_dim) if layout == 0 else \
+        (b.num_layer, 2, b.num_kv_heads, tokens, b.head_dim)  # cache_layout 3
     cache = np.full(shape, CACHE_FILL, dtype=np.int8)
     scale = np.full(shape[:-1] + (b.head_dim // 8,), SCALE_FILL, dtype=np.uint16).view(np.float16)
     return cache, scale
 
 
-def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, scale, ptr=_ptr, paged=None):
-    st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
+def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, scale, ptr=_ptr, paged=None, layout=0):
+    st = _strides(b, paged, layout)
     w.d_current_key, w.d_current_value = ptr(key), ptr(value)
     w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(seqstarts), ptr(cachestarts), ptr(start_pos)
     w.batch, w.total_new_tokens = b.batch, int(key.shape[0])
@@ -75,8 +84,8 @@ def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, 
 
 
 def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out, ptr=_ptr,
-                   cache_prefill=0, split_k=1, paged=None):
-    st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
+                   cache_prefill=0, split_k=1, paged=None, layout=0):
+    st = _strides(b, paged, layout)
     a.d_query, a.d_current_key, a.d_current_value = ptr(q), ptr(k), ptr(v)
     a.d_attn_mask = None
     a.d_alibi_slopes = None
@@ -100,22 +109,22 @@ def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, c
     return a
 
 
-def run_oracle(b, t, cache_prefill=0, want_f64=True, paged=None):
+def run_oracle(b, t, cache_prefill=0, want_f64=True, paged=None, layout=0):
     """History write + MHCA on the CPU oracle. Returns cache (int8), scale (fp16), output (fp16), output_f64."""
     import oracle
     L = oracle.lib()
-    cache, scale = new_slab(b, paged)
+    cache, scale = new_slab(b, paged, layout)
     zeros = np.zeros(b.batch, np.int64)
     cs = np.ascontiguousarray(paged.table) if paged else b.cachestarts
     if b.total_hist_tokens:
         w = fill_write_args(cabi.KvWriteArgs(), b, t["hist_key"], t["hist_value"], b.histstarts, zeros,
-                            cs, cache, scale, paged=paged)
+                            cs, cache, scale, paged=paged, layout=layout)
         assert L.oracle_kv_quantize_write(C.byref(w)) == 0
     out = np.zeros((b.total_new_tokens, b.num_heads, b.head_dim), np.float16)
     out64 = np.zeros(out.shape, np.float64) if want_f64 else None
     seqstarts, kvstarts, sp = b.seqstarts, b.kvstarts, b.start_pos.copy()
     a = fill_mhca_args(cabi.MhcaArgs(), b, t["query"], t["current_key"], t["current_value"], seqstarts, kvstarts,
-                       cs, sp, cache, scale, out, cache_prefill=cache_prefill, paged=paged)
+                       cs, sp, cache, scale, out, cache_prefill=cache_prefill, paged=paged, layout=layout)
     rc = L.oracle_mhca_forward(C.byref(a), _ptr(out64))
     assert rc == 0, rc
     return dict(cache=cache, scale=scale, output=out, output_f64=out64)
@@ -132,12 +141,12 @@ def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None):
+def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0):
     """Same call through the C ABI on cuda:0."""
     import torch
     lib = pkg.load_library()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cache_h, scale_h = new_slab(b, paged)
+    cache_h, scale_h = new_slab(b, paged, layout)
     cache, scale = to_dev(cache_h), to_dev(scale_h)
     d = {k: to_dev(v) for k, v in t.items()}
     tabs = dict(seqstarts=b.seqstarts, kvstarts=b.kvstarts,
@@ -146,12 +155,12 @@ def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None):
     dt = {k: to_dev(v) for k, v in tabs.items()}
     if b.total_hist_tokens:
         w = fill_write_args(cabi.KvWriteArgs(), b, d["hist_key"], d["hist_value"], dt["histstarts"], dt["zeros"],
-                            dt["cachestarts"], cache, scale, ptr=dev_ptr, paged=paged)
+                            dt["cachestarts"], cache, scale, ptr=dev_ptr, paged=paged, layout=layout)
         pkg.check(lib.pplhip_kv_quantize_write(C.byref(w), stream), "kv_quantize_write(history)")
     out = torch.zeros((b.total_new_tokens, b.num_heads, b.head_dim), dtype=torch.float16, device="cuda")
     a = fill_mhca_args(cabi.MhcaArgs(), b, d["query"], d["current_key"], d["current_value"], dt["seqstarts"],
                        dt["kvstarts"], dt["cachestarts"], dt["start_pos"], cache, scale, out, ptr=dev_ptr,
-                       cache_prefill=cache_prefill, split_k=split_k, paged=paged)
+                       cache_prefill=cache_prefill, split_k=split_k, paged=paged, layout=layout)
     plan = cabi.MhcaPlan()
     pkg.check(lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)), "mhca_prepare")
     ws = torch.empty(max(int(plan.workspace_bytes), 256), dtype=torch.uint8, device="cuda")

@@ -283,3 +283,22 @@ def test_paged_cache_full_size_decode():
     got = harness.run_device(b, t, paged=paged)
     flat = harness.run_device(b, t)
     assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
+
+
+def test_cache_layout_3_on_device():
+    """cache_layout 3 (L, 2, KVH, MaxT, Dh): token rows of one head are 128 bytes apart instead of a whole slab row."""
+    for cache_prefill in (0, 1):
+        b = workloads.Batch(8, 2, 128, [1, 1, 1, 70, 200], [130, 5, 1000, 0, 64 * cache_prefill], 3, num_layer=3,
+                            layer_idx=2, name="layout3")
+        t = workloads.make_tensors(b, seed=55)
+        print(f"case {b.name} cache_prefill={cache_prefill}", flush=True)
+        ref = harness.run_oracle(b, t, cache_prefill=cache_prefill, layout=3)
+        got = harness.run_device(b, t, cache_prefill=cache_prefill, layout=3)
+        flat = harness.run_device(b, t, cache_prefill=cache_prefill)
+        assert np.array_equal(ref["cache"], got["cache"]) and np.array_equal(ref["scale"].view(np.uint16),
+                                                                               got["scale"].view(np.uint16))
+        harness.assert_attn_close(got["output"], ref["output_f64"])
+        assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
+        paged = harness.PagedLayout(b, page_size=64, seed=3)
+        both = harness.run_device(b, t, cache_prefill=cache_prefill, layout=3, paged=paged)
+        assert np.array_equal(both["output"].view(np.uint16), flat["output"].view(np.uint16))

@@ -250,3 +250,14 @@ def test_paged_cache_equals_contiguous_cache():
             used |= {int(x) // page_size for x in paged.table[i] if x >= 0}
         free = sorted(set(range(paged.slab_tokens // page_size)) - used)
         assert free and (pg["cache"][free[0] * page_size:(free[0] + 1) * page_size] == harness.CACHE_FILL).all()
+
+
+def test_cache_layout_3_equals_layout_0():
+    """cache_layout 3 = (L, 2, KVH, MaxT, Dh): same bytes, transposed; strides of multi_head_cache_attention_kernel.cc:149-155."""
+    b = workloads.Batch(8, 2, 128, [1, 1, 40], [77, 3, 0], 2, num_layer=3, layer_idx=2, name="layout3")
+    t = workloads.make_tensors(b, seed=54)
+    l0 = harness.run_oracle(b, t, cache_prefill=1)
+    l3 = harness.run_oracle(b, t, cache_prefill=1, layout=3)
+    assert np.array_equal(l0["output_f64"], l3["output_f64"])
+    assert np.array_equal(l0["cache"].transpose(1, 2, 3, 0, 4), l3["cache"])
+    assert np.array_equal(l0["scale"].view(np.uint16).transpose(1, 2, 3, 0, 4), l3["scale"].view(np.uint16))
