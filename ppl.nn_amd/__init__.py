@@ -82,6 +82,12 @@ def load_engine_library():
             "pplnn_hip_builder_preprocess": (u32, [vp]),
             "pplnn_hip_builder_create_runtime": (vp, [vp]),
             "pplnn_hip_builder_destroy": (None, [vp]),
+            "pplnn_hip_engine_configure_str": (u32, [vp, u32, ctypes.c_char_p]),
+            "pplnn_hip_runtime_set_inputs_from_files": (u32, [vp, ctypes.c_char_p]),
+            "pplnn_hip_runtime_save_outputs": (u32, [vp, ctypes.c_char_p]),
+            "pplnn_hip_builder_serialize_op": (u32, [vp, ctypes.c_char_p, vp, ctypes.c_uint64,
+                                                     ctypes.POINTER(ctypes.c_uint64)]),
+            "pplnn_hip_builder_deserialize_op": (u32, [vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_uint64]),
             "pplnn_hip_runtime_input_count": (u32, [vp]),
             "pplnn_hip_runtime_output_count": (u32, [vp]),
             "pplnn_hip_runtime_input": (vp, [vp, u32]),

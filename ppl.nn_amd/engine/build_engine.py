@@ -14,7 +14,7 @@ def build(force=False, verbose=False):
     os.makedirs(LIBDIR, exist_ok=True)
     out = os.path.join(LIBDIR, "libpplnn_llm_hip.so")
     srcs = [os.path.join(HERE, "src", s) for s in SOURCES]
-    deps = srcs + [os.path.join(HERE, "src", h) for h in ("core.h", "params.h", "arena.h")] + \
+    deps = srcs + [os.path.join(HERE, "src", h) for h in ("core.h", "params.h", "arena.h", "pmx_params.h")] + \
         [os.path.join(HERE, "include", "ppl", "nn", "llm_hip_api.h"),
          os.path.join(PKG, "..", "include", "ppl_llm_kernel_hip.h")]
     if not force and os.path.exists(out) and all(os.path.getmtime(d) <= os.path.getmtime(out) for d in deps):

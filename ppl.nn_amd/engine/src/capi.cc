@@ -1,5 +1,11 @@
 // Flat C entry points over the C++ engine API, for hosts without a C++ binding (the Python tests use them via ctypes).
 // Every function returns a ppl::common::RetCode or a handle (NULL on failure, text in pplnn_hip_last_error()).
+#include <cstring>
+#include <fstream>
+#include <iterator>
+#include <string>
+#include <vector>
+
 #include "arena.h"
 #include "core.h"
 
@@ -22,6 +28,9 @@ const char* pplnn_hip_engine_name(void* e) { return static_cast<Engine*>(e)->Get
 uint32_t pplnn_hip_engine_configure_u32(void* e, uint32_t option, uint32_t value) {
     return static_cast<Engine*>(e)->Configure(option, value);
 }
+uint32_t pplnn_hip_engine_configure_str(void* e, uint32_t option, const char* value) {
+    return static_cast<Engine*>(e)->Configure(option, value);
+}
 void pplnn_hip_engine_destroy(void* e) { delete static_cast<Engine*>(e); }
 
 // ---- builder
@@ -42,6 +51,29 @@ uint32_t pplnn_hip_builder_set_engine(void* b, void* engine) {
 uint32_t pplnn_hip_builder_preprocess(void* b) { return static_cast<onnx::RuntimeBuilder*>(b)->Preprocess(); }
 void* pplnn_hip_builder_create_runtime(void* b) { return static_cast<onnx::RuntimeBuilder*>(b)->CreateRuntime(); }
 void pplnn_hip_builder_destroy(void* b) { delete static_cast<onnx::RuntimeBuilder*>(b); }
+// PMX hooks of the op built for a node: its parameters as a FlatBuffers OpParam blob, and back
+uint32_t pplnn_hip_builder_serialize_op(void* b, const char* node_name, void* buf, uint64_t cap, uint64_t* size) {
+    auto op = FindOpOfBuilder(static_cast<onnx::RuntimeBuilder*>(b), node_name);
+    if (!op) {
+        LOG(ERROR) << "no op for node[" << node_name << "]";
+        return RC_NOT_FOUND;
+    }
+    std::string blob;
+    const RetCode rc = op->SerializeData(&blob);
+    if (rc != RC_SUCCESS) return rc;
+    *size = blob.size();
+    if (blob.size() > cap) return RC_OUT_OF_RANGE;
+    memcpy(buf, blob.data(), blob.size());
+    return RC_SUCCESS;
+}
+uint32_t pplnn_hip_builder_deserialize_op(void* b, const char* node_name, const void* buf, uint64_t size) {
+    auto op = FindOpOfBuilder(static_cast<onnx::RuntimeBuilder*>(b), node_name);
+    if (!op) {
+        LOG(ERROR) << "no op for node[" << node_name << "]";
+        return RC_NOT_FOUND;
+    }
+    return op->DeserializeData(buf, size);
+}
 
 // ---- runtime
 uint32_t pplnn_hip_runtime_input_count(void* r) { return static_cast<Runtime*>(r)->GetInputCount(); }
@@ -61,6 +93,109 @@ uint32_t pplnn_hip_runtime_profiling(void* r, uint64_t* micros, uint32_t* counts
         counts[i] = st.prof_info[i].exec_count;
     }
     return (uint32_t)st.prof_info.size();
+}
+// Step replay, file conventions of tools/pplnn_llm.cc: one file per graph input, comma separated, each named
+// "<anything>-<d0_d1_...>-<dtype>.dat" (SetShapedInputsOneByOne, :648-753: shape and type come from the NAME, the
+// bytes from the file); outputs go to "<dir>/pplnn_output-<tensor name>.dat" (SaveOutputsOneByOne, :796-822).
+uint32_t pplnn_hip_runtime_set_inputs_from_files(void* r, const char* files_csv) {
+    auto rt = static_cast<Runtime*>(r);
+    std::vector<std::string> files;
+    std::string cur;
+    for (const char* p = files_csv; ; ++p) {
+        if (*p == ',' || *p == 0) {
+            if (!cur.empty()) files.push_back(cur);
+            cur.clear();
+            if (*p == 0) break;
+        } else {
+            cur.push_back(*p);
+        }
+    }
+    if (files.size() != rt->GetInputCount()) {
+        LOG(ERROR) << "input file num[" << files.size() << "] != graph input num[" << rt->GetInputCount() << "]";
+        return RC_INVALID_VALUE;
+    }
+    for (uint32_t c = 0; c < files.size(); ++c) {
+        const std::string& path = files[c];
+        const size_t slash = path.find_last_of('/');
+        const std::string base = slash == std::string::npos ? path : path.substr(slash + 1);
+        std::vector<std::string> parts(1);
+        for (char ch : base) {
+            if (ch == '-') parts.emplace_back();
+            else parts.back().push_back(ch);
+        }
+        if (parts.size() != 3) {
+            LOG(ERROR) << "illegal file name format: " << base;
+            return RC_INVALID_VALUE;
+        }
+        const std::string dt_str = parts[2].substr(0, parts[2].find('.'));
+        datatype_t dt = DATATYPE_UNKNOWN;
+        for (uint32_t t = 0; t < 32; ++t)
+            if (dt_str == GetDataTypeStr((datatype_t)t) && dt_str != "unknown") dt = (datatype_t)t;
+        if (dt == DATATYPE_UNKNOWN) {
+            LOG(ERROR) << "cannot find data type[" << dt_str << "] in input file[" << base << "]";
+            return RC_INVALID_VALUE;
+        }
+        std::vector<int64_t> dims;
+        bool scalar = parts[1] == "scalar";
+        if (!scalar && parts[1] != "none") {
+            std::string d;
+            for (size_t i = 0; i <= parts[1].size(); ++i) {
+                if (i == parts[1].size() || parts[1][i] == '_') {
+                    if (d.empty()) {
+                        LOG(ERROR) << "illegal dim format.";
+                        return RC_INVALID_VALUE;
+                    }
+                    dims.push_back(atol(d.c_str()));
+                    d.clear();
+                } else {
+                    d.push_back(parts[1][i]);
+                }
+            }
+        }
+        auto t = rt->GetInputTensor(c);
+        t->GetShape()->SetDataType(dt);
+        if (scalar) t->GetShape()->ReshapeAsScalar();
+        else t->GetShape()->Reshape(dims.data(), (uint32_t)dims.size());
+        const uint64_t bytes = t->GetShape()->CalcBytesIncludingPadding();
+        if (bytes == 0) continue;
+        std::ifstream f(path, std::ios::binary);
+        if (!f) {
+            LOG(ERROR) << "mapping file[" << path << "] failed.";
+            return RC_NOT_FOUND;
+        }
+        std::string data((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+        if (data.size() < bytes) {
+            LOG(ERROR) << "input file[" << base << "] size(" << data.size() << ") is less than tensor[" << t->GetName()
+                       << "] size(" << bytes << ")";
+            return RC_INVALID_VALUE;
+        }
+        const RetCode rc = t->ConvertFromHost(data.data(), *t->GetShape());
+        if (rc != RC_SUCCESS) {
+            LOG(ERROR) << "set input[" << t->GetName() << "] failed: " << GetRetCodeStr(rc);
+            return rc;
+        }
+    }
+    return RC_SUCCESS;
+}
+uint32_t pplnn_hip_runtime_save_outputs(void* r, const char* dir) {
+    auto rt = static_cast<Runtime*>(r);
+    for (uint32_t c = 0; c < rt->GetOutputCount(); ++c) {
+        auto t = rt->GetOutputTensor(c);
+        std::vector<char> buffer(t->GetShape()->CalcBytesIncludingPadding());
+        const RetCode rc = t->ConvertToHost(buffer.data(), *t->GetShape());
+        if (rc != RC_SUCCESS) {
+            LOG(ERROR) << "convert data of tensor[" << t->GetName() << "] failed: " << GetRetCodeStr(rc);
+            return rc;
+        }
+        const std::string file = std::string(dir) + "/pplnn_output-" + t->GetName() + ".dat";
+        std::ofstream ofs(file, std::ios_base::out | std::ios_base::binary | std::ios_base::trunc);
+        if (!ofs.is_open()) {
+            LOG(ERROR) << "open output file[" << file << "]";
+            return RC_OTHER_ERROR;
+        }
+        ofs.write(buffer.data(), buffer.size());
+    }
+    return RC_SUCCESS;
 }
 void pplnn_hip_runtime_destroy(void* r) { delete static_cast<Runtime*>(r); }
 

@@ -194,6 +194,13 @@ public:
 };
 
 Device* GetSharedHostDevice(); // process-wide "cpu" device (malloc/free)
+class OptKernel;
+namespace onnx { class RuntimeBuilder; }
+// the op object Preprocess() built for the named node (nullptr before Preprocess or for an unknown name)
+OptKernel* FindOpOfBuilder(onnx::RuntimeBuilder* builder, const char* node_name);
+class TensorImpl;
+// "<tensor name with '/' replaced by '.'>-<dims joined by '_' | scalar | none>-<lower-case type name>.dat"
+std::string DumpFileTail(const TensorImpl* tensor);
 
 // ownership rules of src/ppl/nn/common/buffer_info.cc:65-113
 class BufferInfo final {
@@ -351,6 +358,13 @@ public:
     virtual ~OptKernel() {}
     const ir::Node* GetNode() const { return node_; }
     virtual KernelImpl* CreateKernelImpl() const = 0; // shared, read-only after Init
+    // PMX model hooks (src/ppl/nn/runtime/opt_kernel.h: SerializeData / DeserializeData): the op's parameters as a
+    // FlatBuffers OpParam blob. Ops without parameters write nothing.
+    virtual RetCode SerializeData(std::string* blob) const {
+        blob->clear();
+        return ppl::common::RC_SUCCESS;
+    }
+    virtual RetCode DeserializeData(const void*, uint64_t) { return ppl::common::RC_SUCCESS; }
 
 private:
     const ir::Node* node_;

@@ -10,10 +10,12 @@
 // All device arithmetic goes through the C ABI of libppl_llm_kernel_hip.so.
 #include <hip/hip_runtime.h>
 
+#include <fstream>
 #include <mutex>
 
 #include "arena.h"
 #include "params.h"
+#include "pmx_params.h"
 #include "ppl_llm_kernel_hip.h"
 
 using namespace ppl::common;
@@ -174,6 +176,10 @@ public:
                        << "] failed: " << hipGetErrorString(err);
             return RC_DEVICE_RUNTIME_ERROR;
         }
+        if (GetEngineConfig().enable_tensor_debug) { // kernel.cc:186-192
+            const RetCode drc = DumpOutputTensors(ctx, GetEngineConfig().debug_data_dir);
+            if (drc != RC_SUCCESS) return drc;
+        }
         return RC_SUCCESS;
     }
     uint64_t GetExecutionTime() const override {
@@ -187,6 +193,29 @@ public:
 
 protected:
     virtual RetCode DoExecute(KernelExecContext*) = 0;
+    // One file per output, named like the reference's debug dumps (engines/llm_cuda/kernel.cc:27-88) with this
+    // engine's tag: <dir>/pplnn_llm_hip_dbg_tensor-<tensor name, '/' -> '.'>-<d0_d1_...|scalar|none>-<dtype>.dat.
+    // The three '-'-separated parts are what the step-replay loader splits on (tools/pplnn_llm.cc:660-700).
+    static RetCode DumpOutputTensors(KernelExecContext* ctx, const std::string& dir) {
+        for (uint32_t i = 0; i < ctx->GetOutputCount(); ++i) {
+            auto tensor = ctx->GetOutput<TensorImpl>(i);
+            if (!tensor) continue;
+            const std::string file = dir + "/pplnn_llm_hip_dbg_tensor-" + DumpFileTail(tensor);
+            std::vector<char> host(tensor->GetShape()->CalcBytesExcludingPadding());
+            auto rc = tensor->ConvertToHost(host.data(), *tensor->GetShape());
+            if (rc != RC_SUCCESS) {
+                LOG(ERROR) << "convert data of tensor[" << tensor->GetName() << "] failed: " << GetRetCodeStr(rc);
+                return rc;
+            }
+            std::ofstream ofs(file, std::ios_base::out | std::ios_base::binary | std::ios_base::trunc);
+            if (!ofs.is_open()) {
+                LOG(ERROR) << "open output file[" << file << "] failed";
+                return RC_OTHER_ERROR;
+            }
+            ofs.write(host.data(), host.size());
+        }
+        return RC_SUCCESS;
+    }
     LlmHipDevice* GetHipDevice() const { return static_cast<LlmHipDevice*>(GetEngineContext()->GetDevice()); }
     hipStream_t GetStream() const { return GetHipDevice()->GetStream(); }
     const EngineConfig& GetEngineConfig() const { return *engine_config_; }
@@ -727,6 +756,15 @@ public:
         return new DynamicBatchingMultiHeadCacheAttentionKernel(GetNode(), cfg_, param_.get());
     }
 
+    RetCode SerializeData(std::string* blob) const override {
+        *blob = pmx::SerializeOpParam(*param_);
+        return RC_SUCCESS;
+    }
+    RetCode DeserializeData(const void* base, uint64_t size) override {
+        param_ = std::make_shared<opmx::MultiHeadCacheAttentionParam>();
+        return pmx::DeserializeOpParam(base, size, param_.get());
+    }
+
 private:
     std::shared_ptr<opmx::MultiHeadCacheAttentionParam> param_;
 };
@@ -740,6 +778,15 @@ public:
     }
     KernelImpl* CreateKernelImpl() const override {
         return new DynamicBatchingKeyValueCacheKernel(GetNode(), cfg_, param_.get());
+    }
+
+    RetCode SerializeData(std::string* blob) const override {
+        *blob = pmx::SerializeOpParam(*param_);
+        return RC_SUCCESS;
+    }
+    RetCode DeserializeData(const void* base, uint64_t size) override {
+        param_ = std::make_shared<opmx::KeyValueCacheParam>();
+        return pmx::DeserializeOpParam(base, size, param_.get());
     }
 
 private:
@@ -757,6 +804,15 @@ public:
         return new DynamicBatchingMultiHeadAttentionKernel(GetNode(), cfg_, param_.get());
     }
 
+    RetCode SerializeData(std::string* blob) const override {
+        *blob = pmx::SerializeOpParam(*param_);
+        return RC_SUCCESS;
+    }
+    RetCode DeserializeData(const void* base, uint64_t size) override {
+        param_ = std::make_shared<opmx::MultiHeadAttentionParam>();
+        return pmx::DeserializeOpParam(base, size, param_.get());
+    }
+
 private:
     std::shared_ptr<opmx::MultiHeadAttentionParam> param_;
 };
@@ -770,6 +826,15 @@ public:
     }
     KernelImpl* CreateKernelImpl() const override {
         return new DynamicBatchingRotaryPositionEmbeddingKernel(GetNode(), cfg_, param_.get());
+    }
+
+    RetCode SerializeData(std::string* blob) const override {
+        *blob = pmx::SerializeOpParam(*param_);
+        return RC_SUCCESS;
+    }
+    RetCode DeserializeData(const void* base, uint64_t size) override {
+        param_ = std::make_shared<opmx::RotaryPositionEmbeddingParam>();
+        return pmx::DeserializeOpParam(base, size, param_.get());
     }
 
 private:

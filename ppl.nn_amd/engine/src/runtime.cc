@@ -465,6 +465,17 @@ public:
         return rt;
     }
 
+    // the op object built for a node by Preprocess(), by node name
+    OptKernel* FindOp(const char* node_name) const {
+        if (!preprocessed_) return nullptr;
+        for (auto& node : info_->graph.topo->nodes) {
+            if (node.name != node_name) continue;
+            auto it = info_->partition.kernels.find(node.id);
+            return it == info_->partition.kernels.end() ? nullptr : it->second.get();
+        }
+        return nullptr;
+    }
+
 private:
     std::shared_ptr<RuntimeGraphInfo> info_;
     std::vector<Engine*> engines_;
@@ -472,6 +483,29 @@ private:
 };
 
 } // namespace
+
+std::string DumpFileTail(const TensorImpl* tensor) {
+    auto shape = tensor->GetShape();
+    std::string name = tensor->GetName();
+    for (auto& c : name)
+        if (c == '/') c = '.';
+    std::string dims;
+    if (shape->IsScalar()) {
+        dims = "scalar";
+    } else if (shape->GetRealDimCount() == 0) {
+        dims = "none";
+    } else {
+        dims = std::to_string(shape->GetDim(0));
+        for (uint32_t i = 1; i < shape->GetDimCount(); ++i) dims += "_" + std::to_string(shape->GetDim(i));
+    }
+    std::string dt = ppl::common::GetDataTypeStr(shape->GetDataType());
+    for (auto& c : dt) c = (char)tolower(c);
+    return name + "-" + dims + "-" + dt + ".dat";
+}
+
+OptKernel* FindOpOfBuilder(onnx::RuntimeBuilder* builder, const char* node_name) {
+    return static_cast<RuntimeBuilderImpl*>(builder)->FindOp(node_name);
+}
 
 onnx::RuntimeBuilder* onnx::RuntimeBuilderFactory::Create() {
     return new RuntimeBuilderImpl();

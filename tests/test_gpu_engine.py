@@ -306,3 +306,60 @@ def test_paged_mhca_graph_through_the_engine(hiplib):
     torch.cuda.synchronize()
     assert np.array_equal(cache.cpu().numpy(), ref["cache"])
     s.close()
+
+
+def test_debug_dumps_and_step_replay(hiplib, tmp_path):
+    """ENGINE_CONF_TENSOR_DEBUG / ENGINE_CONF_DEBUG_DATA_DIR dump every kernel's outputs as
+    <dir>/pplnn_llm_hip_dbg_tensor-<name>-<dims>-<dtype>.dat; a step is replayed from files named
+    <name>-<dims>-<dtype>.dat and its outputs saved as pplnn_output-<name>.dat (conventions of tools/pplnn_llm.cc)."""
+    import torch
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(8, 2, 128, [1, 1, 30], [40, 7, 0], 2, name="replay")
+    t = workloads.make_tensors(b, seed=71)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    torch.cuda.synchronize()
+    host = dict(query=t["query"], current_key=t["current_key"], current_value=t["current_value"],
+                seqstarts=b.seqstarts, kvstarts=b.kvstarts, cachestarts=b.cachestarts, start_pos=b.start_pos,
+                decoding_batches=np.array(b.decoding_batches, np.int64), max_seqlen=np.array(b.max_seqlen, np.int64),
+                max_kvlen=np.array(b.max_kvlen, np.int64), cache=cache.cpu().numpy(),
+                scale=scale.cpu().view(torch.int16).numpy().view(np.float16))
+    dt = {np.dtype(np.float16): "fp16", np.dtype(np.int64): "int64", np.dtype(np.int8): "int8"}
+    files = []
+    for name in ow.MHCA_INPUTS:
+        a = np.ascontiguousarray(host[name])
+        dims = "scalar" if a.ndim == 0 else "_".join(str(d) for d in a.shape)
+        f = tmp_path / f"step0_{name}-{dims}-{dt[a.dtype]}.dat"
+        a.tofile(f)
+        files.append(str(f))
+    dbg = tmp_path / "dbg"
+    dbg.mkdir()
+    s = Session(eng, ow.rope_mhca_model(8, 2, 128, 1, 0, 10000.0))
+    # options are read by kernels at run time from the engine's configuration
+    assert eng.pplnn_hip_engine_configure_u32(s.engine, 2, 1) == 0
+    assert eng.pplnn_hip_engine_configure_str(s.engine, 3, str(dbg).encode()) == 0
+    for i in (7, 8, 9):
+        eng.pplnn_hip_tensor_use_host_device(s.input(i))
+    assert eng.pplnn_hip_runtime_set_inputs_from_files(s.rt, ",".join(files).encode()) == 0, eng.pplnn_hip_last_error()
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    out = s.output(0, np.float16)
+    S = b.total_new_tokens
+    names = sorted(p.name for p in dbg.iterdir())
+    assert names == [f"pplnn_llm_hip_dbg_tensor-attn_output-{S}_8_128-fp16.dat",
+                     f"pplnn_llm_hip_dbg_tensor-rotated_key-{S}_2_128-fp16.dat",
+                     f"pplnn_llm_hip_dbg_tensor-rotated_query-{S}_8_128-fp16.dat"]
+    dumped = np.fromfile(dbg / names[0], np.float16).reshape(S, 8, 128)
+    assert np.array_equal(dumped.view(np.uint16), out.view(np.uint16))
+    assert eng.pplnn_hip_runtime_save_outputs(s.rt, str(tmp_path).encode()) == 0
+    saved = np.fromfile(tmp_path / "pplnn_output-attn_output.dat", np.float16).reshape(S, 8, 128)
+    assert np.array_equal(saved.view(np.uint16), out.view(np.uint16))
+    # the replayed step equals the same step driven through tensors (RoPE, then attention, against the oracle)
+    import oracle
+    rq, rk = _rope_on_oracle(oracle.lib(), t["query"], t["current_key"], b, 10000.0)
+    ref = harness.run_oracle(b, dict(t, query=rq, current_key=rk))
+    harness.assert_attn_close(out, ref["output_f64"], abs_tol=3e-3)
+    # error conventions of the loader
+    assert eng.pplnn_hip_runtime_set_inputs_from_files(s.rt, files[0].encode()) == cabi.RC_INVALID_VALUE  # count
+    bad = list(files)
+    bad[0] = str(tmp_path / "query.dat")
+    assert eng.pplnn_hip_runtime_set_inputs_from_files(s.rt, ",".join(bad).encode()) == cabi.RC_INVALID_VALUE  # name
+    s.close()
