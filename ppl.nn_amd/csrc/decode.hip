@@ -415,27 +415,93 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         b += __builtin_popcountll(__ballot(ends_before));
     }
     b = __builtin_amdgcn_readfirstlane(b);
-    for (int64_t pos = r0; pos < r1; ++b) {
-        // ---- segment = the part of sequence b inside this range, as token positions of that sequence
+
+    // A segment = the part of one sequence inside this range; this wave's share of it is tokens [t_begin, t_end).
+    struct Segment {
+        int b;
+        int64_t seg_end, qrow, t_begin;
+        bool whole_sequence;
+        const int64_t* page_row; // paged slab: the sequence's row of the page table
+        const char* cbase; // contiguous slab: K row of token t_begin (this kv head) in the cache / scale tensors
+        const char* sbase;
+        int n_stages, tail_rows_mem, tail_rows_valid;
+    };
+    const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
+    int64_t pos = r0;
+    auto next_segment = [&](Segment& g) { // consumes sequence b from position pos on
         const int64_t seq_lo = p.kvstarts[b], seq_hi = p.kvstarts[b + 1];
         const int64_t seg_begin = pos - seq_lo;
-        const int64_t seg_end = ((r1 < seq_hi) ? r1 : seq_hi) - seq_lo;
-        pos = seq_lo + seg_end;
-        const bool whole_sequence = seg_begin == 0 && seg_end == seq_hi - seq_lo;
-        // contiguous slab region of the sequence, or its row of the page table
-        const int64_t tok0 = PAGED ? 0 : p.cachestarts[b];
-        const int64_t* page_row = PAGED ? p.cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
-        const int64_t qrow = p.seqstarts[b];
-        int64_t sub = (seg_end - seg_begin + tsplits - 1) / tsplits;
+        g.b = b;
+        g.seg_end = ((r1 < seq_hi) ? r1 : seq_hi) - seq_lo;
+        g.whole_sequence = seg_begin == 0 && g.seg_end == seq_hi - seq_lo;
+        g.page_row = PAGED ? p.cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
+        g.qrow = p.seqstarts[b];
+        int64_t sub = (g.seg_end - seg_begin + tsplits - 1) / tsplits;
         sub = (sub + kStageTokens - 1) / kStageTokens * kStageTokens;
-        const int64_t t_begin = seg_begin + (int64_t)ts * sub;
-        const int64_t t_end = (t_begin + sub < seg_end) ? t_begin + sub : seg_end; // may be <= t_begin: no tokens
+        g.t_begin = seg_begin + (int64_t)ts * sub;
+        const int64_t t_end = (g.t_begin + sub < g.seg_end) ? g.t_begin + sub : g.seg_end; // may be <= t_begin: none
+        g.n_stages = t_end > g.t_begin ? (int)((t_end - g.t_begin + kStageTokens - 1) / kStageTokens) : 0;
+        // The wave's last stage may overhang: rows past the end of the SEGMENT are clamped onto its last row (loads
+        // must stay inside memory the sequence owns) and everything past the wave's own range is masked.
+        const int64_t last_stage_t0 = g.t_begin + (int64_t)(g.n_stages - 1) * kStageTokens;
+        g.tail_rows_mem =
+            (int)((g.seg_end - last_stage_t0) < kStageTokens ? (g.seg_end - last_stage_t0) : kStageTokens);
+        g.tail_rows_valid = (int)(t_end - last_stage_t0);
+        const int64_t row0 = (PAGED ? 0 : (p.cachestarts[b] + g.t_begin) * (int64_t)stride) + head_off;
+        g.cbase = reinterpret_cast<const char*>(p.cache) + row0;
+        g.sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
+        pos = seq_lo + g.seg_end;
+        ++b;
+    };
+    // enqueues stage idx of segment g into stage buffer `slot`
+    auto issue_with = [&](const Segment& g, int idx, int slot, const DmaOffsets& off, int rows_mem) {
+        char* dst = wave_lds + slot * kStageBytes;
+        if (PAGED) {
+            // a stage of 32 tokens touches at most two pages (pages hold >= 64 tokens)
+            const int64_t t0 = g.t_begin + (int64_t)idx * kStageTokens;
+            const int64_t in_page = t0 & ((int64_t(1) << p.page_shift) - 1);
+            const int64_t left = (int64_t(1) << p.page_shift) - in_page; // rows of the stage in its first page
+            const int split = left < kStageTokens ? (int)left : kStageTokens;
+            const int64_t pa = g.page_row[t0 >> p.page_shift];
+            // the second page exists whenever one of the stage's (clamped) rows lies in it
+            const int64_t pb = split < rows_mem ? g.page_row[(t0 >> p.page_shift) + 1] : pa;
+            const int64_t ra = (pa + in_page) * (int64_t)stride + head_off;
+            const int64_t rb = (pb - split) * (int64_t)stride + head_off;
+            const char* ca = make_uniform(reinterpret_cast<const char*>(p.cache) + ra);
+            const char* cb = make_uniform(reinterpret_cast<const char*>(p.cache) + rb);
+            const char* sa = make_uniform(reinterpret_cast<const char*>(p.scale) + (ra / kQuantGroup) * 2);
+            const char* sb = make_uniform(reinterpret_cast<const char*>(p.scale) + (rb / kQuantGroup) * 2);
+            dma_stage_paged(dst, ca, cb, sa, sb, split, off, kv_off, kv_off_s);
+        } else {
+            const char* cb = make_uniform(g.cbase + idx * step_c);
+            const char* sb = make_uniform(g.sbase + idx * step_s);
+            dma_stage(dst, cb, sb, off, kv_off, kv_off_s);
+        }
+    };
+    auto issue = [&](const Segment& g, int idx, int slot) {
+        if (idx == g.n_stages - 1 && g.tail_rows_mem < kStageTokens) { // wave-uniform, at most once per segment
+            DmaOffsets tail;
+            make_dma_offsets(tail, lane, stride, sstride_b, g.tail_rows_mem);
+            issue_with(g, idx, slot, tail, g.tail_rows_mem);
+        } else {
+            issue_with(g, idx, slot, full, kStageTokens);
+        }
+    };
 
+    // When every wave owns a whole kv head (no token split inside the workgroup) nothing is combined through LDS, the
+    // stage buffers stay private to their wave, and the first stage of the NEXT segment is put in flight before the
+    // current segment's results are normalised and stored: the transition between two sequences costs no DMA bubble.
+    const bool direct = tsplits == 1;
+    Segment cur, nxt;
+    next_segment(cur);
+    int slot0 = 0; // stage buffer of the current segment's stage 0
+    bool cur_in_flight = false; // stage 0 of `cur` already enqueued by the previous segment's last iteration
+    for (;;) {
         // ---- Q^T as the B operand, kept for the whole segment: qB[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
         half8_t qB[2][2];
         {
             const bool live = m < p.rep;
-            const half_t* qp = p.q + ((qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
+            const half_t* qp = p.q + ((cur.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
@@ -452,114 +518,122 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         ss.m_run = -INFINITY;
         ss.l_part = 0.f;
 
-        if (t_begin < t_end) {
-            const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
-            const int64_t row0 = p.addr.row(tok0 + t_begin, 0, kvh);
-            const char* cbase = reinterpret_cast<const char*>(p.cache) + row0;
-            const char* sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
-            // The wave's last stage may overhang: rows past the end of the SEGMENT are clamped onto its last row (loads
-            // must stay inside memory the sequence owns) and everything past the wave's own range is masked.
-            const int n_stages = (int)((t_end - t_begin + kStageTokens - 1) / kStageTokens);
-            const int64_t last_stage_t0 = t_begin + (int64_t)(n_stages - 1) * kStageTokens;
-            const int tail_rows_mem =
-                (int)((seg_end - last_stage_t0) < kStageTokens ? (seg_end - last_stage_t0) : kStageTokens);
-            const int tail_rows_valid = (int)(t_end - last_stage_t0);
-            auto issue_with = [&](int idx, const DmaOffsets& off, int rows_mem) {
-                char* dst = wave_lds + (idx & 1) * kStageBytes;
-                if (PAGED) {
-                    // a stage of 32 tokens touches at most two pages (pages hold >= 64 tokens)
-                    const int64_t t0 = t_begin + (int64_t)idx * kStageTokens;
-                    const int64_t in_page = t0 & ((int64_t(1) << p.page_shift) - 1);
-                    const int64_t left = (int64_t(1) << p.page_shift) - in_page; // rows of the stage in its first page
-                    const int split = left < kStageTokens ? (int)left : kStageTokens;
-                    const int64_t pa = page_row[t0 >> p.page_shift];
-                    // the second page exists whenever one of the stage's (clamped) rows lies in it
-                    const int64_t pb = split < rows_mem ? page_row[(t0 >> p.page_shift) + 1] : pa;
-                    const int64_t ra = (pa + in_page) * (int64_t)stride + head_off;
-                    const int64_t rb = (pb - split) * (int64_t)stride + head_off;
-                    const char* ca = make_uniform(reinterpret_cast<const char*>(p.cache) + ra);
-                    const char* cb = make_uniform(reinterpret_cast<const char*>(p.cache) + rb);
-                    const char* sa = make_uniform(reinterpret_cast<const char*>(p.scale) + (ra / kQuantGroup) * 2);
-                    const char* sb = make_uniform(reinterpret_cast<const char*>(p.scale) + (rb / kQuantGroup) * 2);
-                    dma_stage_paged(dst, ca, cb, sa, sb, split, off, kv_off, kv_off_s);
+        bool has_next = false;
+        if (cur.n_stages > 0) {
+            if (!cur_in_flight) issue(cur, 0, slot0);
+            for (int it = 0; it < cur.n_stages; ++it) {
+                const int slot = (slot0 + it) & 1;
+                // the buffer the next stage lands in was last read by compute(it-1), which has finished in program order
+                if (it + 1 < cur.n_stages) {
+                    issue(cur, it + 1, slot ^ 1);
+                    // everything older than the transfers just enqueued has landed: stage `it`, and at it == 0 the
+                    // query loads (global stores still in flight only make this wait longer, never shorter)
+                    PPLHIP_WAIT_VMCNT(kDmaPerStage);
                 } else {
-                    const char* cb = make_uniform(cbase + idx * step_c);
-                    const char* sb = make_uniform(sbase + idx * step_s);
-                    dma_stage(dst, cb, sb, off, kv_off, kv_off_s);
-                }
-            };
-            auto issue = [&](int idx) {
-                if (idx == n_stages - 1 && tail_rows_mem < kStageTokens) { // wave-uniform, at most once per segment
-                    DmaOffsets tail;
-                    make_dma_offsets(tail, lane, stride, sstride_b, tail_rows_mem);
-                    issue_with(idx, tail, tail_rows_mem);
-                } else {
-                    issue_with(idx, full, kStageTokens);
-                }
-            };
-
-            issue(0);
-            // The query loads are older than stage 0's transfers: retire them here, with stage 0 already in flight, so
-            // that no full drain of the DMA queue is needed at their first use inside the loop.
-            PPLHIP_WAIT_VMCNT(kDmaPerStage);
-            for (int it = 0; it < n_stages; ++it) {
-                // the buffer stage it+1 lands in was last read by compute(it-1), which has finished in program order
-                if (it + 1 < n_stages) {
-                    issue(it + 1);
-                    PPLHIP_WAIT_VMCNT(kDmaPerStage); // everything but the transfers just enqueued has landed
-                } else {
-                    PPLHIP_WAIT_VMCNT(0);
+                    has_next = direct && pos < r1;
+                    if (has_next) {
+                        next_segment(nxt);
+                        issue(nxt, 0, slot ^ 1);
+                        PPLHIP_WAIT_VMCNT(kDmaPerStage);
+                    } else {
+                        PPLHIP_WAIT_VMCNT(0);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                compute_stage(wave_lds_addr + (it & 1) * kStageBytes, ro, ss, qB, kq,
-                              it + 1 == n_stages ? tail_rows_valid : kStageTokens, p.score_scale);
+                compute_stage(wave_lds_addr + slot * kStageBytes, ro, ss, qB, kq,
+                              it + 1 == cur.n_stages ? cur.tail_rows_valid : kStageTokens, p.score_scale);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         const float l_tot = wave_sum_over_quads(ss.l_part);
 
-        // ---- combine the token splits of each kv head: LDS layout [wave][head][Dh + 2] (acc, then max, sum), reusing
-        // the stage buffers
-        __syncthreads();
-        if (m < p.rep) {
-            float* dst = lds + ((size_t)wave * p.rep + m) * row_f;
+        if (direct) {
+            // ---- straight from registers: lane (m, kq) holds channels 8*(4*kq + e) .. +7 of query head m in oacc[.][e]
+            if (m < p.rep) {
+                const int head = kvh * p.rep + m;
+                if (cur.whole_sequence) {
+                    half_t* dst = p.out + (cur.qrow * p.num_heads + head) * kDh + 32 * kq;
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+                    for (int e = 0; e < 4; ++e) {
+                        half_t o[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) dst[8 * (4 * kq + e) + i] = ss.oacc[i][e];
-            if (kq == 0) {
-                dst[kDh] = ss.m_run;
-                dst[kDh + 1] = l_tot;
-            }
-        }
-        __syncthreads();
-        const int n_out = p.hpb * p.rep * kDh; // (kv head of the group, query head of the kv head, channel)
-        for (int idx = threadIdx.x; idx < n_out; idx += kDecodeWaves * kWave) {
-            const int d = idx & (kDh - 1);
-            const int hh = idx >> 7; // kv_local * rep + h
-            const int kl = hh / p.rep, h = hh - kl * p.rep;
-            float mx = -INFINITY;
-            for (int t = 0; t < tsplits; ++t) mx = fmaxf(mx, lds[((size_t)(t * p.hpb + kl) * p.rep + h) * row_f + kDh]);
-            float acc = 0.f, l = 0.f;
-            for (int t = 0; t < tsplits; ++t) {
-                const float* src = lds + ((size_t)(t * p.hpb + kl) * p.rep + h) * row_f;
-                const float wgt = __builtin_amdgcn_exp2f(src[kDh] - mx); // a wave without tokens has max -inf -> 0
-                acc += wgt * src[d];
-                l += wgt * src[kDh + 1];
-            }
-            const int head = (hg * p.hpb + kl) * p.rep + h;
-            if (whole_sequence) {
-                p.out[(qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
-            } else {
-                const int64_t prow = (s_idx + b) * p.num_heads + head;
-                p.part_acc[prow * kDh + d] = acc;
-                if (d == 0) {
-                    p.part_ml[prow * 2 + 0] = mx;
-                    p.part_ml[prow * 2 + 1] = l;
+                        for (int i = 0; i < 8; ++i) o[i] = (half_t)(ss.oacc[i][e] / l_tot);
+                        uint4 packed;
+                        __builtin_memcpy(&packed, o, 16);
+                        *reinterpret_cast<uint4*>(dst + 8 * e) = packed;
+                    }
+                } else {
+                    const int64_t prow = (s_idx + cur.b) * p.num_heads + head;
+                    float* dst = p.part_acc + prow * kDh + 32 * kq;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        *reinterpret_cast<float4_t*>(dst + 8 * e) =
+                            float4_t{ss.oacc[0][e], ss.oacc[1][e], ss.oacc[2][e], ss.oacc[3][e]};
+                        *reinterpret_cast<float4_t*>(dst + 8 * e + 4) =
+                            float4_t{ss.oacc[4][e], ss.oacc[5][e], ss.oacc[6][e], ss.oacc[7][e]};
+                    }
+                    if (kq == 0) {
+                        p.part_ml[prow * 2 + 0] = ss.m_run;
+                        p.part_ml[prow * 2 + 1] = l_tot;
+                    }
                 }
             }
+        } else {
+            // ---- combine the token splits of each kv head: LDS layout [wave][head][Dh + 2] (acc, then max, sum),
+            // reusing the stage buffers
+            __syncthreads();
+            if (m < p.rep) {
+                float* dst = lds + ((size_t)wave * p.rep + m) * row_f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) dst[8 * (4 * kq + e) + i] = ss.oacc[i][e];
+                if (kq == 0) {
+                    dst[kDh] = ss.m_run;
+                    dst[kDh + 1] = l_tot;
+                }
+            }
+            __syncthreads();
+            const int n_out = p.hpb * p.rep * kDh; // (kv head of the group, query head of the kv head, channel)
+            for (int idx = threadIdx.x; idx < n_out; idx += kDecodeWaves * kWave) {
+                const int d = idx & (kDh - 1);
+                const int hh = idx >> 7; // kv_local * rep + h
+                const int kl = hh / p.rep, h = hh - kl * p.rep;
+                float mx = -INFINITY;
+                for (int t = 0; t < tsplits; ++t)
+                    mx = fmaxf(mx, lds[((size_t)(t * p.hpb + kl) * p.rep + h) * row_f + kDh]);
+                float acc = 0.f, l = 0.f;
+                for (int t = 0; t < tsplits; ++t) {
+                    const float* src = lds + ((size_t)(t * p.hpb + kl) * p.rep + h) * row_f;
+                    const float wgt = __builtin_amdgcn_exp2f(src[kDh] - mx); // a wave without tokens: max -inf -> 0
+                    acc += wgt * src[d];
+                    l += wgt * src[kDh + 1];
+                }
+                const int head = (hg * p.hpb + kl) * p.rep + h;
+                if (cur.whole_sequence) {
+                    p.out[(cur.qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
+                } else {
+                    const int64_t prow = (s_idx + cur.b) * p.num_heads + head;
+                    p.part_acc[prow * kDh + d] = acc;
+                    if (d == 0) {
+                        p.part_ml[prow * 2 + 0] = mx;
+                        p.part_ml[prow * 2 + 1] = l;
+                    }
+                }
+            }
+            __syncthreads(); // the next segment's transfers overwrite the combine area
         }
-        __syncthreads(); // the next segment's transfers overwrite the combine area
+
+        if (has_next) { // its stage 0 is already in flight, in the buffer the last stage did not use
+            slot0 = (slot0 + cur.n_stages) & 1;
+            cur = nxt;
+            cur_in_flight = true;
+        } else {
+            if (pos >= r1) break;
+            next_segment(cur);
+            slot0 = 0;
+            cur_in_flight = false;
+        }
     }
 }
 
