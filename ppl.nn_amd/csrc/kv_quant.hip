@@ -59,7 +59,13 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     const int r2 = r - kv * per_kv;
     const int head = r2 / gph;
     const int grp = r2 - head * gph;
-    const int b = find_sequence(p.seqstarts, p.batch, t);
+    // decode sequences come first and hold one token each, so for them the packed token index IS the sequence index:
+    // two independent loads settle it; only prompt tokens pay for the binary search (a chain of dependent loads)
+    int b;
+    if (t < p.batch && p.seqstarts[t] == t && p.seqstarts[t + 1] == t + 1)
+        b = (int)t;
+    else
+        b = find_sequence(p.seqstarts, p.batch, t);
     const int64_t tok = p.pages.token(b, p.start_pos[b] + (t - p.seqstarts[b]));
     const half_t* src = (kv ? p.value : p.key) + ((t * p.kv_heads + head) * gph + grp) * 8;
     const uint4 raw = *reinterpret_cast<const uint4*>(src);
