@@ -35,6 +35,7 @@ def parse():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--split-k", type=int, default=1)
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the cfg1 / cfg3 decode runs")
     ap.add_argument("--no-churn", action="store_true", help="skip the cfg4 continuous-batching churn run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy (the reference point for scaling the "
@@ -365,6 +366,22 @@ def main():
         del dec.slabs[1:], dec.args[1:]
         torch.cuda.empty_cache()
         result["churn_cfg4"] = churn_cfg4(pkg, lib)
+    if args.workload == "cfg2" and not args.no_other_configs:
+        # the other decode configurations at their full sizes, same timing loop, shorter runs
+        others = {}
+        for name, ob in (("cfg1 Llama-2-7B pure decode (H32/KVH32/Dh128): 64 seqs kv~U[128,2048]",
+                          workloads.cfg1_llama2_7b_decode()),
+                         ("cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]",
+                          workloads.cfg3_long_context())):
+            odb = DeviceBatch(pkg, lib, ob, seed=4, n_slabs=N_SLABS)
+            o_wall, o_ev = timed(odb, max(args.steps // 2, 10), max(args.warmup // 2, 3))
+            o_gbs = ob.decode_bytes() / (o_ev * 1e-3) / 1e9
+            others[name] = {"tokens_per_s": ob.decoding_batches / (o_wall * 1e-3), "ms_per_step": o_wall,
+                            "achieved_GBs": o_gbs, "frac_of_hbm_peak": o_gbs / HBM_PEAK_GBS,
+                            "kv_tokens": int(ob.kvlens.sum()), "decode_ranges": int(odb.plan.decode_num_ranges)}
+            del odb
+            torch.cuda.empty_cache()
+        result["other_decode_configs"] = others
     if args.copy_calibration:
         copy_calibration()
     if not args.no_cpu_baseline:

@@ -637,44 +637,54 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     }
 }
 
-// One workgroup of 256 lanes per decode sequence: lane = (query head slot, 16-channel slice); every lane walks the
-// sequence's partial slots (one per range the sequence touches, consecutive by construction) and keeps its own
-// running (max, sum, acc): out[d] = sum_s w_s acc_s[d] / sum_s w_s l_s with w_s = exp2(m_s - max_s m_s). No LDS, no
-// barrier; the launch is small (one workgroup per sequence) because its cost is launch latency, not bandwidth.
-// Sequences that lie inside a single range were already written by the decode kernel.
+// One workgroup of 256 lanes per (decode sequence, query head): 8 groups of 32 lanes stride over the partial slots of
+// the sequence (one per range it touches), each lane owning 4 channels; the groups' running (max, sum, acc) are combined
+// through LDS. out[d] = sum_s w_s acc_s[d] / sum_s w_s l_s with w_s = exp2(m_s - max_s m_s). Sequences that lie inside a
+// single range were already written by the decode kernel.
+constexpr int kMergeGroups = 8;
 __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p) {
-    const int b = blockIdx.x;
+    __shared__ float red[kMergeGroups][kDh + 2];
+    const int b = blockIdx.y;
+    const int head = blockIdx.x;
+    const int g = threadIdx.x >> 5;
+    const int d4 = (threadIdx.x & 31) * 4;
     const int64_t R = range_tokens(p.kvstarts[p.nd], p.num_ranges);
     const int64_t s_lo = p.kvstarts[b] / R, s_hi = (p.kvstarts[b + 1] - 1) / R;
     if (s_lo == s_hi) return;
-    const int64_t qrow = p.seqstarts[b];
-    const int slice = threadIdx.x & 7; // channels 16 * slice .. +15
-    for (int head = threadIdx.x >> 3; head < p.num_heads; head += 32) {
-        float mx = -INFINITY, l = 0.f;
-        float4_t acc[4];
+    float mx = -INFINITY, l = 0.f;
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t s = s_lo + g; s <= s_hi; s += kMergeGroups) {
+        const int64_t prow = (s + b) * p.num_heads + head;
+        const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
+        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
+        const float m_new = fmaxf(mx, mc);
+        const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc - m_new);
+        acc = acc * w_old + a * w_new;
+        l = l * w_old + lc * w_new;
+        mx = m_new;
+    }
+    red[g][d4 + 0] = acc[0];
+    red[g][d4 + 1] = acc[1];
+    red[g][d4 + 2] = acc[2];
+    red[g][d4 + 3] = acc[3];
+    if ((threadIdx.x & 31) == 0) {
+        red[g][kDh] = mx;
+        red[g][kDh + 1] = l;
+    }
+    __syncthreads();
+    if (threadIdx.x < kDh) {
+        const int d = threadIdx.x;
+        float M = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-        for (int64_t s = s_lo; s <= s_hi; ++s) {
-            const int64_t prow = (s + b) * p.num_heads + head;
-            const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
-            const float4_t* src = reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + 16 * slice);
-            const float m_new = fmaxf(mx, mc);
-            const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc - m_new);
+        for (int i = 0; i < kMergeGroups; ++i) M = fmaxf(M, red[i][kDh]);
+        float a = 0.f, L = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] = acc[i] * w_old + src[i] * w_new;
-            l = l * w_old + lc * w_new;
-            mx = m_new;
+        for (int i = 0; i < kMergeGroups; ++i) {
+            const float w = __builtin_amdgcn_exp2f(red[i][kDh] - M); // groups that saw no slot have max -inf -> 0
+            a += w * red[i][d];
+            L += w * red[i][kDh + 1];
         }
-        half_t o[16];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) o[4 * i + e] = (half_t)(acc[i][e] / l);
-        uint4 packed[2];
-        __builtin_memcpy(packed, o, 32);
-        uint4* dst = reinterpret_cast<uint4*>(p.out + (qrow * p.num_heads + head) * kDh + 16 * slice);
-        dst[0] = packed[0];
-        dst[1] = packed[1];
+        p.out[(p.seqstarts[b] * p.num_heads + head) * kDh + d] = (half_t)(a / L);
     }
 }
 
@@ -740,7 +750,7 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
         hipLaunchKernelGGL(decode_int8kv_kernel<false>, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes,
                            stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
-    hipLaunchKernelGGL(decode_merge_kernel, dim3(nd), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_merge");
     return PPLHIP_RC_SUCCESS;
 }
