@@ -488,6 +488,21 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         }
     };
 
+    // Q^T as the B operand, kept for a whole segment: q[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
+    constexpr int kQueryLoads = 4;
+    auto load_query = [&](const Segment& g, half8_t (&q)[2][2]) {
+        const bool live = m < p.rep;
+        const half_t* qp = p.q + ((g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                uint4 x = *reinterpret_cast<const uint4*>(qp + 32 * kq + 16 * jj + 8 * i);
+                if (!live) x = make_uint4(0, 0, 0, 0);
+                __builtin_memcpy(&q[jj][i], &x, 16);
+            }
+    };
+
     // When every wave owns a whole kv head (no token split inside the workgroup) nothing is combined through LDS, the
     // stage buffers stay private to their wave, and the first stage of the NEXT segment is put in flight before the
     // current segment's results are normalised and stored: the transition between two sequences costs no DMA bubble.
@@ -496,22 +511,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     next_segment(cur);
     int slot0 = 0; // stage buffer of the current segment's stage 0
     bool cur_in_flight = false; // stage 0 of `cur` already enqueued by the previous segment's last iteration
+    half8_t qB[2][2], qN[2][2];
+    load_query(cur, qB);
     for (;;) {
-        // ---- Q^T as the B operand, kept for the whole segment: qB[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
-        half8_t qB[2][2];
-        {
-            const bool live = m < p.rep;
-            const half_t* qp = p.q + ((cur.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    uint4 x = *reinterpret_cast<const uint4*>(qp + 32 * kq + 16 * jj + 8 * i);
-                    if (!live) x = make_uint4(0, 0, 0, 0);
-                    __builtin_memcpy(&qB[jj][i], &x, 16);
-                }
-        }
-
         SoftmaxState ss;
 #pragma unroll
         for (int i = 0; i < 8; ++i) ss.oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -533,8 +535,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                     has_next = direct && pos < r1;
                     if (has_next) {
                         next_segment(nxt);
+                        load_query(nxt, qN); // older than the transfers below: landed before they are waited for
                         issue(nxt, 0, slot ^ 1);
-                        PPLHIP_WAIT_VMCNT(kDmaPerStage);
+                        PPLHIP_WAIT_VMCNT(kDmaPerStage + kQueryLoads); // stage `it` only
                     } else {
                         PPLHIP_WAIT_VMCNT(0);
                     }
@@ -553,11 +556,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                 const int head = kvh * p.rep + m;
                 if (cur.whole_sequence) {
                     half_t* dst = p.out + (cur.qrow * p.num_heads + head) * kDh + 32 * kq;
+                    const float inv_l = 1.0f / l_tot;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         half_t o[8];
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) o[i] = (half_t)(ss.oacc[i][e] / l_tot);
+                        for (int i = 0; i < 8; ++i) o[i] = (half_t)(ss.oacc[i][e] * inv_l);
                         uint4 packed;
                         __builtin_memcpy(&packed, o, 16);
                         *reinterpret_cast<uint4*>(dst + 8 * e) = packed;
@@ -627,10 +631,15 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         if (has_next) { // its stage 0 is already in flight, in the buffer the last stage did not use
             slot0 = (slot0 + cur.n_stages) & 1;
             cur = nxt;
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) qB[jj][i] = qN[jj][i];
             cur_in_flight = true;
         } else {
             if (pos >= r1) break;
             next_segment(cur);
+            load_query(cur, qB);
             slot0 = 0;
             cur_in_flight = false;
         }
