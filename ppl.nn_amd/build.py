@@ -30,7 +30,8 @@ def build_kernels(force=False, verbose=False):
     os.makedirs(LIBDIR, exist_ok=True)
     out = os.path.join(LIBDIR, "libppl_llm_kernel_hip.so")
     srcs = [os.path.join(CSRC, s) for s in KERNEL_SOURCES]
-    deps = srcs + [os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip.h")]
+    deps = srcs + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "exports.map"),
+                   os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip.h")]
     if not force and not _newer(out, deps):
         return out
     objs = []
@@ -53,7 +54,8 @@ def build_kernels(force=False, verbose=False):
             print(txt)
     if failed:
         raise RuntimeError("hipcc failed")
-    subprocess.check_call([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", out] + objs)
+    subprocess.check_call([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950",
+                           "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), "-o", out] + objs)
     return out
 
 

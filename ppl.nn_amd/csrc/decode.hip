@@ -38,6 +38,7 @@
 // one un-normalised partial (max, sum, acc[Dh]) per query head into workspace slot (range index + sequence index) --
 // consecutive (range, sequence) segments get consecutive slots -- and `decode_merge_kernel` combines the slots of a
 // sequence with the usual log-sum-exp weights.
+#include <atomic>
 #include "common.h"
 
 namespace pplhip {
@@ -741,8 +742,13 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     const int64_t blocks = (int64_t)p.num_ranges * (p.kv_heads / p.hpb);
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many tasks");
     const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
-    static bool lds_opt_in = false; // more than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in
-    if (!lds_opt_in) {
+    // more than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in, once per device (the attribute is kept
+    // per device by the runtime); setting it twice from two threads is harmless, so a relaxed bit mask is enough
+    static std::atomic<uint64_t> lds_opted_in{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: no current device");
+    if (!(lds_opted_in.load(std::memory_order_relaxed) >> dev & 1)) {
         for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false>),
                                reinterpret_cast<const void*>(decode_int8kv_kernel<true>)}) {
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -750,7 +756,7 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
                 PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
                             lds_bytes, hipGetErrorString(e));
         }
-        lds_opt_in = true;
+        lds_opted_in.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
     }
     if (p.page_shift)
         hipLaunchKernelGGL(decode_int8kv_kernel<true>, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes,
