@@ -72,12 +72,28 @@ struct TileRegs<true> { // int8 slab: 8 bytes + one fp16 scale per token for K a
 };
 
 // Pins a pointer that is wave-uniform by construction into scalar registers, so that memory instructions take the
-// "scalar base + 32-bit lane offset" addressing form.
-__device__ inline const char* uniform_ptr(const char* p) {
+// "scalar base + 32-bit lane offset" addressing form. The integer round trip loses the pointer's address space, so the
+// result is typed as a global-memory pointer explicitly: loads through a generic pointer become flat_load, which
+// counts on the LDS counter as well, and every wait for an LDS read would then also wait for the tile prefetch.
+typedef const char __attribute__((address_space(1))) * gptr_t;
+__device__ inline gptr_t uniform_ptr(const char* p) {
     const uint64_t u = reinterpret_cast<uint64_t>(p);
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
     const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
-    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+    return reinterpret_cast<gptr_t>(((uint64_t)hi << 32) | lo);
+}
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ inline uint4 gload16(gptr_t p) {
+    const u32x4_t x = *reinterpret_cast<const u32x4_t __attribute__((address_space(1)))*>(p);
+    return make_uint4(x[0], x[1], x[2], x[3]);
+}
+__device__ inline uint2 gload8(gptr_t p) {
+    const u32x2_t x = *reinterpret_cast<const u32x2_t __attribute__((address_space(1)))*>(p);
+    return make_uint2(x[0], x[1]);
+}
+__device__ inline uint16_t gload2(gptr_t p) {
+    return *reinterpret_cast<const uint16_t __attribute__((address_space(1)))*>(p);
 }
 
 // Where a workgroup's K/V rows come from. Token j of the sequence is at (uniform base) + j * row_bytes, and a
@@ -114,12 +130,12 @@ struct TileSrc<true> {
 __device__ inline void fetch_tile(TileRegs<false>& t, const TileSrc<false>& src, int64_t j0, int64_t kvlen) {
     const int r0 = threadIdx.x >> 4;
     if (j0 + kBN <= kvlen) { // whole tile inside the sequence (wave-uniform)
-        const char* kb = uniform_ptr(src.k + j0 * src.row_bytes);
-        const char* vb = uniform_ptr(src.v + j0 * src.row_bytes);
+        const gptr_t kb = uniform_ptr(src.k + j0 * src.row_bytes);
+        const gptr_t vb = uniform_ptr(src.v + j0 * src.row_bytes);
 #pragma unroll
         for (int pass = 0; pass < 4; ++pass) {
-            t.k[pass] = *reinterpret_cast<const uint4*>(kb + pass * src.row_bytes + src.voff);
-            t.v[pass] = *reinterpret_cast<const uint4*>(vb + pass * src.row_bytes + src.voff);
+            t.k[pass] = gload16(kb + pass * src.row_bytes + src.voff);
+            t.v[pass] = gload16(vb + pass * src.row_bytes + src.voff);
         }
     } else { // last, partial tile: rows past the end read as zero
 #pragma unroll
@@ -138,17 +154,17 @@ __device__ inline void fetch_tile(TileRegs<false>& t, const TileSrc<false>& src,
 __device__ inline void fetch_tile(TileRegs<true>& t, const TileSrc<true>& src, int64_t j0, int64_t kvlen) {
     const int r0 = threadIdx.x >> 4;
     const int64_t tok = src.tile_token(j0);
-    const char* kb = uniform_ptr(src.k + tok * src.row_bytes);
-    const char* vb = uniform_ptr(src.v + tok * src.row_bytes);
-    const char* ksb = uniform_ptr(src.ks + tok * src.srow_bytes);
-    const char* vsb = uniform_ptr(src.vs + tok * src.srow_bytes);
+    const gptr_t kb = uniform_ptr(src.k + tok * src.row_bytes);
+    const gptr_t vb = uniform_ptr(src.v + tok * src.row_bytes);
+    const gptr_t ksb = uniform_ptr(src.ks + tok * src.srow_bytes);
+    const gptr_t vsb = uniform_ptr(src.vs + tok * src.srow_bytes);
     if (j0 + kBN <= kvlen) {
 #pragma unroll
         for (int pass = 0; pass < 4; ++pass) {
-            t.kq[pass] = *reinterpret_cast<const uint2*>(kb + pass * src.row_bytes + src.voff);
-            t.vq[pass] = *reinterpret_cast<const uint2*>(vb + pass * src.row_bytes + src.voff);
-            t.ks[pass] = *reinterpret_cast<const uint16_t*>(ksb + pass * src.srow_bytes + src.svoff);
-            t.vs[pass] = *reinterpret_cast<const uint16_t*>(vsb + pass * src.srow_bytes + src.svoff);
+            t.kq[pass] = gload8(kb + pass * src.row_bytes + src.voff);
+            t.vq[pass] = gload8(vb + pass * src.row_bytes + src.voff);
+            t.ks[pass] = gload2(ksb + pass * src.srow_bytes + src.svoff);
+            t.vs[pass] = gload2(vsb + pass * src.srow_bytes + src.svoff);
         }
     } else {
 #pragma unroll
@@ -157,10 +173,10 @@ __device__ inline void fetch_tile(TileRegs<true>& t, const TileSrc<true>& src, i
             t.kq[pass] = t.vq[pass] = make_uint2(0, 0);
             t.ks[pass] = t.vs[pass] = 0;
             if (j < kvlen) {
-                t.kq[pass] = *reinterpret_cast<const uint2*>(kb + pass * src.row_bytes + src.voff);
-                t.vq[pass] = *reinterpret_cast<const uint2*>(vb + pass * src.row_bytes + src.voff);
-                t.ks[pass] = *reinterpret_cast<const uint16_t*>(ksb + pass * src.srow_bytes + src.svoff);
-                t.vs[pass] = *reinterpret_cast<const uint16_t*>(vsb + pass * src.srow_bytes + src.svoff);
+                t.kq[pass] = gload8(kb + pass * src.row_bytes + src.voff);
+                t.vq[pass] = gload8(vb + pass * src.row_bytes + src.voff);
+                t.ks[pass] = gload2(ksb + pass * src.srow_bytes + src.svoff);
+                t.vs[pass] = gload2(vsb + pass * src.srow_bytes + src.svoff);
             }
         }
     }
@@ -339,28 +355,48 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     // pipeline: registers hold tile t+1 (in flight from global memory) while tile t is computed out of LDS buffer t & 1;
     // after the compute the registers are parked in the other buffer and the loads of tile t+2 are issued
     store_tile(regs, lds, lds + kLdsKBytes);
+    // The query loads were issued behind tile 0: wait for them here, explicitly (s_waitcnt vmcnt(0)). Otherwise the
+    // wait lands at the top of the loop, in front of the first MFMA that reads qB, and on every iteration it also
+    // waits for the next tile's loads that were issued just before: the prefetch distance would be zero.
+    __builtin_amdgcn_s_waitcnt(0x0f70);
     if (kBN < kv_end) fetch_tile(regs, src, kBN, kvlen);
     __syncthreads();
     int buf = 0;
     for (int64_t j0 = 0; j0 < kv_end; j0 += kBN, buf ^= 1) {
         const char* tile = lds + buf * kLdsBufBytes;
         if (j0 <= wave_last_vis) { // else the whole tile is above this wave's diagonal (wave-uniform)
-            // ---- S^T tiles: 2 x (32 kv tokens x 32 query rows)
+            // ---- S^T tiles: 2 x (32 kv tokens x 32 query rows). The 16 K operands rotate through four registers sets
+            // with their LDS reads issued four steps ahead of the MFMA that consumes them (the scheduling barriers pin
+            // that order: left alone, the compiler issues each read right before its use and every MFMA waits out a
+            // full LDS latency); the first V^T operand group is requested behind the last K reads.
             float16_t sT[2];
 #pragma unroll
-            for (int blk = 0; blk < 2; ++blk) {
-                float16_t acc;
+            for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-                const char* kr = tile + 32 * blk * kLdsRow + k_off;
+                for (int r = 0; r < 16; ++r) sT[blk][r] = 0.f;
+            const char* kr = tile + k_off;
+            auto lds_k = [&](int step) { // step = 8 * blk + kk
+                half8_t a;
+                const uint4 x = *reinterpret_cast<const uint4*>(kr + (step >> 3) * 32 * kLdsRow + 32 * (step & 7));
+                __builtin_memcpy(&a, &x, 16);
+                return a;
+            };
+            auto lds_v = [&](int J, int i) {
+                half8_t a;
+                const uint4 x = *reinterpret_cast<const uint4*>(tile + vt_off[J ^ i] + i * 32 * kVtRow);
+                __builtin_memcpy(&a, &x, 16);
+                return a;
+            };
+            half8_t kb[4], va[2][4];
 #pragma unroll
-                for (int kk = 0; kk < 8; ++kk) {
-                    half8_t a;
-                    const uint4 x = *reinterpret_cast<const uint4*>(kr + 32 * kk);
-                    __builtin_memcpy(&a, &x, 16);
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qB[kk], acc, 0, 0, 0);
-                }
-                sT[blk] = acc;
+            for (int st = 0; st < 4; ++st) kb[st] = lds_k(st);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int st = 0; st < 16; ++st) {
+                sT[st >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[st & 3], qB[st & 7], sT[st >> 3], 0, 0, 0);
+                if (st + 4 < 16) kb[st & 3] = lds_k(st + 4);
+                else va[0][st - 12] = lds_v(0, st - 12);
+                __builtin_amdgcn_sched_barrier(0);
             }
             const bool need_mask = (j0 + kBN - 1 > wave_first_vis) || (j0 + kBN > kvlen);
             if (need_mask) {
@@ -410,16 +446,20 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
                 }
             l_part += psum;
 
-            // ---- O^T += V^T * P^T: channel block i (32 channels), 16 tokens per MFMA k-block
+            // ---- O^T += V^T * P^T: channel block i (32 channels), 16 tokens per MFMA k-block; the operands of token
+            // group J + 1 are requested before the MFMAs of group J are issued
 #pragma unroll
-            for (int J = 0; J < 4; ++J)
+            for (int J = 0; J < 4; ++J) {
+                if (J < 3) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    half8_t a;
-                    const uint4 x = *reinterpret_cast<const uint4*>(tile + vt_off[J ^ i] + i * 32 * kVtRow);
-                    __builtin_memcpy(&a, &x, 16);
-                    oT[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pB[J], oT[i], 0, 0, 0);
+                    for (int i = 0; i < 4; ++i) va[(J + 1) & 1][i] = lds_v(J + 1, i);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    oT[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[J & 1][i], pB[J], oT[i], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (j0 + kBN < kv_end) {
             // the other buffer was last read during the previous iteration, which every wave left through the barrier
