@@ -498,6 +498,344 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// fp16 K/V source: tiles travel global -> LDS by DMA (global_load_lds_dwordx4), no registers and no LDS stores.
+//   * K rows land as they are (256 B per token, no padding); the 16-byte chunk q of row r is stored at position
+//     q ^ (r & 15), chosen on the GLOBAL side of the transfer (lane i of an instruction fills LDS bytes 16*i .. +15 of
+//     four consecutive rows and may fetch any 16 bytes it likes), so the 16-byte operand reads of 16 consecutive rows
+//     spread over all banks.
+//   * V lands row-major as well (64-byte chunk index ^ (r & 3)); the PV operand is read with ds_read_b64_tr_b16, which
+//     hands lane j of a 16-lane block element (j % 4) of the 8 bytes addressed by lanes 4*i + j/4, i = 0..3: with lane
+//     4*i + g addressing token t0 + i, channels c0 + 4g .. +3, lane j receives channel c0 + j of tokens t0 .. t0+3,
+//     i.e. V^T in MFMA operand layout without any transposition pass.
+// The DMA instructions are written as inline assembly: the compiler then does not know that LDS is written behind
+// its back and does not make every LDS read wait for the transfers in flight; completion is waited for explicitly
+// (s_waitcnt vmcnt(0) by the issuing wave, then the workgroup barrier that ends the iteration).
+// Ring: K slots 0/1 at LDS bytes 0 / 16384, V slots 0/1 at 32768 / 49152. Iteration t computes tile t out of slot
+// t & 1 while tile t + 1 lands in the other slot (last read in iteration t - 1, which every wave left through the
+// barrier).
+constexpr int kDmaTile = kBN * kPDh * 2; // 16384 bytes of K (or V) per tile
+constexpr int kDmaVBase = 2 * kDmaTile;
+
+__device__ inline void dma16(uint32_t voff, gptr_t base, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(lds_addr)
+                 : "memory"); // M0 is written here and nowhere else in this kernel (gfx9 LDS instructions do not read it)
+}
+
+__device__ inline void tile_softmax(float16_t (&sT)[2], float16_t (&oT)[4], half8_t (&pB)[4], float& m_ref,
+                                    float& l_part, float c) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sT[blk][r]);
+    mx = fmaxf(mx, other_half(mx));
+    const bool moved = (mx - m_ref) * c > kRescaleLog2;
+    if (__any(moved)) { // a row's result depends on its own scores only: rows that did not move keep theirs
+        const float m_new = moved ? mx : m_ref;
+        const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
+        m_ref = m_new;
+        l_part *= alpha;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) oT[i] *= alpha;
+    }
+    const float neg_mc = -m_ref * c;
+    float psum = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int J = 0; J < 2; ++J) {
+            float pe[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sT[blk][8 * J + e], c, neg_mc));
+                psum += pe[e];
+            }
+            pB[2 * blk + J] = half8_t{(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3],
+                                      (half_t)pe[4], (half_t)pe[5], (half_t)pe[6], (half_t)pe[7]};
+        }
+    l_part += psum;
+}
+
+typedef __attribute__((address_space(3))) char* lds_char_t;
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef short short8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) short4_t* lds_short4_t;
+
+__global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams p) {
+    __shared__ __attribute__((aligned(1024))) char lds[4 * kDmaTile];
+
+    const int per_tile = p.num_seqs * p.num_heads;
+    const int qt_rev = blockIdx.x / per_tile;
+    const int rem = blockIdx.x - qt_rev * per_tile;
+    const int b = p.first_seq + rem / p.num_heads;
+    const int hl = rem % p.num_heads;
+    const int kvh = hl % p.kv_heads;
+    const int head = kvh * p.rep + hl / p.kv_heads;
+    const int64_t s0 = p.seqstarts[b];
+    const int64_t L = p.seqstarts[b + 1] - s0;
+    const int64_t kv0 = p.kvstarts[b];
+    const int64_t kvlen = p.kvstarts[b + 1] - kv0;
+    const int64_t sp = kvlen > L ? kvlen - L : 0;
+    const int ntiles = (int)((L + kBM - 1) / kBM);
+    const int ntiles_max = gridDim.x / per_tile;
+    const int qt = ntiles_max - 1 - qt_rev;
+    if (qt >= ntiles) return;
+    const int64_t q0 = (int64_t)qt * kBM;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 31;
+    const int hb = lane >> 5;
+    const int64_t row = q0 + 32 * wave + n;
+    const bool row_ok = row < L;
+    const int64_t last_row = (q0 + kBM < L ? q0 + kBM : L) - 1;
+    int64_t kv_end = p.is_causal ? sp + last_row + 1 : kvlen;
+    if (kv_end > kvlen) kv_end = kvlen;
+    const int nkv = (int)((kv_end + kBN - 1) / kBN);
+
+    // ---- DMA source: instruction i of this wave fills LDS rows 16*wave + 4*i + lane/16, chunk position lane % 16.
+    // Per-lane offsets are relative to row 16*wave + 4*i of the tile: K needs one per instruction (its swizzle key
+    // depends on i), V a single one.
+    const uint32_t row_bytes = (uint32_t)p.kv_heads * kPDh * 2;
+    const char* k_seq = reinterpret_cast<const char*>(p.k) + (kv0 * p.kv_heads + kvh) * kPDh * 2;
+    const char* v_seq = reinterpret_cast<const char*>(p.v) + (kv0 * p.kv_heads + kvh) * kPDh * 2;
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char_t)lds);
+    const int dq = lane & 15, dr = lane >> 4;
+    uint32_t k_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) k_src[i] = (uint32_t)dr * row_bytes + (uint32_t)((dq ^ (4 * i + dr)) << 4);
+    const uint32_t v_src = (uint32_t)dr * row_bytes + (uint32_t)((dq ^ (dr << 2)) << 4);
+    // tile t of K (IS_V = false) or V into ring slot t & 1
+    auto issue = [&](int t, bool is_v) {
+        const int64_t j0 = (int64_t)t * kBN;
+        const int rows_mem = (int)(kvlen - j0 < kBN ? kvlen - j0 : kBN); // rows of the tile that exist (>= 1)
+        const char* seq = is_v ? v_seq : k_seq;
+        const uint32_t slot = lds_base + (is_v ? kDmaVBase : 0) + (uint32_t)(t & 1) * kDmaTile + (uint32_t)wave * 4096;
+        const gptr_t base = uniform_ptr(seq + j0 * row_bytes);
+        if (rows_mem == kBN) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) // (scalar row offset) + (per-lane offset): one vector add per transfer
+                dma16((is_v ? v_src : k_src[i]) + (uint32_t)(16 * wave + 4 * i) * row_bytes, base, slot + 1024 * i);
+        } else { // last, partial tile: rows past the end re-read the last one (their scores are masked)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = 16 * wave + 4 * i + dr;
+                const int rm = r < rows_mem ? r : rows_mem - 1;
+                const int key = is_v ? ((r & 3) << 2) : (r & 15);
+                dma16((uint32_t)rm * row_bytes + (uint32_t)((dq ^ key) << 4), base, slot + 1024 * i);
+            }
+        }
+    };
+    issue(0, false);
+    issue(0, true);
+    if (nkv > 1) issue(1, false);
+
+    // Q^T as the B operand: qB[kk] = Q[row][16*kk + 8*hb .. +7]
+    half8_t qB[8];
+    {
+        const half_t* qp = p.q + ((s0 + (row_ok ? row : 0)) * p.num_heads + head) * kPDh + 8 * hb;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            uint4 x = *reinterpret_cast<const uint4*>(qp + 16 * kk);
+            if (!row_ok) x = make_uint4(0, 0, 0, 0);
+            __builtin_memcpy(&qB[kk], &x, 16);
+        }
+    }
+
+    float16_t oT[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oT[i][r] = 0.f;
+    float m_ref = -INFINITY, l_part = 0.f;
+
+    const int64_t wave_last_vis = p.is_causal ? sp + q0 + 32 * wave + 31 : kvlen;
+    const int64_t wave_first_vis = p.is_causal ? sp + q0 + 32 * wave : kvlen;
+    const int64_t vis = p.is_causal ? sp + row : kvlen;
+    const int64_t last_key = vis < kvlen - 1 ? vis : kvlen - 1;
+    const float c = p.score_scale;
+    // tiles this wave computes: those with a key some row of the wave sees (a prefix of the workgroup's tiles)
+    int n_act = (int)(wave_last_vis / kBN) + 1;
+    if (n_act > nkv) n_act = nkv;
+
+    // ---- per-lane LDS read offsets (relative to the slot)
+    // K operand of step (blk, kk): row 32*blk + n, chunk 2*kk + hb, stored at position chunk ^ (n & 15), which is
+    // (position of chunk hb) ^ 2*kk: one register, one XOR per read
+    const int k_off0 = n * 256 + ((hb ^ (n & 15)) << 4);
+    // V operand of (channel block i, token group): this lane addresses token 4*hb + (lane % 16) / 4 of the group's
+    // 8-token half, channels 32*i + 16*((lane / 16) & 1) + 4*(lane % 4) .. +3; 64-byte chunk i sits at i ^ (token & 3)
+    const int v_off0 = kDmaVBase + (4 * hb + ((lane & 15) >> 2)) * 256 + (((lane & 15) >> 2) << 6) +
+                       32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+    const lds_char_t lds3 = (lds_char_t)lds;
+    auto lds_k = [&](int t, int step) { // step = 8 * blk + kk
+        half8_t a;
+        const u32x4_t x = *reinterpret_cast<const __attribute__((address_space(3))) u32x4_t*>(
+            lds3 + (t & 1) * kDmaTile + (k_off0 ^ ((step & 7) << 5)) + (step >> 3) * 32 * 256);
+        __builtin_memcpy(&a, &x, 16);
+        return a;
+    };
+    // tokens 16*G + 8*q + 4*hb + e, e = 0..3, for q = 0 (low half of the operand) and q = 1
+    auto lds_v = [&](int t, int G, int i) {
+        const lds_char_t at = lds3 + (t & 1) * kDmaTile + (v_off0 ^ (i << 6));
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t)(at + (16 * G) * 256));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t)(at + (16 * G + 8) * 256));
+        const short8_t x = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        half8_t a;
+        __builtin_memcpy(&a, &x, 16);
+        return a;
+    };
+
+    // tile 0 and the queries have to be there before the first MFMA (see prefill_attention_kernel for why the wait
+    // is explicit)
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+
+    // Software pipeline over the tiles: iteration t exponentiates the scores of tile t (vector ALU) while the MFMAs
+    // of tile t + 1's scores are issued from the same instruction stream, then accumulates P(t) * V(t). Ring use in
+    // iteration t: reads K(t+1) and V(t), transfers K(t+2) -> K slot t & 1 and V(t+1) -> V slot (t+1) & 1, both last
+    // read in iteration t - 1.
+    float16_t sA[2], sB[2]; // raw scores of the current and the next tile, alternating
+    {
+        half8_t kb[4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sA[blk][r] = 0.f;
+#pragma unroll
+        for (int st = 0; st < 4; ++st) kb[st] = lds_k(0, st);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int st = 0; st < 16; ++st) {
+            sA[st >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[st & 3], qB[st & 7], sA[st >> 3], 0, 0, 0);
+            if (st + 4 < 16) kb[st & 3] = lds_k(0, st + 4);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    __syncthreads(); // every wave is done with K(0) before K(2) is sent into its slot
+
+    auto step = [&](int t, float16_t (&sC)[2], float16_t (&sN)[2]) __attribute__((always_inline)) {
+        const int64_t j0 = (int64_t)t * kBN;
+        if (t + 2 < nkv) issue(t + 2, false);
+        if (t + 1 < nkv) issue(t + 1, true);
+        if (t < n_act) {
+            // ---- stage 1 (vector ALU only): mask, row maxima, move the reference maximum if it has to
+            const bool need_mask = (j0 + kBN - 1 > wave_first_vis) || (j0 + kBN > kvlen);
+            if (need_mask) {
+                const int64_t lim64 = last_key - j0;
+                const int lim = (int)(lim64 < -1 ? -1 : (lim64 > kBN - 1 ? kBN - 1 : lim64));
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (32 * blk + 8 * (r >> 2) + 4 * hb + (r & 3) > lim) sC[blk][r] = -INFINITY;
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sC[blk][r]);
+            mx = fmaxf(mx, other_half(mx));
+            const bool moved = (mx - m_ref) * c > kRescaleLog2;
+            if (__any(moved)) { // a row's result depends on its own scores only: rows that did not move keep theirs
+                const float m_new = moved ? mx : m_ref;
+                const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
+                m_ref = m_new;
+                l_part *= alpha;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) oT[i] *= alpha;
+            }
+            const float neg_mc = -m_ref * c;
+            half8_t pB[4]; // pB[G]: k-slot e8 <-> token 16*G + 8*(e8/4) + 4*hb + e8%4
+            half8_t va[4]; // V^T operands, requested four MFMAs ahead
+            float psum = 0.f;
+            // scores 2*j and 2*j + 1 of the lane's 32 (j = 0..15): two fma, two exp2, two adds, one packed conversion
+            auto exp_pair = [&](int j, float nm) {
+                const int G = j >> 2, e = 2 * (j & 3);
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sC[G >> 1][8 * (G & 1) + e], c, nm));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sC[G >> 1][8 * (G & 1) + e + 1], c, nm));
+                psum += p0;
+                psum += p1;
+                pB[G][e] = (half_t)p0;
+                pB[G][e + 1] = (half_t)p1;
+            };
+            // ---- stage 2: scores of tile t + 1 (MFMA) interleaved with the exponentials of tile t (vector ALU): the
+            // source order below is the instruction order (the scheduling barriers keep the compiler from regrouping
+            // it). The empty asm makes the exponent offset a value of the branch, so that the exponentials are not
+            // hoisted above it as code common to both sides, out of the block that holds the MFMAs.
+            __builtin_amdgcn_sched_barrier(0);
+            if (t + 1 < n_act) {
+                float nm = neg_mc;
+                asm volatile("" : "+v"(nm));
+                half8_t kb[4];
+#pragma unroll
+                for (int st = 0; st < 4; ++st) kb[st] = lds_k(t + 1, st);
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sN[blk][r] = 0.f;
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int st = 0; st < 16; ++st) {
+                    sN[st >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[st & 3], qB[st & 7], sN[st >> 3], 0, 0, 0);
+                    if (st + 4 < 16) kb[st & 3] = lds_k(t + 1, st + 4);
+                    else va[st - 12] = lds_v(t, 0, st - 12);
+                    exp_pair(st, nm);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) va[i] = lds_v(t, 0, i);
+                float nm = neg_mc;
+                asm volatile("" : "+v"(nm));
+#pragma unroll
+                for (int j = 0; j < 16; ++j) exp_pair(j, nm);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            l_part += psum;
+            // ---- stage 3: O^T += V^T * P^T, step 4*G + i = token group G, channel block i
+#pragma unroll
+            for (int st = 0; st < 16; ++st) {
+                oT[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[st & 3], pB[st >> 2], oT[st & 3], 0, 0, 0);
+                if (st + 4 < 16) va[st & 3] = lds_v(t, (st + 4) >> 2, st & 3);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // this wave's transfers have landed; the barrier publishes everybody's and frees the slots read above
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+    };
+    for (int t = 0; t < nkv; t += 2) { // the two score register sets swap roles from tile to tile
+        step(t, sA, sB);
+        if (t + 1 < nkv) step(t + 1, sB, sA);
+    }
+
+    const float l_tot = l_part + other_half(l_part);
+    const float inv = 1.0f / l_tot;
+    char* otile = lds + wave * 32 * kLdsRow;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int ch = 32 * i + 8 * g + 4 * hb;
+            const half4_t o = {(half_t)(oT[i][4 * g] * inv), (half_t)(oT[i][4 * g + 1] * inv),
+                               (half_t)(oT[i][4 * g + 2] * inv), (half_t)(oT[i][4 * g + 3] * inv)};
+            uint2 packed;
+            __builtin_memcpy(&packed, &o, 8);
+            *reinterpret_cast<uint2*>(otile + n * kLdsRow + ch * 2) = packed;
+        }
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+        const int rr = 4 * pass + (lane >> 4);
+        const int64_t orow = q0 + 32 * wave + rr;
+        const uint4 x = *reinterpret_cast<const uint4*>(otile + rr * kLdsRow + (lane & 15) * 16);
+        if (orow < L)
+            *reinterpret_cast<uint4*>(p.out + ((s0 + orow) * p.num_heads + head) * kPDh + (lane & 15) * 8) = x;
+    }
+}
+
 pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, hipStream_t stream) {
     const int npre = (int)(a->batch - a->decoding_batches);
     if (npre <= 0 || plan->prefill_num_q_tiles <= 0) return PPLHIP_RC_SUCCESS;
@@ -527,7 +865,7 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     if (a->enable_cache_prefill)
         hipLaunchKernelGGL(prefill_attention_kernel<true>, grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL(prefill_attention_kernel<false>, grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(prefill_f16_kernel, grid, dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("prefill_attention");
     return PPLHIP_RC_SUCCESS;
 }
@@ -558,7 +896,7 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
     const int64_t q_tiles = (a->max_seqlen + kBM - 1) / kBM;
     const int64_t blocks = q_tiles * a->batch * a->num_heads;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many query tiles in one call");
-    hipLaunchKernelGGL(prefill_attention_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(prefill_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("multi_head_attention");
     return PPLHIP_RC_SUCCESS;
 }
