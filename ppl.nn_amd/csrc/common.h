@@ -76,6 +76,23 @@ __device__ inline int find_sequence(const int64_t* __restrict__ starts, int n, i
     return lo;
 }
 
+// The same index for an x that every ACTIVE lane of the wave shares (inactive lanes are allowed): the table is read
+// one entry per active lane at a time and the entries <= x are counted, so the look-up costs one memory latency per
+// 64 sequences instead of a chain of log2(n) dependent loads.
+__device__ inline int find_sequence_wave(const int64_t* __restrict__ starts, int n, int64_t x) {
+    const uint64_t active = __ballot(1);
+    const int lane = threadIdx.x & 63;
+    const int rank = __popcll(active & ((uint64_t(1) << lane) - 1));
+    const int width = __popcll(active);
+    int count = 0;
+    for (int base = 1; base <= n; base += width) {
+        const int i = base + rank;
+        const bool le = i <= n && starts[i] <= x;
+        count += __popcll(__ballot(le));
+    }
+    return count;
+}
+
 inline int ceil_div(int64_t a, int64_t b) {
     return (int)((a + b - 1) / b);
 }

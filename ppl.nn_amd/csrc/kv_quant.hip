@@ -1,6 +1,6 @@
 // Quantize-on-write of new K/V tokens into the int8 group-8 KV slab, and the KeyValueCache op's
-// gather + dequantise. Both are pure streaming kernels: one lane owns one group of 8 channels
-// (16 B fp16 in, 8 B int8 + 2 B scale out), so a wavefront moves 1 KiB / 512 B + 128 B per instruction.
+// gather + dequantise. Both are pure streaming kernels over groups of 8 channels (16 B fp16 <-> 8 B int8 + 2 B
+// scale); the write kernel gives a lane four consecutive groups, the gather one.
 //
 // Rounding rule (bit-exact contract with the CPU oracle):
 //   a = max|x_i| ; s = max(fp16_rne(float(a) / 127.0f), fp16_rne(1e-5f)) ; q_i = int8(rint(fp16_rne(float(x_i) / float(s))))
@@ -20,8 +20,10 @@ struct QuantWriteParams {
     CacheAddr addr;
     int32_t batch;
     int32_t kv_heads;
-    int32_t groups_per_head; // head_dim / 8
-    int64_t total_groups; // S * 2 * kv_heads * groups_per_head
+    int32_t per_tok; // 4-group units per token: 2 * kv_heads * (head_dim / 32)
+    int32_t blocks_per_tok, tok_per_block; // one of the two is 1
+    uint32_t inv_per_tok; // ceil(65536 / per_tok)
+    int64_t total_tokens;
 };
 
 __device__ inline void quantize_group8(const uint4 raw, uint2* q_out, half_t* s_out) {
@@ -47,34 +49,62 @@ __device__ inline void quantize_group8(const uint4 raw, uint2* q_out, half_t* s_
     *s_out = s;
 }
 
+// One thread owns four consecutive groups (64 B of fp16 in, 32 B of int8 + 8 B of scales out) so that enough bytes
+// are in flight per CU to cover the memory latency. Thread -> (token, K or V, head, quarter of the head) without
+// integer division: a token has per_tok = 2 * kv_heads * 4 such units (head_dim is 128); a block covers 256 / per_tok
+// whole tokens, one token, or a 256-unit slice of one.
 __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWriteParams p) {
-    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (g >= p.total_groups) return;
-    const int gph = p.groups_per_head;
-    const int per_kv = p.kv_heads * gph;
-    const int per_tok = 2 * per_kv;
-    const int64_t t = g / per_tok; // packed new-token index
-    const int r = (int)(g - t * per_tok);
-    const int kv = r / per_kv;
-    const int r2 = r - kv * per_kv;
-    const int head = r2 / gph;
-    const int grp = r2 - head * gph;
+    int64_t t; // packed new-token index
+    int r; // unit index inside the token
+    if (p.tok_per_block == 1) {
+        const uint32_t tb = blockIdx.x / p.blocks_per_tok; // block-uniform
+        t = tb;
+        r = (int)(blockIdx.x - tb * p.blocks_per_tok) * 256 + (int)threadIdx.x;
+        if (r >= p.per_tok) return;
+    } else {
+        const int lt = (int)((threadIdx.x * p.inv_per_tok) >> 16); // threadIdx.x / per_tok, exact below 256
+        if (lt >= p.tok_per_block) return;
+        t = (int64_t)blockIdx.x * p.tok_per_block + lt;
+        r = (int)threadIdx.x - lt * p.per_tok;
+    }
+    if (t >= p.total_tokens) return;
+    const int hi = r >> 2; // 0 .. 2 * kv_heads - 1: K heads, then V heads
+    const int grp = (r & 3) * 4; // first of the unit's four groups
+    const int kv = hi >= p.kv_heads;
+    const int head = hi - kv * p.kv_heads;
+    // the values do not depend on which sequence the token belongs to: their loads go out before the look-up
+    const uint4* src = reinterpret_cast<const uint4*>((kv ? p.value : p.key) + ((t * p.kv_heads + head) * 16 + grp) * 8);
+    uint4 raw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = src[i];
     // decode sequences come first and hold one token each, so for them the packed token index IS the sequence index:
-    // two independent loads settle it; only prompt tokens pay for the binary search (a chain of dependent loads)
+    // two independent loads settle it; only prompt tokens pay for a search of the table
     int b;
-    if (t < p.batch && p.seqstarts[t] == t && p.seqstarts[t + 1] == t + 1)
+    if (t < p.batch && p.seqstarts[t] == t && p.seqstarts[t + 1] == t + 1) {
         b = (int)t;
-    else
-        b = find_sequence(p.seqstarts, p.batch, t);
+    } else {
+        // a wave normally sits inside one token: then the table is searched by the whole wave at once
+        const int64_t t0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(t >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+        if (__all(t == t0))
+            b = find_sequence_wave(p.seqstarts, p.batch, t0);
+        else
+            b = find_sequence(p.seqstarts, p.batch, t);
+    }
     const int64_t tok = p.pages.token(b, p.start_pos[b] + (t - p.seqstarts[b]));
-    const half_t* src = (kv ? p.value : p.key) + ((t * p.kv_heads + head) * gph + grp) * 8;
-    const uint4 raw = *reinterpret_cast<const uint4*>(src);
-    uint2 q;
-    half_t s;
-    quantize_group8(raw, &q, &s);
+    uint2 q[4];
+    half_t sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) quantize_group8(raw[i], &q[i], &sc[i]);
     const int64_t row = p.addr.row(tok, kv, head);
-    *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = q;
-    p.scale[row / kQuantGroup + grp] = s;
+    uint4* dst = reinterpret_cast<uint4*>(p.cache + row + grp * 8); // rows and grp * 8 are multiples of 16
+    dst[0] = make_uint4(q[0].x, q[0].y, q[1].x, q[1].y);
+    dst[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
+    uint32_t packed[2];
+    __builtin_memcpy(packed, sc, 8);
+    uint32_t* sdst = reinterpret_cast<uint32_t*>(p.scale + row / kQuantGroup + grp); // row / 8 and grp are even
+    sdst[0] = packed[0];
+    sdst[1] = packed[1];
 }
 
 pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream) {
@@ -90,9 +120,14 @@ pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream
     p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
     p.batch = (int32_t)a->batch;
     p.kv_heads = a->num_kv_heads;
-    p.groups_per_head = a->head_dim / kQuantGroup;
-    p.total_groups = a->total_new_tokens * 2 * (int64_t)a->num_kv_heads * p.groups_per_head;
-    const int64_t blocks = (p.total_groups + 255) / 256;
+    if (a->head_dim != 128) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: head_dim must be 128");
+    p.per_tok = 2 * a->num_kv_heads * (a->head_dim / (4 * kQuantGroup));
+    p.blocks_per_tok = p.per_tok >= 256 ? (p.per_tok + 255) / 256 : 1;
+    p.tok_per_block = p.per_tok >= 256 ? 1 : 256 / p.per_tok;
+    p.inv_per_tok = (65536u + (uint32_t)p.per_tok - 1) / (uint32_t)p.per_tok;
+    p.total_tokens = a->total_new_tokens;
+    const int64_t blocks = p.tok_per_block == 1 ? a->total_new_tokens * p.blocks_per_tok
+                                                : (a->total_new_tokens + p.tok_per_block - 1) / p.tok_per_block;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "kv_quantize_write: too many groups");
     hipLaunchKernelGGL(kv_quantize_write_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("kv_quantize_write");
@@ -125,7 +160,15 @@ __global__ __launch_bounds__(256) void kv_gather_dequant_kernel(const GatherPara
     const int r2 = r - kv * per_kv;
     const int head = r2 / gph;
     const int grp = r2 - head * gph;
-    const int b = find_sequence(p.kvstarts, p.batch, j);
+    int b;
+    {
+        const int64_t j0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(j >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)j);
+        if (__all(j == j0))
+            b = find_sequence_wave(p.kvstarts, p.batch, j0);
+        else
+            b = find_sequence(p.kvstarts, p.batch, j);
+    }
     const int64_t tok = p.cachestarts[b] + (j - p.kvstarts[b]);
     const int64_t row = p.addr.row(tok, kv, head);
     const uint2 q = *reinterpret_cast<const uint2*>(p.cache + row + grp * 8);

@@ -604,30 +604,33 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     const char* v_seq = reinterpret_cast<const char*>(p.v) + (kv0 * p.kv_heads + kvh) * kPDh * 2;
     const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char_t)lds);
     const int dq = lane & 15, dr = lane >> 4;
-    uint32_t k_src[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) k_src[i] = (uint32_t)dr * row_bytes + (uint32_t)((dq ^ (4 * i + dr)) << 4);
-    const uint32_t v_src = (uint32_t)dr * row_bytes + (uint32_t)((dq ^ (dr << 2)) << 4);
-    // tile t of K (IS_V = false) or V into ring slot t & 1
-    auto issue = [&](int t, bool is_v) {
+    const int dma_row0 = 16 * wave + dr; // LDS row of transfer 0; transfer i: + 4 * i
+    const uint32_t k_swz0 = (uint32_t)((dq ^ dr) << 4); // K: chunk dq ^ (row & 15), row & 15 = 4*i + dr -> ^ (i << 6)
+    const uint32_t v_swz = (uint32_t)((dq ^ (dr << 2)) << 4); // V: chunk dq ^ ((row & 3) << 2), row & 3 = dr
+    // one tile of K or V = 4 transfers per wave; everything that is the same for the 4 is in TileDma
+    struct TileDma {
+        gptr_t base; // row 0 of the tile
+        uint32_t slot; // LDS address of this wave's 16 rows in the ring slot
+        int last_row; // rows past the end of the sequence re-read the last one (their scores are masked)
+    };
+    auto tile_dma = [&](int t, bool is_v) {
         const int64_t j0 = (int64_t)t * kBN;
-        const int rows_mem = (int)(kvlen - j0 < kBN ? kvlen - j0 : kBN); // rows of the tile that exist (>= 1)
-        const char* seq = is_v ? v_seq : k_seq;
-        const uint32_t slot = lds_base + (is_v ? kDmaVBase : 0) + (uint32_t)(t & 1) * kDmaTile + (uint32_t)wave * 4096;
-        const gptr_t base = uniform_ptr(seq + j0 * row_bytes);
-        if (rows_mem == kBN) {
+        TileDma d;
+        d.base = uniform_ptr((is_v ? v_seq : k_seq) + j0 * row_bytes);
+        d.slot = lds_base + (is_v ? kDmaVBase : 0) + (uint32_t)(t & 1) * kDmaTile + (uint32_t)wave * 4096;
+        d.last_row = (int)(kvlen - j0 < kBN ? kvlen - j0 : kBN) - 1;
+        return d;
+    };
+    auto issue_one = [&](const TileDma& d, bool is_v, int i) {
+        const int r = dma_row0 + 4 * i;
+        const uint32_t rm = (uint32_t)(r < d.last_row ? r : d.last_row);
+        dma16(__umul24(rm, row_bytes) + (is_v ? v_swz : (k_swz0 ^ (uint32_t)(i << 6))), d.base,
+              d.slot + 1024 * i);
+    };
+    auto issue = [&](int t, bool is_v) {
+        const TileDma d = tile_dma(t, is_v);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) // (scalar row offset) + (per-lane offset): one vector add per transfer
-                dma16((is_v ? v_src : k_src[i]) + (uint32_t)(16 * wave + 4 * i) * row_bytes, base, slot + 1024 * i);
-        } else { // last, partial tile: rows past the end re-read the last one (their scores are masked)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int r = 16 * wave + 4 * i + dr;
-                const int rm = r < rows_mem ? r : rows_mem - 1;
-                const int key = is_v ? ((r & 3) << 2) : (r & 15);
-                dma16((uint32_t)rm * row_bytes + (uint32_t)((dq ^ key) << 4), base, slot + 1024 * i);
-            }
-        }
+        for (int i = 0; i < 4; ++i) issue_one(d, is_v, i);
     };
     issue(0, false);
     issue(0, true);
@@ -644,19 +647,29 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
             __builtin_memcpy(&qB[kk], &x, 16);
         }
     }
+    // the queries are scaled once by log2(e) / sqrt(Dh), so that the MFMA result is the exponent of exp2 directly and
+    // no per-score multiply is left in the loop. Packed fp16 multiplies: the factor is rounded to fp16, i.e. the
+    // softmax runs at a temperature that is off by at most 2^-12 relative, far inside the output tolerance.
+    {
+        const half_t c16 = (half_t)p.score_scale;
+        const half8_t cv = {c16, c16, c16, c16, c16, c16, c16, c16};
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) qB[kk] = qB[kk] * cv;
+    }
 
     float16_t oT[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oT[i][r] = 0.f;
-    float m_ref = -INFINITY, l_part = 0.f;
+    // m_ref: reference maximum of a row in exponent units, always a value fp16 holds exactly; score registers hold
+    // (exponent - the m_ref that was current when their MFMAs were issued)
+    float m_ref = 0.f, l_part = 0.f;
 
     const int64_t wave_last_vis = p.is_causal ? sp + q0 + 32 * wave + 31 : kvlen;
     const int64_t wave_first_vis = p.is_causal ? sp + q0 + 32 * wave : kvlen;
     const int64_t vis = p.is_causal ? sp + row : kvlen;
     const int64_t last_key = vis < kvlen - 1 ? vis : kvlen - 1;
-    const float c = p.score_scale;
     // tiles this wave computes: those with a key some row of the wave sees (a prefix of the workgroup's tiles)
     int n_act = (int)(wave_last_vis / kBN) + 1;
     if (n_act > nkv) n_act = nkv;
@@ -714,10 +727,17 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+    // running maximum of the raw scores of the tile about to be exponentiated (per lane: half of a query row's keys)
+    float mx_raw = -INFINITY;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx_raw = fmaxf(mx_raw, sA[blk][r]);
     __syncthreads(); // every wave is done with K(0) before K(2) is sent into its slot
 
     auto step = [&](int t, float16_t (&sC)[2], float16_t (&sN)[2]) __attribute__((always_inline)) {
         const int64_t j0 = (int64_t)t * kBN;
+        // transfers of this iteration: K(t+2) and V(t+1)
         if (t + 2 < nkv) issue(t + 2, false);
         if (t + 1 < nkv) issue(t + 1, true);
         if (t < n_act) {
@@ -732,76 +752,105 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
                     for (int r = 0; r < 16; ++r)
                         if (32 * blk + 8 * (r >> 2) + 4 * hb + (r & 3) > lim) sC[blk][r] = -INFINITY;
             }
-            float mx = -INFINITY;
-#pragma unroll
-            for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sC[blk][r]);
-            mx = fmaxf(mx, other_half(mx));
-            const bool moved = (mx - m_ref) * c > kRescaleLog2;
-            if (__any(moved)) { // a row's result depends on its own scores only: rows that did not move keep theirs
-                const float m_new = moved ? mx : m_ref;
-                const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
-                m_ref = m_new;
-                l_part *= alpha;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) oT[i] *= alpha;
-            }
-            const float neg_mc = -m_ref * c;
-            half8_t pB[4]; // pB[G]: k-slot e8 <-> token 16*G + 8*(e8/4) + 4*hb + e8%4
-            half8_t va[4]; // V^T operands, requested four MFMAs ahead
-            float psum = 0.f;
-            // scores 2*j and 2*j + 1 of the lane's 32 (j = 0..15): two fma, two exp2, two adds, one packed conversion
-            auto exp_pair = [&](int j, float nm) {
-                const int G = j >> 2, e = 2 * (j & 3);
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sC[G >> 1][8 * (G & 1) + e], c, nm));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sC[G >> 1][8 * (G & 1) + e + 1], c, nm));
-                psum += p0;
-                psum += p1;
-                pB[G][e] = (half_t)p0;
-                pB[G][e + 1] = (half_t)p1;
-            };
-            // ---- stage 2: scores of tile t + 1 (MFMA) interleaved with the exponentials of tile t (vector ALU): the
-            // source order below is the instruction order (the scheduling barriers keep the compiler from regrouping
-            // it). The empty asm makes the exponent offset a value of the branch, so that the exponentials are not
-            // hoisted above it as code common to both sides, out of the block that holds the MFMAs.
-            __builtin_amdgcn_sched_barrier(0);
-            if (t + 1 < n_act) {
-                float nm = neg_mc;
-                asm volatile("" : "+v"(nm));
-                half8_t kb[4];
-#pragma unroll
-                for (int st = 0; st < 4; ++st) kb[st] = lds_k(t + 1, st);
+            float mx = mx_raw; // taken over the unmasked scores while the previous tile's PV MFMAs ran
+            if (need_mask) {
+                mx = -INFINITY;
 #pragma unroll
                 for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) sN[blk][r] = 0.f;
+                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sC[blk][r]);
+            }
+            mx = fmaxf(mx, other_half(mx));
+            // mx is relative to m_ref. The reference only moves when the row's maximum has outgrown it by more than
+            // 2^kRescaleLog2 (always on the first tile, where it becomes the tile's maximum: key 0 is visible to every
+            // row, so that maximum is finite)
+            const bool moved = mx > kRescaleLog2 || t == 0;
+            if (__any(moved)) { // a row's result depends on its own scores only: rows that did not move keep theirs
+                const float m_new = (float)(half_t)(m_ref + mx);
+                const float delta = moved ? m_new - m_ref : 0.f; // exact: both are fp16 values
+                // (nothing is accumulated yet on the first tile, and 0 * 2^(large) must not be formed)
+                const float alpha = t == 0 ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+                m_ref += delta;
+                l_part *= alpha;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) oT[i] *= alpha;
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk) sC[blk] -= delta;
+            }
+            half8_t pB[4]; // pB[G]: k-slot e8 <-> token 16*G + 8*(e8/4) + 4*hb + e8%4
+            half8_t va[4]; // V^T operands, requested four MFMAs ahead
+            float psum = 0.f;
+            // scores 2*j and 2*j + 1 of the lane's 32 (j = 0..15): two exp2; one step later (so that nothing waits for
+            // the exponentials' latency) one packed conversion and one dot2 that adds the two ROUNDED probabilities to
+            // the row sum (the sum then matches what the PV MFMAs multiply)
+            float e0 = 0.f, e1 = 0.f;
+            auto pack_pair = [&](int j) {
+                const int G = j >> 2, e = 2 * (j & 3);
+                const half2_t pk = {(half_t)e0, (half_t)e1};
+                psum = __builtin_amdgcn_fdot2(pk, half2_t{(half_t)1.0f, (half_t)1.0f}, psum, false);
+                pB[G][e] = pk[0];
+                pB[G][e + 1] = pk[1];
+            };
+            auto exp_pair = [&](int j, float x0, float x1) {
+                if (j > 0) pack_pair(j - 1);
+                e0 = __builtin_amdgcn_exp2f(x0);
+                e1 = __builtin_amdgcn_exp2f(x1);
+                if (j == 15) pack_pair(15);
+            };
+            // ---- stage 2: scores of tile t + 1 (MFMA) interleaved with the exponentials of tile t (vector ALU): the
+            // source order below is the instruction order (the scheduling barriers keep the compiler from regrouping
+            // it). The two sides of the branch must not look alike, or the exponentials are hoisted above it as common
+            // code, out of the block that holds the MFMAs.
+            __builtin_amdgcn_sched_barrier(0);
+            if (t + 1 < n_act) {
+                half8_t kb[4];
+#pragma unroll
+                for (int st = 0; st < 4; ++st) kb[st] = lds_k(t + 1, st);
+                // -m_ref enters the scores through one MFMA per block: A = ones, B = -m_ref in a single k-slot
+                half8_t mB;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mB[e] = (half_t)0.f;
+                mB[0] = hb == 0 ? (half_t)(-m_ref) : (half_t)0.f;
+                half8_t ones;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ones[e] = (half_t)1.0f;
+                float16_t zero;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+                __builtin_amdgcn_sched_barrier(0);
+                sN[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, mB, zero, 0, 0, 0);
+                sN[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, mB, zero, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int st = 0; st < 16; ++st) {
                     sN[st >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[st & 3], qB[st & 7], sN[st >> 3], 0, 0, 0);
                     if (st + 4 < 16) kb[st & 3] = lds_k(t + 1, st + 4);
                     else va[st - 12] = lds_v(t, 0, st - 12);
-                    exp_pair(st, nm);
+                    exp_pair(st, sC[st >> 3][2 * (st & 7)], sC[st >> 3][2 * (st & 7) + 1]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) va[i] = lds_v(t, 0, i);
-                float nm = neg_mc;
-                asm volatile("" : "+v"(nm));
+                float bias = 0.f; // (opaque zero: keeps this copy of the exponentials from being merged with the other)
+                asm volatile("" : "+v"(bias));
 #pragma unroll
-                for (int j = 0; j < 16; ++j) exp_pair(j, nm);
+                for (int j = 0; j < 16; ++j) exp_pair(j, sC[j >> 3][2 * (j & 7)] + bias, sC[j >> 3][2 * (j & 7) + 1] + bias);
                 __builtin_amdgcn_sched_barrier(0);
             }
             l_part += psum;
             // ---- stage 3: O^T += V^T * P^T, step 4*G + i = token group G, channel block i
+            float mxa = -INFINITY, mxb = -INFINITY;
 #pragma unroll
             for (int st = 0; st < 16; ++st) {
                 oT[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[st & 3], pB[st >> 2], oT[st & 3], 0, 0, 0);
                 if (st + 4 < 16) va[st & 3] = lds_v(t, (st + 4) >> 2, st & 3);
+                // the next tile's row maximum rides along (two chains of max3; unused after the wave's last tile)
+                if (st & 1) mxb = fmaxf(fmaxf(mxb, sN[st >> 3][2 * (st & 7)]), sN[st >> 3][2 * (st & 7) + 1]);
+                else mxa = fmaxf(fmaxf(mxa, sN[st >> 3][2 * (st & 7)]), sN[st >> 3][2 * (st & 7) + 1]);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            mx_raw = fmaxf(mxa, mxb);
         }
         // this wave's transfers have landed; the barrier publishes everybody's and frees the slots read above
         __builtin_amdgcn_s_waitcnt(0x0f70);
