@@ -382,6 +382,17 @@ def main():
             del odb
             torch.cuda.empty_cache()
         result["other_decode_configs"] = others
+        # the prefill kernel away from launch and tail effects: four 8k-token prompts of the same head shape
+        import numpy as _np
+        lb = workloads.Batch(32, 8, 128, _np.full(4, 8192, _np.int64), _np.zeros(4, _np.int64), 0, name="4x8192 prefill")
+        ldb = DeviceBatch(pkg, lib, lb, seed=5, n_slabs=1)
+        _, l_ms = timed(ldb, 5, 2)
+        lfl = lb.prefill_flops()
+        result["prefill_long_prompts"] = {"workload": "4 prompts x 8192 tokens, H32/KVH8/Dh128, causal, incl. quantize-on-write",
+                                          "tflops": lfl / (l_ms * 1e-3) / 1e12, "ms": l_ms,
+                                          "frac_of_fp16_mfma_peak": lfl / (l_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS}
+        del ldb
+        torch.cuda.empty_cache()
     if args.copy_calibration:
         copy_calibration()
     if not args.no_cpu_baseline:
