@@ -63,6 +63,31 @@ inline int page_shift_of(int cache_mode, int page_size) { // host: 0 for the con
     return s;
 }
 
+// One quantisation group: 8 fp16 values -> 8 int8 + one fp16 scale. THE rounding rule of the KV cache (bit-exact
+// contract with the CPU oracle): s = max(fp16(absmax / 127), fp16(1e-5)), q = int8(rint(fp16(x / s))).
+__device__ inline void quantize_group8(const uint4 raw, uint2* q_out, half_t* s_out) {
+    half_t x[8];
+    __builtin_memcpy(x, &raw, 16);
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf((float)x[i]));
+    half_t s = (half_t)(amax / 127.0f);
+    const half_t eps = (half_t)1e-5f;
+    if ((float)s < (float)eps) s = eps;
+    const float sf = (float)s;
+    uint32_t w[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float ratio = (float)(half_t)((float)x[i] / sf);
+        float r = rintf(ratio);
+        r = fminf(fmaxf(r, -128.f), 127.f);
+        const int qi = (int)r;
+        w[i >> 2] |= (uint32_t)(qi & 0xff) << (8 * (i & 3));
+    }
+    *q_out = make_uint2(w[0], w[1]);
+    *s_out = s;
+}
+
 // first index b in [0, n) with starts[b+1] > x  (starts is a non-decreasing prefix-sum table with n+1 entries)
 __device__ inline int find_sequence(const int64_t* __restrict__ starts, int n, int64_t x) {
     int lo = 0, hi = n;
@@ -98,7 +123,8 @@ inline int ceil_div(int64_t a, int64_t b) {
 }
 
 // launchers implemented in the .hip files
-pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream);
+// first_token: packed new tokens before it are skipped (the decode kernel writes the decode tokens itself)
+pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token = 0);
 pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream_t stream);
 int decode_heads_per_block(int kv_heads);
 int decode_blocks_per_cu();

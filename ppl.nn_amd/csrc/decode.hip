@@ -61,8 +61,10 @@ constexpr int kDecodeLdsBytes = kDecodeWaves * kWaveLdsBytes; // 81920: two work
 
 struct DecodeParams {
     const half_t* q; // [S, H, Dh]
-    const int8_t* cache;
-    const half_t* scale;
+    const half_t* cur_key; // [S, KVH, Dh] new tokens; null: the slab already holds them
+    const half_t* cur_value;
+    int8_t* cache;
+    half_t* scale;
     const int64_t* seqstarts;
     const int64_t* kvstarts;
     const int64_t* cachestarts; // [nd], or the [nd, cs_stride_b] page table when page_shift > 0
@@ -426,6 +428,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         const char* cbase; // contiguous slab: K row of token t_begin (this kv head) in the cache / scale tensors
         const char* sbase;
         int n_stages, tail_rows_mem, tail_rows_valid;
+        // this wave's chunk ends with the sequence's NEW token (its last one), which the wave quantises into the slab
+        // and into its stage buffer itself; new_row: slab offset of that token's K row for this kv head
+        bool has_new;
+        int64_t new_row;
     };
     const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
     int64_t pos = r0;
@@ -448,6 +454,14 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         g.tail_rows_mem =
             (int)((g.seg_end - last_stage_t0) < kStageTokens ? (g.seg_end - last_stage_t0) : kStageTokens);
         g.tail_rows_valid = (int)(t_end - last_stage_t0);
+        const int64_t seq_len = seq_hi - seq_lo;
+        g.has_new = p.cur_key != nullptr && g.n_stages > 0 && t_end == seq_len;
+        {
+            const int64_t tl = seq_len - 1;
+            const int64_t tok = PAGED ? g.page_row[tl >> p.page_shift] + (tl & ((int64_t(1) << p.page_shift) - 1))
+                                      : p.cachestarts[b] + tl;
+            g.new_row = tok * (int64_t)stride + head_off;
+        }
         const int64_t row0 = (PAGED ? 0 : (p.cachestarts[b] + g.t_begin) * (int64_t)stride) + head_off;
         g.cbase = reinterpret_cast<const char*>(p.cache) + row0;
         g.sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
@@ -481,17 +495,28 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     };
     auto issue = [&](const Segment& g, int idx, int slot) {
         if (idx == g.n_stages - 1 && g.tail_rows_mem < kStageTokens) { // wave-uniform, at most once per segment
+            // When the last row is the new token, which this wave has yet to write, the overhanging rows are clamped
+            // onto the token before it instead: they are masked, but their V scales are multiplied by zero
+            // probabilities and have to be finite, which the bytes of a row nobody has written need not be.
+            const int rows_mem = g.tail_rows_mem - ((g.has_new && g.tail_rows_mem >= 2) ? 1 : 0);
             DmaOffsets tail;
-            make_dma_offsets(tail, lane, stride, sstride_b, g.tail_rows_mem);
-            issue_with(g, idx, slot, tail, g.tail_rows_mem);
+            make_dma_offsets(tail, lane, stride, sstride_b, rows_mem);
+            issue_with(g, idx, slot, tail, rows_mem);
         } else {
             issue_with(g, idx, slot, full, kStageTokens);
         }
     };
 
     // Q^T as the B operand, kept for a whole segment: q[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
-    constexpr int kQueryLoads = 4;
-    auto load_query = [&](const Segment& g, half8_t (&q)[2][2]) {
+    constexpr int kQueryLoads = 5; // four query pieces + the lane's group of the sequence's new token
+    // lanes 0..15: groups of the new token's K row (this kv head), lanes 16..31: of its V row (upper half-wave mirrors)
+    auto load_query = [&](const Segment& g, half8_t (&q)[2][2], uint4& newtok) {
+        {
+            const half_t* src = ((lane & 16) ? p.cur_value : p.cur_key);
+            if (src == nullptr) src = p.q; // (never used then; keeps the load count the same)
+            else src += (g.qrow * p.kv_heads + kvh) * kDh + 8 * (lane & 15);
+            newtok = *reinterpret_cast<const uint4*>(src);
+        }
         const bool live = m < p.rep;
         const half_t* qp = p.q + ((g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
 #pragma unroll
@@ -513,7 +538,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     int slot0 = 0; // stage buffer of the current segment's stage 0
     bool cur_in_flight = false; // stage 0 of `cur` already enqueued by the previous segment's last iteration
     half8_t qB[2][2], qN[2][2];
-    load_query(cur, qB);
+    uint4 newB, newN;
+    load_query(cur, qB, newB);
     for (;;) {
         SoftmaxState ss;
 #pragma unroll
@@ -536,11 +562,33 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                     has_next = direct && pos < r1;
                     if (has_next) {
                         next_segment(nxt);
-                        load_query(nxt, qN); // older than the transfers below: landed before they are waited for
+                        load_query(nxt, qN, newN); // older than the transfers below: landed before they are waited for
                         issue(nxt, 0, slot ^ 1);
                         PPLHIP_WAIT_VMCNT(kDmaPerStage + kQueryLoads); // stage `it` only
                     } else {
                         PPLHIP_WAIT_VMCNT(0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (it + 1 == cur.n_stages && cur.has_new) {
+                    // The stage has landed with whatever the slab held in the new token's row: the row is replaced in
+                    // the stage buffer by the freshly quantised token (LDS operations of one wave execute in order, so
+                    // the reads below see it), and the same bytes go to the slab.
+                    if (lane < 32) {
+                        const int grp = lane & 15, isv = lane >> 4, r = cur.tail_rows_valid - 1;
+                        uint2 qv;
+                        half_t sc;
+                        quantize_group8(newB, &qv, &sc);
+                        char* st = wave_lds + slot * kStageBytes;
+                        *reinterpret_cast<uint2*>(st + (isv ? kLdsV : kLdsK) + r * 128 + (((grp >> 1) ^ (r & 7)) * 16) +
+                                                  (grp & 1) * 8) = qv;
+                        *reinterpret_cast<half_t*>(st + (isv ? kLdsVs : kLdsKs) + r * 32 + grp * 2) = sc;
+                        if (cur.tail_rows_mem == 1) // the new token is the stage's only row: every row is a copy of it
+                            for (int r2 = 1; r2 < kStageTokens; ++r2)
+                                *reinterpret_cast<half_t*>(st + (isv ? kLdsVs : kLdsKs) + r2 * 32 + grp * 2) = sc;
+                        const int64_t row = cur.new_row + (isv ? (int64_t)kv_off : 0);
+                        *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
+                        p.scale[row / kQuantGroup + grp] = sc;
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -636,11 +684,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                 for (int i = 0; i < 2; ++i) qB[jj][i] = qN[jj][i];
+            newB = newN;
             cur_in_flight = true;
         } else {
             if (pos >= r1) break;
             next_segment(cur);
-            load_query(cur, qB);
+            load_query(cur, qB, newB);
             slot0 = 0;
             cur_in_flight = false;
         }
@@ -717,8 +766,10 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     if (nd == 0) return PPLHIP_RC_SUCCESS;
     DecodeParams p;
     p.q = (const half_t*)a->d_query;
-    p.cache = (const int8_t*)a->d_cache;
-    p.scale = (const half_t*)a->d_scale;
+    p.cur_key = (const half_t*)a->d_current_key;
+    p.cur_value = (const half_t*)a->d_current_value;
+    p.cache = (int8_t*)a->d_cache;
+    p.scale = (half_t*)a->d_scale;
     p.seqstarts = a->d_seqstarts;
     p.kvstarts = a->d_kvstarts;
     p.cachestarts = a->d_cachestarts;

@@ -23,31 +23,8 @@ struct QuantWriteParams {
     int32_t per_tok; // 4-group units per token: 2 * kv_heads * (head_dim / 32)
     int32_t blocks_per_tok, tok_per_block; // one of the two is 1
     uint32_t inv_per_tok; // ceil(65536 / per_tok)
-    int64_t total_tokens;
+    int64_t first_token, end_token; // packed tokens [first_token, end_token) are written
 };
-
-__device__ inline void quantize_group8(const uint4 raw, uint2* q_out, half_t* s_out) {
-    half_t x[8];
-    __builtin_memcpy(x, &raw, 16);
-    float amax = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf((float)x[i]));
-    half_t s = (half_t)(amax / 127.0f);
-    const half_t eps = (half_t)1e-5f;
-    if ((float)s < (float)eps) s = eps;
-    const float sf = (float)s;
-    uint32_t w[2] = {0u, 0u};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float ratio = (float)(half_t)((float)x[i] / sf);
-        float r = rintf(ratio);
-        r = fminf(fmaxf(r, -128.f), 127.f);
-        const int qi = (int)r;
-        w[i >> 2] |= (uint32_t)(qi & 0xff) << (8 * (i & 3));
-    }
-    *q_out = make_uint2(w[0], w[1]);
-    *s_out = s;
-}
 
 // One thread owns four consecutive groups (64 B of fp16 in, 32 B of int8 + 8 B of scales out) so that enough bytes
 // are in flight per CU to cover the memory latency. Thread -> (token, K or V, head, quarter of the head) without
@@ -58,16 +35,16 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     int r; // unit index inside the token
     if (p.tok_per_block == 1) {
         const uint32_t tb = blockIdx.x / p.blocks_per_tok; // block-uniform
-        t = tb;
+        t = p.first_token + tb;
         r = (int)(blockIdx.x - tb * p.blocks_per_tok) * 256 + (int)threadIdx.x;
         if (r >= p.per_tok) return;
     } else {
         const int lt = (int)((threadIdx.x * p.inv_per_tok) >> 16); // threadIdx.x / per_tok, exact below 256
         if (lt >= p.tok_per_block) return;
-        t = (int64_t)blockIdx.x * p.tok_per_block + lt;
+        t = p.first_token + (int64_t)blockIdx.x * p.tok_per_block + lt;
         r = (int)threadIdx.x - lt * p.per_tok;
     }
-    if (t >= p.total_tokens) return;
+    if (t >= p.end_token) return;
     const int hi = r >> 2; // 0 .. 2 * kv_heads - 1: K heads, then V heads
     const int grp = (r & 3) * 4; // first of the unit's four groups
     const int kv = hi >= p.kv_heads;
@@ -107,8 +84,9 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     sdst[1] = packed[1];
 }
 
-pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream) {
-    if (a->total_new_tokens == 0 || a->batch == 0) return PPLHIP_RC_SUCCESS;
+pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token) {
+    const int64_t num_tokens = a->total_new_tokens - first_token;
+    if (num_tokens <= 0 || a->batch == 0) return PPLHIP_RC_SUCCESS;
     QuantWriteParams p;
     p.key = (const half_t*)a->d_current_key;
     p.value = (const half_t*)a->d_current_value;
@@ -125,9 +103,10 @@ pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream
     p.blocks_per_tok = p.per_tok >= 256 ? (p.per_tok + 255) / 256 : 1;
     p.tok_per_block = p.per_tok >= 256 ? 1 : 256 / p.per_tok;
     p.inv_per_tok = (65536u + (uint32_t)p.per_tok - 1) / (uint32_t)p.per_tok;
-    p.total_tokens = a->total_new_tokens;
-    const int64_t blocks = p.tok_per_block == 1 ? a->total_new_tokens * p.blocks_per_tok
-                                                : (a->total_new_tokens + p.tok_per_block - 1) / p.tok_per_block;
+    p.first_token = first_token;
+    p.end_token = a->total_new_tokens;
+    const int64_t blocks = p.tok_per_block == 1 ? num_tokens * p.blocks_per_tok
+                                                : (num_tokens + p.tok_per_block - 1) / p.tok_per_block;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "kv_quantize_write: too many groups");
     hipLaunchKernelGGL(kv_quantize_write_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("kv_quantize_write");

@@ -302,3 +302,36 @@ def test_cache_layout_3_on_device():
         paged = harness.PagedLayout(b, page_size=64, seed=3)
         both = harness.run_device(b, t, cache_prefill=cache_prefill, layout=3, paged=paged)
         assert np.array_equal(both["output"].view(np.uint16), flat["output"].view(np.uint16))
+
+
+@pytest.mark.parametrize("KVH", [8, 1])
+def test_decode_writes_its_new_tokens_into_a_slab_of_garbage(monkeypatch, KVH):
+    """Rows of the slab nobody has written hold NaN scales and -128 bytes: the decode kernel fetches the row of the
+    new token before it has quantised it, and the rows it pads a partial last stage with are multiplied by zero
+    probabilities, so none of that may reach the output. History lengths cover a last stage that is full (31 old
+    tokens + the new one), one that holds only the new token (32, 64, 0 old tokens) and ragged ones; KVH = 1 splits a
+    sequence's tokens between the waves of a workgroup."""
+    monkeypatch.setattr(harness, "SCALE_FILL", 0x7E00)
+    monkeypatch.setattr(harness, "CACHE_FILL", -128)
+    hist = [31, 32, 64, 0, 1, 33, 63, 95, 100, 257, 1024, 7]
+    b = workloads.Batch(8, KVH, 128, [1] * len(hist), hist, len(hist), name="decode into garbage")
+    check(b, workloads.make_tensors(b, seed=11))
+    # and next to prompts in the same call
+    b = workloads.Batch(8, KVH, 128, [1] * 5 + [70, 129], [31, 32, 0, 5, 200, 0, 0], 5, name="mixed into garbage")
+    check(b, workloads.make_tensors(b, seed=12))
+
+
+def test_decode_new_tokens_in_a_paged_slab_of_garbage(monkeypatch):
+    """The same with a page table: new tokens that open a page (kv position 64, 128), close one (63) or sit alone in
+    the stage that straddles two pages."""
+    monkeypatch.setattr(harness, "SCALE_FILL", 0x7E00)
+    monkeypatch.setattr(harness, "CACHE_FILL", -128)
+    hist = [63, 64, 127, 128, 0, 95, 96, 500, 1000]
+    b = workloads.Batch(8, 2, 128, [1] * len(hist), hist, len(hist), name="paged decode into garbage")
+    t = workloads.make_tensors(b, seed=13)
+    paged = harness.PagedLayout(b, page_size=64, seed=5)
+    ref = harness.run_oracle(b, t, paged=paged)
+    got = harness.run_device(b, t, paged=paged)
+    assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
+    assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
+    harness.assert_attn_close(got["output"], ref["output_f64"])
