@@ -197,9 +197,10 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     hipStream_t s = (hipStream_t)stream;
     pplhip_kv_write_args w;
     write_args_from_mhca(a, &w);
-    // the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens) into
-    // the slab itself, next to reading their history; the launch below covers the prompt tokens
-    pplhip_retcode rc = launch_kv_quantize_write(&w, s, a->decoding_batches);
+    // when the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens)
+    // into the slab itself, the launch below covers the prompt tokens only
+    const bool fused = decode_writes_new_tokens(a->decoding_batches, plan->decode_num_ranges);
+    pplhip_retcode rc = launch_kv_quantize_write(&w, s, fused ? a->decoding_batches : 0);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
     rc = launch_decode(a, plan, d_workspace, s);
     if (rc != PPLHIP_RC_SUCCESS) return rc;

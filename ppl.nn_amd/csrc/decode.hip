@@ -165,6 +165,13 @@ __device__ inline uint32_t lds_read_u16(uint32_t addr) {
     asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
     return r;
 }
+// LDS stores the compiler does not see either: a visible LDS access makes it wait for every transfer in flight
+__device__ inline void lds_write_b64(uint32_t addr, uint2 v) {
+    asm volatile("ds_write_b64 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
+__device__ inline void lds_write_b16(uint32_t addr, uint32_t v) {
+    asm volatile("ds_write_b16 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
 #define PPLHIP_WAIT_LGKMCNT(n)                                  \
     do {                                                        \
         asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory"); \
@@ -371,7 +378,9 @@ __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, 
     }
 }
 
-template <bool PAGED>
+// FUSED_WRITE: the wave that owns the tail of a sequence quantises the sequence's new token into the slab (and into
+// its stage buffer) itself; otherwise the slab already holds it.
+template <bool PAGED, bool FUSED_WRITE>
 __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63;
@@ -422,16 +431,14 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     // A segment = the part of one sequence inside this range; this wave's share of it is tokens [t_begin, t_end).
     struct Segment {
         int b;
-        int64_t seg_end, qrow, t_begin;
+        int32_t seg_end, qrow, t_begin; // positions inside a sequence and packed token rows fit 32 bits
         bool whole_sequence;
         const int64_t* page_row; // paged slab: the sequence's row of the page table
-        const char* cbase; // contiguous slab: K row of token t_begin (this kv head) in the cache / scale tensors
-        const char* sbase;
+        const char* cbase; // contiguous slab: K row of token t_begin (this kv head) in the cache tensor
         int n_stages, tail_rows_mem, tail_rows_valid;
         // this wave's chunk ends with the sequence's NEW token (its last one), which the wave quantises into the slab
-        // and into its stage buffer itself; new_row: slab offset of that token's K row for this kv head
+        // and into its stage buffer itself
         bool has_new;
-        int64_t new_row;
     };
     const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
     int64_t pos = r0;
@@ -439,32 +446,25 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         const int64_t seq_lo = p.kvstarts[b], seq_hi = p.kvstarts[b + 1];
         const int64_t seg_begin = pos - seq_lo;
         g.b = b;
-        g.seg_end = ((r1 < seq_hi) ? r1 : seq_hi) - seq_lo;
+        g.seg_end = (int32_t)(((r1 < seq_hi) ? r1 : seq_hi) - seq_lo);
         g.whole_sequence = seg_begin == 0 && g.seg_end == seq_hi - seq_lo;
         g.page_row = PAGED ? p.cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
-        g.qrow = p.seqstarts[b];
+        g.qrow = (int32_t)p.seqstarts[b];
         int64_t sub = (g.seg_end - seg_begin + tsplits - 1) / tsplits;
         sub = (sub + kStageTokens - 1) / kStageTokens * kStageTokens;
-        g.t_begin = seg_begin + (int64_t)ts * sub;
-        const int64_t t_end = (g.t_begin + sub < g.seg_end) ? g.t_begin + sub : g.seg_end; // may be <= t_begin: none
+        g.t_begin = (int32_t)(seg_begin + (int64_t)ts * sub);
+        const int64_t t_end = (g.t_begin + sub < g.seg_end) ? g.t_begin + sub : (int64_t)g.seg_end; // may be <= t_begin: none
         g.n_stages = t_end > g.t_begin ? (int)((t_end - g.t_begin + kStageTokens - 1) / kStageTokens) : 0;
         // The wave's last stage may overhang: rows past the end of the SEGMENT are clamped onto its last row (loads
         // must stay inside memory the sequence owns) and everything past the wave's own range is masked.
         const int64_t last_stage_t0 = g.t_begin + (int64_t)(g.n_stages - 1) * kStageTokens;
         g.tail_rows_mem =
-            (int)((g.seg_end - last_stage_t0) < kStageTokens ? (g.seg_end - last_stage_t0) : kStageTokens);
+            (int)(((int64_t)g.seg_end - last_stage_t0) < kStageTokens ? ((int64_t)g.seg_end - last_stage_t0) : kStageTokens);
         g.tail_rows_valid = (int)(t_end - last_stage_t0);
         const int64_t seq_len = seq_hi - seq_lo;
-        g.has_new = p.cur_key != nullptr && g.n_stages > 0 && t_end == seq_len;
-        {
-            const int64_t tl = seq_len - 1;
-            const int64_t tok = PAGED ? g.page_row[tl >> p.page_shift] + (tl & ((int64_t(1) << p.page_shift) - 1))
-                                      : p.cachestarts[b] + tl;
-            g.new_row = tok * (int64_t)stride + head_off;
-        }
-        const int64_t row0 = (PAGED ? 0 : (p.cachestarts[b] + g.t_begin) * (int64_t)stride) + head_off;
+        g.has_new = FUSED_WRITE && g.n_stages > 0 && t_end == seq_hi - seq_lo;
+        const int64_t row0 = (PAGED ? 0 : (p.cachestarts[b] + (int64_t)g.t_begin) * (int64_t)stride) + head_off;
         g.cbase = reinterpret_cast<const char*>(p.cache) + row0;
-        g.sbase = reinterpret_cast<const char*>(p.scale) + (row0 / kQuantGroup) * 2;
         pos = seq_lo + g.seg_end;
         ++b;
     };
@@ -473,7 +473,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         char* dst = wave_lds + slot * kStageBytes;
         if (PAGED) {
             // a stage of 32 tokens touches at most two pages (pages hold >= 64 tokens)
-            const int64_t t0 = g.t_begin + (int64_t)idx * kStageTokens;
+            const int64_t t0 = (int64_t)g.t_begin + (int64_t)idx * kStageTokens;
             const int64_t in_page = t0 & ((int64_t(1) << p.page_shift) - 1);
             const int64_t left = (int64_t(1) << p.page_shift) - in_page; // rows of the stage in its first page
             const int split = left < kStageTokens ? (int)left : kStageTokens;
@@ -489,7 +489,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
             dma_stage_paged(dst, ca, cb, sa, sb, split, off, kv_off, kv_off_s);
         } else {
             const char* cb = make_uniform(g.cbase + idx * step_c);
-            const char* sb = make_uniform(g.sbase + idx * step_s);
+            const char* sb = make_uniform(reinterpret_cast<const char*>(p.scale) +
+                                          ((g.cbase - reinterpret_cast<const char*>(p.cache)) / kQuantGroup) * 2 + idx * step_s);
             dma_stage(dst, cb, sb, off, kv_off, kv_off_s);
         }
     };
@@ -508,17 +509,17 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     };
 
     // Q^T as the B operand, kept for a whole segment: q[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
-    constexpr int kQueryLoads = 5; // four query pieces + the lane's group of the sequence's new token
+    // four query pieces (+ the lane's group of the sequence's new token)
+    constexpr int kQueryLoads = FUSED_WRITE ? 5 : 4;
     // lanes 0..15: groups of the new token's K row (this kv head), lanes 16..31: of its V row (upper half-wave mirrors)
     auto load_query = [&](const Segment& g, half8_t (&q)[2][2], uint4& newtok) {
-        {
-            const half_t* src = ((lane & 16) ? p.cur_value : p.cur_key);
-            if (src == nullptr) src = p.q; // (never used then; keeps the load count the same)
-            else src += (g.qrow * p.kv_heads + kvh) * kDh + 8 * (lane & 15);
+        if (FUSED_WRITE) {
+            const half_t* src = ((lane & 16) ? p.cur_value : p.cur_key) +
+                                ((int64_t)g.qrow * p.kv_heads + kvh) * kDh + 8 * (lane & 15);
             newtok = *reinterpret_cast<const uint4*>(src);
         }
         const bool live = m < p.rep;
-        const half_t* qp = p.q + ((g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
+        const half_t* qp = p.q + (((int64_t)g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
@@ -570,7 +571,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (it + 1 == cur.n_stages && cur.has_new) {
+                if (FUSED_WRITE && it + 1 == cur.n_stages && cur.has_new) {
                     // The stage has landed with whatever the slab held in the new token's row: the row is replaced in
                     // the stage buffer by the freshly quantised token (LDS operations of one wave execute in order, so
                     // the reads below see it), and the same bytes go to the slab.
@@ -579,14 +580,26 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                         uint2 qv;
                         half_t sc;
                         quantize_group8(newB, &qv, &sc);
-                        char* st = wave_lds + slot * kStageBytes;
-                        *reinterpret_cast<uint2*>(st + (isv ? kLdsV : kLdsK) + r * 128 + (((grp >> 1) ^ (r & 7)) * 16) +
-                                                  (grp & 1) * 8) = qv;
-                        *reinterpret_cast<half_t*>(st + (isv ? kLdsVs : kLdsKs) + r * 32 + grp * 2) = sc;
+                        const uint32_t st = wave_lds_addr + slot * kStageBytes;
+                        uint16_t sbits;
+                        __builtin_memcpy(&sbits, &sc, 2);
+                        lds_write_b64(st + (isv ? kLdsV : kLdsK) + r * 128 + (((grp >> 1) ^ (r & 7)) * 16) + (grp & 1) * 8,
+                                      qv);
+                        lds_write_b16(st + (isv ? kLdsVs : kLdsKs) + r * 32 + grp * 2, sbits);
                         if (cur.tail_rows_mem == 1) // the new token is the stage's only row: every row is a copy of it
                             for (int r2 = 1; r2 < kStageTokens; ++r2)
-                                *reinterpret_cast<half_t*>(st + (isv ? kLdsVs : kLdsKs) + r2 * 32 + grp * 2) = sc;
-                        const int64_t row = cur.new_row + (isv ? (int64_t)kv_off : 0);
+                                lds_write_b16(st + (isv ? kLdsVs : kLdsKs) + r2 * 32 + grp * 2, sbits);
+                        // the token's K row of this kv head in the slab: r rows into the wave's last stage
+                        const int64_t tl = (int64_t)(cur.n_stages - 1) * kStageTokens + r; // relative to t_begin
+                        int64_t row;
+                        if (PAGED) {
+                            const int64_t ta = (int64_t)cur.t_begin + tl;
+                            row = (cur.page_row[ta >> p.page_shift] + (ta & ((int64_t(1) << p.page_shift) - 1))) *
+                                      (int64_t)stride + head_off;
+                        } else {
+                            row = (cur.cbase - reinterpret_cast<const char*>(p.cache)) + tl * (int64_t)stride;
+                        }
+                        row += isv ? (int64_t)kv_off : 0;
                         *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
                         p.scale[row / kQuantGroup + grp] = sc;
                     }
@@ -604,7 +617,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
             if (m < p.rep) {
                 const int head = kvh * p.rep + m;
                 if (cur.whole_sequence) {
-                    half_t* dst = p.out + (cur.qrow * p.num_heads + head) * kDh + 32 * kq;
+                    half_t* dst = p.out + ((int64_t)cur.qrow * p.num_heads + head) * kDh + 32 * kq;
                     const float inv_l = 1.0f / l_tot;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -664,7 +677,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                 }
                 const int head = (hg * p.hpb + kl) * p.rep + h;
                 if (cur.whole_sequence) {
-                    p.out[(cur.qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
+                    p.out[((int64_t)cur.qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
                 } else {
                     const int64_t prow = (s_idx + cur.b) * p.num_heads + head;
                     p.part_acc[prow * kDh + d] = acc;
@@ -761,6 +774,14 @@ int decode_heads_per_block(int kv_heads) {
     return hpb;
 }
 
+// Whether the decode kernel quantises the decode sequences' new tokens itself. It saves the separate launch, but
+// the tail of every sequence then costs its owner extra work on the launch's critical path: worth it as long as at
+// most half of the workgroups own a tail (measured: 120 sequences over 256 ranges -2.7 %, 8 over 512 -7 %, 64 over
+// 64 +3 %).
+bool decode_writes_new_tokens(int64_t decoding_batches, int num_ranges) {
+    return decoding_batches > 0 && 2 * decoding_batches <= (int64_t)num_ranges;
+}
+
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
     const int nd = (int)a->decoding_batches;
     if (nd == 0) return PPLHIP_RC_SUCCESS;
@@ -800,8 +821,10 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
         PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: no current device");
     if (!(lds_opted_in.load(std::memory_order_relaxed) >> dev & 1)) {
-        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true>)}) {
+        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true>)}) {
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
             if (e != hipSuccess)
                 PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
@@ -809,12 +832,16 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
         }
         lds_opted_in.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
     }
-    if (p.page_shift)
-        hipLaunchKernelGGL(decode_int8kv_kernel<true>, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes,
-                           stream, p);
+    const bool fused = decode_writes_new_tokens(nd, p.num_ranges);
+    const dim3 grid((unsigned)blocks), block(kDecodeWaves * kWave);
+    if (p.page_shift && fused)
+        hipLaunchKernelGGL((decode_int8kv_kernel<true, true>), grid, block, lds_bytes, stream, p);
+    else if (p.page_shift)
+        hipLaunchKernelGGL((decode_int8kv_kernel<true, false>), grid, block, lds_bytes, stream, p);
+    else if (fused)
+        hipLaunchKernelGGL((decode_int8kv_kernel<false, true>), grid, block, lds_bytes, stream, p);
     else
-        hipLaunchKernelGGL(decode_int8kv_kernel<false>, dim3((unsigned)blocks), dim3(kDecodeWaves * kWave), lds_bytes,
-                           stream, p);
+        hipLaunchKernelGGL((decode_int8kv_kernel<false, false>), grid, block, lds_bytes, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
     hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_merge");
