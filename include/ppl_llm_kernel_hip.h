@@ -130,7 +130,9 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* args, pplhip_mhca_pla
 
 /* Enqueues: quantize-on-write of the new K/V tokens, decode attention (+ split-k merge) for the first
  * `decoding_batches` sequences and causal prefill attention for the rest. Replaces `forward(stream)`
- * (multi_head_cache_attention_kernel.cc:230). `d_workspace` must hold plan->workspace_bytes (256-byte aligned). */
+ * (multi_head_cache_attention_kernel.cc:230). `d_workspace` must hold plan->workspace_bytes (256-byte aligned).
+ * As in the reference, the decode sequences come first and bring exactly one new token each (their packed token
+ * index is their sequence index); which kernel quantises which new token into the cache is an implementation detail. */
 pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* args, const pplhip_mhca_plan* plan, void* d_workspace,
                                    void* stream);
 
