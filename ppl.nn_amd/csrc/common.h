@@ -124,10 +124,12 @@ inline int ceil_div(int64_t a, int64_t b) {
 
 // launchers implemented in the .hip files
 // first_token: packed new tokens before it are skipped (the decode kernel writes the decode tokens itself)
-pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token = 0);
+pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token = 0,
+                                        int64_t end_token = -1);
 pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream_t stream);
 int decode_heads_per_block(int kv_heads);
 bool decode_writes_new_tokens(int64_t decoding_batches, int num_ranges);
+bool prefill_writes_new_tokens(const pplhip_mhca_args* a);
 int decode_blocks_per_cu();
 int decode_waves_per_block();
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);

@@ -84,8 +84,10 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     sdst[1] = packed[1];
 }
 
-pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token) {
-    const int64_t num_tokens = a->total_new_tokens - first_token;
+pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token,
+                                        int64_t end_token) {
+    if (end_token < 0) end_token = a->total_new_tokens;
+    const int64_t num_tokens = end_token - first_token;
     if (num_tokens <= 0 || a->batch == 0) return PPLHIP_RC_SUCCESS;
     QuantWriteParams p;
     p.key = (const half_t*)a->d_current_key;
@@ -104,7 +106,7 @@ pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream
     p.tok_per_block = p.per_tok >= 256 ? 1 : 256 / p.per_tok;
     p.inv_per_tok = (65536u + (uint32_t)p.per_tok - 1) / (uint32_t)p.per_tok;
     p.first_token = first_token;
-    p.end_token = a->total_new_tokens;
+    p.end_token = end_token;
     const int64_t blocks = p.tok_per_block == 1 ? num_tokens * p.blocks_per_tok
                                                 : (num_tokens + p.tok_per_block - 1) / p.tok_per_block;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "kv_quantize_write: too many groups");

@@ -54,6 +54,12 @@ struct PrefillParams {
     int32_t num_heads, kv_heads, rep;
     int32_t is_causal;
     float score_scale; // log2(e) / sqrt(Dh)
+    // quantize-on-write of the prompt tokens, done by this launch (prefill_f16_kernel only; w_cache null: not)
+    int8_t* w_cache;
+    half_t* w_scale;
+    int64_t w_first_token, w_end_token; // packed new tokens [first, end)
+    int32_t w_batch; // all sequences of the call (the sequence of a token is looked up in seqstarts)
+    int32_t w_per_tok; // 4-group units per token: 2 * kv_heads * 4
 };
 
 // A thread's share of a 64-token K/V tile: channels 8*col .. 8*col+7 (col = tid & 15) of the four consecutive tokens
@@ -582,11 +588,53 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     const int ntiles = (int)((L + kBM - 1) / kBM);
     const int ntiles_max = gridDim.x / per_tile;
     const int qt = ntiles_max - 1 - qt_rev;
-    if (qt >= ntiles) return;
-    const int64_t q0 = (int64_t)qt * kBM;
-
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    // This launch's share of the prompt tokens' quantize-on-write: the units of four quantisation groups are dealt
+    // out over ALL threads of the grid (workgroups without a query tile do theirs and leave). A workgroup with a
+    // tile runs it between issuing its first transfers and waiting for them, where it would otherwise sit idle.
+    auto write_share = [&]() {
+        if (p.w_cache == nullptr) return;
+        // (workgroup i takes units 256*i .. 256*i+255: the work sits in the leading workgroups, which all run in the
+        // first round, when every workgroup of the launch is waiting for its first loads and the vector ALUs have
+        // nothing else to do; spreading it evenly over the grid measured 3 us slower)
+        const int64_t units = (p.w_end_token - p.w_first_token) * p.w_per_tok;
+        for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.x * 256) {
+            const int64_t t = p.w_first_token + u / p.w_per_tok;
+            const int r = (int)(u % p.w_per_tok);
+            const int hi = r >> 2, grp = (r & 3) * 4; // K heads then V heads; first of the unit's four groups
+            const int kv = hi >= p.kv_heads, wh = hi - kv * p.kv_heads;
+            const uint4* src = reinterpret_cast<const uint4*>((kv ? p.v : p.k) + ((t * p.kv_heads + wh) * 16 + grp) * 8);
+            uint4 raw[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) raw[i] = src[i];
+            const int64_t t0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(t >> 32)) << 32) |
+                               (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+            const int wb = __all(t == t0) ? find_sequence_wave(p.seqstarts, p.w_batch, t0)
+                                          : find_sequence(p.seqstarts, p.w_batch, t);
+            const int64_t tok = p.pages.token(wb, p.start_pos[wb] + (t - p.seqstarts[wb]));
+            uint2 q[4];
+            half_t sc[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) quantize_group8(raw[i], &q[i], &sc[i]);
+            const int64_t row = p.addr.row(tok, kv, wh);
+            uint4* dst = reinterpret_cast<uint4*>(p.w_cache + row + grp * 8);
+            dst[0] = make_uint4(q[0].x, q[0].y, q[1].x, q[1].y);
+            dst[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
+            uint32_t packed[2];
+            __builtin_memcpy(packed, sc, 8);
+            uint32_t* sdst = reinterpret_cast<uint32_t*>(p.w_scale + row / kQuantGroup + grp);
+            sdst[0] = packed[0];
+            sdst[1] = packed[1];
+        }
+    };
+    if (qt >= ntiles) {
+        write_share();
+        return;
+    }
+    const int64_t q0 = (int64_t)qt * kBM;
+
     const int n = lane & 31;
     const int hb = lane >> 5;
     const int64_t row = q0 + 32 * wave + n;
@@ -701,6 +749,7 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
         return a;
     };
 
+    write_share();
     // tile 0 and the queries have to be there before the first MFMA (see prefill_attention_kernel for why the wait
     // is explicit)
     __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -885,6 +934,12 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     }
 }
 
+// Whether the prefill launch quantises the prompt tokens into the slab itself (instead of a separate launch before
+// it): whenever it reads K/V from the fp16 inputs, i.e. does not depend on the slab holding them.
+bool prefill_writes_new_tokens(const pplhip_mhca_args* a) {
+    return !a->enable_cache_prefill && a->batch > a->decoding_batches;
+}
+
 pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, hipStream_t stream) {
     const int npre = (int)(a->batch - a->decoding_batches);
     if (npre <= 0 || plan->prefill_num_q_tiles <= 0) return PPLHIP_RC_SUCCESS;
@@ -908,6 +963,15 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     p.is_causal = a->is_causal;
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
     p.num_seqs = npre;
+    p.w_cache = nullptr;
+    if (prefill_writes_new_tokens(a)) {
+        p.w_cache = (int8_t*)a->d_cache;
+        p.w_scale = (half_t*)a->d_scale;
+        p.w_first_token = a->decoding_batches; // one new token per decode sequence, then the prompts
+        p.w_end_token = a->total_new_tokens;
+        p.w_batch = (int32_t)a->batch;
+        p.w_per_tok = 2 * a->num_kv_heads * 4;
+    }
     const int64_t blocks = (int64_t)plan->prefill_num_q_tiles * npre * a->num_heads;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many query tiles in one call");
     const dim3 grid((unsigned)blocks);
@@ -942,6 +1006,8 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
     p.is_causal = a->is_causal;
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
     p.num_seqs = (int32_t)a->batch;
+    p.w_cache = nullptr; // MultiHeadAttention has no cache to write
+    p.w_scale = nullptr;
     const int64_t q_tiles = (a->max_seqlen + kBM - 1) / kBM;
     const int64_t blocks = q_tiles * a->batch * a->num_heads;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many query tiles in one call");
