@@ -346,7 +346,7 @@ def main():
                    "slabs_rotated": N_SLABS},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": recorded_traffic(args.workload),
-                     "kernel": "decode_int8kv_kernel (+ kv_quantize_write + decode_merge in the same call)",
+                     "kernel": "decode_int8kv_kernel (reads the int8 slab once, quantises the new tokens into it) + decode_merge in the same call",
                      "algorithmic_bytes_per_launch": dec_bytes, "event_ms_per_launch": ev_ms},
     }
     if pre_b is not None:
