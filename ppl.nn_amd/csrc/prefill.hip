@@ -690,21 +690,10 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
         const half_t* qp = p.q + ((s0 + (row_ok ? row : 0)) * p.num_heads + head) * kPDh + 8 * hb;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-            uint4 x = *reinterpret_cast<const uint4*>(qp + 16 * kk);
-            if (!row_ok) x = make_uint4(0, 0, 0, 0);
+            const uint4 x = *reinterpret_cast<const uint4*>(qp + 16 * kk); // rows past the end: row 0, zeroed below
             __builtin_memcpy(&qB[kk], &x, 16);
         }
     }
-    // the queries are scaled once by log2(e) / sqrt(Dh), so that the MFMA result is the exponent of exp2 directly and
-    // no per-score multiply is left in the loop. Packed fp16 multiplies: the factor is rounded to fp16, i.e. the
-    // softmax runs at a temperature that is off by at most 2^-12 relative, far inside the output tolerance.
-    {
-        const half_t c16 = (half_t)p.score_scale;
-        const half8_t cv = {c16, c16, c16, c16, c16, c16, c16, c16};
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) qB[kk] = qB[kk] * cv;
-    }
-
     float16_t oT[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -754,6 +743,18 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     // is explicit)
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
+    // the queries are scaled once by log2(e) / sqrt(Dh), so that the MFMA result is the exponent of exp2 directly and
+    // no per-score multiply is left in the loop. Packed fp16 multiplies: the factor is rounded to fp16, i.e. the
+    // softmax runs at a temperature that is off by at most 2^-12 relative, far inside the output tolerance.
+    {
+        // (rows past the end of the sequence loaded a real row to stay inside memory: factor 0 makes them zero
+        // queries, whose scores are finite and whose output rows are never stored)
+        const half_t c16 = row_ok ? (half_t)p.score_scale : (half_t)0.f;
+        const half8_t cv = {c16, c16, c16, c16, c16, c16, c16, c16};
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) qB[kk] = qB[kk] * cv;
+    }
+
 
     // Software pipeline over the tiles: iteration t exponentiates the scores of tile t (vector ALU) while the MFMAs
     // of tile t + 1's scores are issued from the same instruction stream, then accumulates P(t) * V(t). Ring use in
