@@ -166,11 +166,15 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         if (const char* env = getenv("PPLHIP_DECODE_TASKS_PER_SLOT")) { // tuning aid, in workgroups per slot
             if (atoll(env) > 0) half_slots = 2 * atoll(env);
         }
-        int64_t ranges = (slots * half_slots / 2 + groups - 1) / groups;
+        // ranges x groups workgroups must not spill over the slots (a second, nearly empty round doubles the time:
+        // 40 kv heads = 10 groups took 56 ranges = 560 workgroups on 512 slots), so everything rounds DOWN to the
+        // multiple of 8 the XCD-aware numbering needs
+        int64_t ranges = slots * half_slots / 2 / groups;
         // never more ranges than 128-token pieces of the worst case (every sequence max_kvlen long)
         const int64_t cap = (nd * a->max_kvlen + 127) / 128;
         if (ranges > cap) ranges = cap;
-        ranges = (ranges + 7) / 8 * 8;
+        ranges = ranges / 8 * 8;
+        if (ranges < 8) ranges = 8;
         if (ranges > 0x3fffffff) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many ranges");
         plan->decode_num_ranges = (int32_t)ranges;
         plan->decode_heads_per_block = hpb;
