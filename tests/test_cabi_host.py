@@ -94,6 +94,24 @@ def test_prepare_rejects(hiplib, mutate, rc):
     assert len(hiplib.pplhip_last_error()) > 0
 
 
+@pytest.mark.parametrize("kvh", [1, 2, 3, 4, 5, 8, 12, 16, 32, 40, 64])
+def test_decode_plan_fills_one_round_of_workgroup_slots(hiplib, kvh):
+    """The decode launch runs (ranges x groups of <= 4 kv heads) workgroups, two per compute unit: with the default
+    knob they must fit the 512 slots of the 256-CU part (that is also what prepare assumes without a device), or a
+    nearly empty second round doubles the time; a multiple of 8 for the XCD-aware numbering."""
+    b = workloads.Batch(kvh * 2, kvh, 128, [1] * 200, [4000] * 200, 200)
+    a = cabi.MhcaArgs()
+    fake = lambda t: C.c_void_p(0x1000)
+    harness.fill_mhca_args(a, b, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, ptr=fake, split_k=1)
+    plan = cabi.MhcaPlan()
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+    groups = kvh // plan.decode_heads_per_block
+    assert kvh % plan.decode_heads_per_block == 0 and plan.decode_heads_per_block <= 4
+    assert plan.decode_num_ranges % 8 == 0 and plan.decode_num_ranges >= 8
+    assert plan.decode_num_ranges * groups <= 512 or plan.decode_num_ranges == 8
+    assert (plan.decode_num_ranges + 8) * groups > 512  # and no more than one step of 8 below it
+
+
 def test_prepare_accepts_paged_cache(hiplib):
     a, plan = _valid_args(), cabi.MhcaPlan()
     a.cache_mode, a.cachestart_stride_b, a.page_size = 1, 4, 128
