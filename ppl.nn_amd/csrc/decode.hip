@@ -725,15 +725,29 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
     if (s_lo == s_hi) return;
     float mx = -INFINITY, l = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    for (int64_t s = s_lo + g; s <= s_hi; s += kMergeGroups) {
-        const int64_t prow = (s + b) * p.num_heads + head;
-        const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
-        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
-        const float m_new = fmaxf(mx, mc);
-        const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc - m_new);
-        acc = acc * w_old + a * w_new;
-        l = l * w_old + lc * w_new;
-        mx = m_new;
+    // four slots per step, their loads issued together: a long sequence has dozens of slots per lane group, and one
+    // memory latency per slot would add up (slots past the end repeat the last one with weight 0)
+    for (int64_t s = s_lo + g; s <= s_hi; s += 4 * kMergeGroups) {
+        float mc[4], lc[4];
+        float4_t a[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t su = s + u * kMergeGroups;
+            const int64_t prow = ((su <= s_hi ? su : s_hi) + b) * p.num_heads + head;
+            mc[u] = p.part_ml[prow * 2];
+            lc[u] = p.part_ml[prow * 2 + 1];
+            a[u] = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
+            if (su > s_hi) mc[u] = -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float m_new = fmaxf(mx, mc[u]);
+            // (mx = m_new = -inf can only happen for padding slots in front of a real one: never, the first is real)
+            const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc[u] - m_new);
+            acc = acc * w_old + a[u] * w_new;
+            l = l * w_old + lc[u] * w_new;
+            mx = m_new;
+        }
     }
     red[g][d4 + 0] = acc[0];
     red[g][d4 + 1] = acc[1];
