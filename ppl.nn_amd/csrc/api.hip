@@ -179,7 +179,8 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         plan->decode_num_ranges = (int32_t)ranges;
         plan->decode_heads_per_block = hpb;
         const uint64_t rows = ((uint64_t)ranges + (uint64_t)nd) * a->num_heads;
-        plan->workspace_bytes = rows * (a->head_dim + 2) * sizeof(float);
+        // partial accumulators and (max, sum) pairs per (slot, head), then one int per range (its first sequence)
+        plan->workspace_bytes = rows * (a->head_dim + 2) * sizeof(float) + (uint64_t)ranges * sizeof(int32_t);
     }
     // ---- prefill
     plan->prefill_q_tile = 128;

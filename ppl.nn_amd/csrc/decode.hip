@@ -73,11 +73,13 @@ struct DecodeParams {
     half_t* out; // [S, H, Dh]
     float* part_acc; // [slots, H, Dh], slots = num_ranges + nd
     float* part_ml; // [slots, H, 2]
+    int32_t* range_first; // [num_ranges] first sequence of every range, written by the decode kernel for the merge
     CacheAddr addr;
     int32_t nd; // decode sequences (the first nd entries of the tables)
     int32_t num_heads, kv_heads, rep; // rep = num_heads / kv_heads (<= 16)
     int32_t num_ranges; // S, a multiple of 8
     int32_t hpb; // kv heads per workgroup: min(kv_heads, 4), a power of two dividing kv_heads
+    int32_t merge_by_boundary; // merge kernel: blockIdx.y counts range boundaries instead of sequences
     float score_scale; // log2(e) / sqrt(Dh)
 };
 
@@ -123,15 +125,25 @@ __device__ inline half8_t dequant8(uint32_t w0, uint32_t w1, half_t scale) {
     return half8_t{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
 }
 
+// Reductions over the four 16-lane rows of the wave (lanes l, l^16, l^32, l^48) in the vector ALU: the swap
+// instructions hand every lane of a row pair both rows' values, where a shuffle would be a round trip through the LDS
+// pipeline. v_permlane16_swap(x, y) exchanges the odd rows of x with the even rows of y; v_permlane32_swap(x, y) the
+// upper half of x with the lower half of y; with x = y = v the two results hold the two partners' values.
 __device__ inline float wave_max_over_quads(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
+    const uint32_t u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const uint32_t w = __float_as_uint(v);
+    const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ inline float wave_sum_over_quads(float v) {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+    const uint32_t u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const uint32_t w = __float_as_uint(v);
+    const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // Pins a pointer that is wave-uniform by construction into scalar registers, so that memory instructions take the
@@ -427,6 +439,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         b += __builtin_popcountll(__ballot(ends_before));
     }
     b = __builtin_amdgcn_readfirstlane(b);
+    if (hg == 0 && threadIdx.x == 0) p.range_first[s_idx] = b; // saves the merge kernel the same search
 
     // A segment = the part of one sequence inside this range; this wave's share of it is tokens [t_begin, t_end).
     struct Segment {
@@ -716,11 +729,21 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
 constexpr int kMergeGroups = 8;
 __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p) {
     __shared__ float red[kMergeGroups][kDh + 2];
-    const int b = blockIdx.y;
     const int head = blockIdx.x;
     const int g = threadIdx.x >> 5;
     const int d4 = (threadIdx.x & 31) * 4;
     const int64_t R = range_tokens(p.kvstarts[p.nd], p.num_ranges);
+    // blockIdx.y is a sequence, or (when there are more sequences than ranges) a boundary between two ranges: only
+    // a sequence that straddles a boundary has anything to merge, and it is handled by the first boundary it crosses
+    int b;
+    if (p.merge_by_boundary) {
+        const int64_t edge = ((int64_t)blockIdx.y + 1) * R; // first token of range blockIdx.y + 1
+        if (edge >= p.kvstarts[p.nd]) return;
+        b = p.range_first[blockIdx.y + 1]; // the sequence that holds token `edge` (found by the decode kernel)
+        if (p.kvstarts[b] >= edge || p.kvstarts[b] / R != blockIdx.y) return; // starts there, or crossed one before
+    } else {
+        b = blockIdx.y;
+    }
     const int64_t s_lo = p.kvstarts[b] / R, s_hi = (p.kvstarts[b + 1] - 1) / R;
     if (s_lo == s_hi) return;
     float mx = -INFINITY, l = 0.f;
@@ -825,6 +848,7 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     const size_t slots = (size_t)p.num_ranges + nd;
     p.part_acc = (float*)ws;
     p.part_ml = (float*)((char*)ws + slots * p.num_heads * kDh * sizeof(float));
+    p.range_first = (int32_t*)((char*)ws + slots * p.num_heads * (kDh + 2) * sizeof(float));
     const int64_t blocks = (int64_t)p.num_ranges * (p.kv_heads / p.hpb);
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many tasks");
     const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
@@ -857,7 +881,11 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     else
         hipLaunchKernelGGL((decode_int8kv_kernel<false, false>), grid, block, lds_bytes, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
-    hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, nd), dim3(256), 0, stream, p);
+    // the sequences that need merging are those that straddle a range boundary: at most num_ranges - 1 of them,
+    // however many sequences there are (2048 short sequences launched 65k workgroups that all left at once: 35 us)
+    p.merge_by_boundary = nd > p.num_ranges - 1;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, p.merge_by_boundary ? p.num_ranges - 1 : nd), dim3(256), 0,
+                       stream, p);
     PPLHIP_CHECK_LAUNCH("decode_merge");
     return PPLHIP_RC_SUCCESS;
 }
