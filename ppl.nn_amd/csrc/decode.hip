@@ -192,6 +192,19 @@ __device__ inline void lds_write_b16(uint32_t addr, uint32_t v) {
 
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at "no wait"), gfx9 encoding
 #define PPLHIP_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | 0x0f70)
+// the same with `extra` (0, 2, 4, 6, 10 or 12: the result stores of the previous segment) younger operations more left
+// in flight; the immediate has to be a constant
+#define PPLHIP_WAIT_VMCNT_PLUS(n, extra)              \
+    do {                                              \
+        switch (extra) {                              \
+            case 2: PPLHIP_WAIT_VMCNT((n) + 2); break;   \
+            case 4: PPLHIP_WAIT_VMCNT((n) + 4); break;   \
+            case 6: PPLHIP_WAIT_VMCNT((n) + 6); break;   \
+            case 10: PPLHIP_WAIT_VMCNT((n) + 10); break; \
+            case 12: PPLHIP_WAIT_VMCNT((n) + 12); break; \
+            default: PPLHIP_WAIT_VMCNT(n); break;        \
+        }                                             \
+    } while (0)
 constexpr int kDmaPerStage = 2 * (kStageTokens / 8) + 2; // 4 K + 4 V + K scales + V scales
 
 // Per-lane source offsets of the stage DMA (relative to the wave-uniform stage base).
@@ -551,6 +564,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     next_segment(cur);
     int slot0 = 0; // stage buffer of the current segment's stage 0
     bool cur_in_flight = false; // stage 0 of `cur` already enqueued by the previous segment's last iteration
+    // store instructions issued behind the stage-0 transfers of a segment that was put in flight early (see the waits)
+    int pending_stores = 0;
     half8_t qB[2][2], qN[2][2];
     uint4 newB, newN;
     load_query(cur, qB, newB);
@@ -570,19 +585,22 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                 if (it + 1 < cur.n_stages) {
                     issue(cur, it + 1, slot ^ 1);
                     // everything older than the transfers just enqueued has landed: stage `it`, and at it == 0 the
-                    // query loads (global stores still in flight only make this wait longer, never shorter)
-                    PPLHIP_WAIT_VMCNT(kDmaPerStage);
+                    // query loads. The previous segment's result stores were issued AFTER this segment's stage 0 (which
+                    // was put in flight ahead of them), so they may stay in flight: waiting for their acknowledgement
+                    // here cost 2 us per sequence boundary.
+                    PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage, pending_stores);
                 } else {
                     has_next = direct && pos < r1;
                     if (has_next) {
                         next_segment(nxt);
                         load_query(nxt, qN, newN); // older than the transfers below: landed before they are waited for
                         issue(nxt, 0, slot ^ 1);
-                        PPLHIP_WAIT_VMCNT(kDmaPerStage + kQueryLoads); // stage `it` only
+                        PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage + kQueryLoads, pending_stores); // stage `it` only
                     } else {
-                        PPLHIP_WAIT_VMCNT(0);
+                        PPLHIP_WAIT_VMCNT_PLUS(0, pending_stores);
                     }
                 }
+                pending_stores = 0;
                 __builtin_amdgcn_sched_barrier(0);
                 if (FUSED_WRITE && it + 1 == cur.n_stages && cur.has_new) {
                     // The stage has landed with whatever the slab held in the new token's row: the row is replaced in
@@ -615,6 +633,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                         row += isv ? (int64_t)kv_off : 0;
                         *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
                         p.scale[row / kQuantGroup + grp] = sc;
+                        // (counted below: two store instructions)
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -704,6 +723,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         }
 
         if (has_next) { // its stage 0 is already in flight, in the buffer the last stage did not use
+            // (has_next implies the register epilogue: 4 stores of a finished row, or 8 + 2 of a partial result, and
+            // two more where the wave wrote its sequence's new token)
+            pending_stores = (cur.whole_sequence ? 4 : 10) + ((FUSED_WRITE && cur.has_new) ? 2 : 0);
             slot0 = (slot0 + cur.n_stages) & 1;
             cur = nxt;
 #pragma unroll
