@@ -335,3 +335,19 @@ def test_decode_new_tokens_in_a_paged_slab_of_garbage(monkeypatch):
     assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
     assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
     harness.assert_attn_close(got["output"], ref["output_f64"])
+
+
+@pytest.mark.parametrize("KVH", [8, 2])
+def test_more_decode_sequences_than_ranges(KVH):
+    """20 to 40 short sequences over 8 ranges: several sequence boundaries inside every range, the partial results of
+    the sequences that straddle a range boundary are merged by the (head, boundary) grid, and some ranges hold whole
+    sequences only."""
+    plans = []
+    b = workloads.Batch(8, KVH, 128, [1] * 20, [100] * 20, 20, name="20 short sequences")
+    check(b, workloads.make_tensors(b, seed=21), plans=plans)
+    assert plans[-1].decode_num_ranges <= 20
+    rng = np.random.default_rng(22)
+    hist = rng.integers(0, 90, 40).tolist()
+    b = workloads.Batch(8, KVH, 128, [1] * 40, hist, 40, name="40 ragged short sequences")
+    check(b, workloads.make_tensors(b, seed=23), plans=plans)
+    assert plans[-1].decode_num_ranges <= 40
