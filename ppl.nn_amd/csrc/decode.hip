@@ -307,8 +307,10 @@ __device__ inline void read_stage_sub(uint4 (&kr)[2], uint2& ksr, uint2 (&vr)[4]
 
 // lds_stage: LDS byte address of the stage buffer. rows_valid: tokens of this stage that belong to the wave's range
 // (1..32); the rest is masked out of the softmax.
+template <typename AfterReads>
 __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, SoftmaxState& ss,
-                                     const half8_t (&qB)[2][2], int kq, int rows_valid, float score_scale) {
+                                     const half8_t (&qB)[2][2], int kq, int rows_valid, float score_scale,
+                                     AfterReads&& after_reads) {
     static_assert(kSubBlocks == 2, "the stage is processed as two 16-token sub-blocks");
     const uint32_t ak[2] = {ro.k[0] + lds_stage, ro.k[1] + lds_stage};
     const uint32_t aks = ro.ks + lds_stage, avs = ro.vs + lds_stage;
@@ -320,6 +322,9 @@ __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, 
     read_stage_sub<0>(kr[0], ksr[0], vraw[0], vsr[0], ak, aks, av, avs);
     read_stage_sub<1>(kr[1], ksr[1], vraw[1], vsr[1], ak, aks, av, avs);
     PPLHIP_WAIT_LGKMCNT(0);
+    // the stage now lives in registers: its buffer may take the transfers of a later stage while the arithmetic runs
+    after_reads();
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- scores S^T[token, head]: v_mfma_f32_16x16x32_f16, one quantisation group (8 channels) per lane per MFMA
     float4_t sc[kSubBlocks];
@@ -405,7 +410,9 @@ __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, 
 
 // FUSED_WRITE: the wave that owns the tail of a sequence quantises the sequence's new token into the slab (and into
 // its stage buffer) itself; otherwise the slab already holds it.
-template <bool PAGED, bool FUSED_WRITE>
+// DIRECT: every wave owns a whole kv head (hpb == waves per workgroup); otherwise the waves split the tokens of a kv
+// head and combine through LDS.
+template <bool PAGED, bool FUSED_WRITE, bool DIRECT>
 __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63;
@@ -423,8 +430,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
 
     const int kvh_local = wave & (p.hpb - 1);
     const int kvh = hg * p.hpb + kvh_local;
-    const int tsplits = kDecodeWaves / p.hpb;
-    const int ts = wave / p.hpb;
+    const int tsplits = DIRECT ? 1 : kDecodeWaves / p.hpb;
+    const int ts = DIRECT ? 0 : wave / p.hpb;
     const int m = lane & 15;
     const int kq = lane >> 4;
 
@@ -559,7 +566,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     // When every wave owns a whole kv head (no token split inside the workgroup) nothing is combined through LDS, the
     // stage buffers stay private to their wave, and the first stage of the NEXT segment is put in flight before the
     // current segment's results are normalised and stored: the transition between two sequences costs no DMA bubble.
-    const bool direct = tsplits == 1;
+    constexpr bool direct = DIRECT;
+    // When the waves of a workgroup share one kv head (token split) the transfers run TWO stages ahead: a stage is
+    // read into registers at the top of its arithmetic, so its buffer can take the stage after next while the
+    // arithmetic runs (measured: 8 x 32k..128k tokens on one kv head 55.2 -> 52.4 us; with a kv head per wave the
+    // deeper queue is slower, 148 -> 160 us on 64 x 32 kv heads, so those keep one stage ahead).
+    constexpr bool deep = !DIRECT;
     Segment cur, nxt;
     next_segment(cur);
     int slot0 = 0; // stage buffer of the current segment's stage 0
@@ -583,7 +595,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                 const int slot = (slot0 + it) & 1;
                 // the buffer the next stage lands in was last read by compute(it-1), which has finished in program order
                 if (it + 1 < cur.n_stages) {
-                    issue(cur, it + 1, slot ^ 1);
+                    if (!deep || it == 0) issue(cur, it + 1, slot ^ 1);
                     // everything older than the transfers just enqueued has landed: stage `it`, and at it == 0 the
                     // query loads. The previous segment's result stores were issued AFTER this segment's stage 0 (which
                     // was put in flight ahead of them), so they may stay in flight: waiting for their acknowledgement
@@ -638,7 +650,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 compute_stage(wave_lds_addr + slot * kStageBytes, ro, ss, qB, kq,
-                              it + 1 == cur.n_stages ? cur.tail_rows_valid : kStageTokens, p.score_scale);
+                              it + 1 == cur.n_stages ? cur.tail_rows_valid : kStageTokens, p.score_scale, [&]() {
+                                  if (deep && it + 2 < cur.n_stages) issue(cur, it + 2, slot);
+                              });
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -771,28 +785,36 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
     float mx = -INFINITY, l = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
     // four slots per step, their loads issued together: a long sequence has dozens of slots per lane group, and one
-    // memory latency per slot would add up (slots past the end repeat the last one with weight 0)
-    for (int64_t s = s_lo + g; s <= s_hi; s += 4 * kMergeGroups) {
+    // memory latency per slot would add up; what is left after the full steps goes one slot at a time
+    int64_t s = s_lo + g;
+    for (; s + 3 * kMergeGroups <= s_hi; s += 4 * kMergeGroups) {
         float mc[4], lc[4];
         float4_t a[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int64_t su = s + u * kMergeGroups;
-            const int64_t prow = ((su <= s_hi ? su : s_hi) + b) * p.num_heads + head;
+            const int64_t prow = (s + u * kMergeGroups + b) * p.num_heads + head;
             mc[u] = p.part_ml[prow * 2];
             lc[u] = p.part_ml[prow * 2 + 1];
             a[u] = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
-            if (su > s_hi) mc[u] = -INFINITY;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const float m_new = fmaxf(mx, mc[u]);
-            // (mx = m_new = -inf can only happen for padding slots in front of a real one: never, the first is real)
             const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc[u] - m_new);
             acc = acc * w_old + a[u] * w_new;
             l = l * w_old + lc[u] * w_new;
             mx = m_new;
         }
+    }
+    for (; s <= s_hi; s += kMergeGroups) {
+        const int64_t prow = (s + b) * p.num_heads + head;
+        const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
+        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
+        const float m_new = fmaxf(mx, mc);
+        const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc - m_new);
+        acc = acc * w_old + a * w_new;
+        l = l * w_old + lc * w_new;
+        mx = m_new;
     }
     red[g][d4 + 0] = acc[0];
     red[g][d4 + 1] = acc[1];
@@ -881,10 +903,14 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
         PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: no current device");
     if (!(lds_opted_in.load(std::memory_order_relaxed) >> dev & 1)) {
-        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true>)}) {
+        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, false, true>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true, true>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false, true>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true, true>)}) {
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
             if (e != hipSuccess)
                 PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
@@ -894,14 +920,23 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     }
     const bool fused = decode_writes_new_tokens(nd, p.num_ranges);
     const dim3 grid((unsigned)blocks), block(kDecodeWaves * kWave);
+    const bool direct = p.hpb == kDecodeWaves;
+#define PPLHIP_LAUNCH_DECODE(PAGED, FUSED)                                                                          \
+    do {                                                                                                            \
+        if (direct)                                                                                                 \
+            hipLaunchKernelGGL((decode_int8kv_kernel<PAGED, FUSED, true>), grid, block, lds_bytes, stream, p);      \
+        else                                                                                                        \
+            hipLaunchKernelGGL((decode_int8kv_kernel<PAGED, FUSED, false>), grid, block, lds_bytes, stream, p);     \
+    } while (0)
     if (p.page_shift && fused)
-        hipLaunchKernelGGL((decode_int8kv_kernel<true, true>), grid, block, lds_bytes, stream, p);
+        PPLHIP_LAUNCH_DECODE(true, true);
     else if (p.page_shift)
-        hipLaunchKernelGGL((decode_int8kv_kernel<true, false>), grid, block, lds_bytes, stream, p);
+        PPLHIP_LAUNCH_DECODE(true, false);
     else if (fused)
-        hipLaunchKernelGGL((decode_int8kv_kernel<false, true>), grid, block, lds_bytes, stream, p);
+        PPLHIP_LAUNCH_DECODE(false, true);
     else
-        hipLaunchKernelGGL((decode_int8kv_kernel<false, false>), grid, block, lds_bytes, stream, p);
+        PPLHIP_LAUNCH_DECODE(false, false);
+#undef PPLHIP_LAUNCH_DECODE
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
     // the sequences that need merging are those that straddle a range boundary: at most num_ranges - 1 of them,
     // however many sequences there are (2048 short sequences launched 65k workgroups that all left at once: 35 us)
