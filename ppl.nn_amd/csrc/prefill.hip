@@ -60,6 +60,7 @@ struct PrefillParams {
     int64_t w_first_token, w_end_token; // packed new tokens [first, end)
     int32_t w_batch; // all sequences of the call (the sequence of a token is looked up in seqstarts)
     int32_t w_per_tok; // 4-group units per token: 2 * kv_heads * 4
+    int32_t attn_blocks; // workgroups [0, attn_blocks) map to query tiles; the ones behind them only write tokens
 };
 
 // A thread's share of a 64-token K/V tile: channels 8*col .. 8*col+7 (col = tid & 15) of the four consecutive tokens
@@ -570,12 +571,21 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef short short8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) short4_t* lds_short4_t;
 
+constexpr int kWriteUnits = 2; // units of four quantisation groups per thread of a write-only workgroup
 __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams p) {
     __shared__ __attribute__((aligned(1024))) char lds[4 * kDmaTile];
 
+    // Workgroups [0, attn_blocks) map to query tiles. The ones behind them quantise the prompt tokens into the slab
+    // and leave: they are dispatched last, into the slots that the launch's tail leaves idle. (Measured against the
+    // alternatives on 8 prompts of 64..1024 tokens: the same work as a share of every tile workgroup's prologue 67 us,
+    // behind the tiles 62 us; dealt evenly INTO the grid 70 us, because that shifts the tiles' workgroup -> XCD
+    // assignment and with it the L2 reuse of K/V among the query heads of a kv head.)
+    const uint32_t wblock = blockIdx.x - p.attn_blocks;
+    const bool is_wblock = blockIdx.x >= (unsigned)p.attn_blocks;
+    const uint32_t ablock = is_wblock ? 0 : blockIdx.x;
     const int per_tile = p.num_seqs * p.num_heads;
-    const int qt_rev = blockIdx.x / per_tile;
-    const int rem = blockIdx.x - qt_rev * per_tile;
+    const int qt_rev = ablock / per_tile;
+    const int rem = ablock - qt_rev * per_tile;
     const int b = p.first_seq + rem / p.num_heads;
     const int hl = rem % p.num_heads;
     const int kvh = hl % p.kv_heads;
@@ -586,53 +596,67 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     const int64_t kvlen = p.kvstarts[b + 1] - kv0;
     const int64_t sp = kvlen > L ? kvlen - L : 0;
     const int ntiles = (int)((L + kBM - 1) / kBM);
-    const int ntiles_max = gridDim.x / per_tile;
+    const int ntiles_max = p.attn_blocks / per_tile;
     const int qt = ntiles_max - 1 - qt_rev;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
-    // This launch's share of the prompt tokens' quantize-on-write: the units of four quantisation groups are dealt
-    // out over ALL threads of the grid (workgroups without a query tile do theirs and leave). A workgroup with a
-    // tile runs it between issuing its first transfers and waiting for them, where it would otherwise sit idle.
+    // A write-only workgroup's share of the prompt tokens' quantize-on-write: units of four quantisation groups,
+    // kWriteUnits per thread and pass.
     auto write_share = [&]() {
         if (p.w_cache == nullptr) return;
-        // (workgroup i takes units 256*i .. 256*i+255: the work sits in the leading workgroups, which all run in the
-        // first round, when every workgroup of the launch is waiting for its first loads and the vector ALUs have
-        // nothing else to do; spreading it evenly over the grid measured 3 us slower)
         const int64_t units = (p.w_end_token - p.w_first_token) * p.w_per_tok;
-        for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.x * 256) {
-            const int64_t t = p.w_first_token + u / p.w_per_tok;
-            const int r = (int)(u % p.w_per_tok);
-            const int hi = r >> 2, grp = (r & 3) * 4; // K heads then V heads; first of the unit's four groups
-            const int kv = hi >= p.kv_heads, wh = hi - kv * p.kv_heads;
-            const uint4* src = reinterpret_cast<const uint4*>((kv ? p.v : p.k) + ((t * p.kv_heads + wh) * 16 + grp) * 8);
-            uint4 raw[4];
+        // kWriteUnits units per thread per pass, their 64-byte loads all issued before the first is used
+        for (int64_t u0 = (int64_t)wblock * (256 * kWriteUnits) + threadIdx.x; u0 < units;
+             u0 += (int64_t)(gridDim.x - p.attn_blocks) * (256 * kWriteUnits)) {
+            uint4 raw[kWriteUnits][4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) raw[i] = src[i];
-            const int64_t t0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(t >> 32)) << 32) |
-                               (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
-            const int wb = __all(t == t0) ? find_sequence_wave(p.seqstarts, p.w_batch, t0)
-                                          : find_sequence(p.seqstarts, p.w_batch, t);
-            const int64_t tok = p.pages.token(wb, p.start_pos[wb] + (t - p.seqstarts[wb]));
-            uint2 q[4];
-            half_t sc[4];
+            for (int k = 0; k < kWriteUnits; ++k) {
+                int64_t u = u0 + 256 * k;
+                if (u >= units) u = units - 1; // loaded twice, written once
+                const int64_t t = p.w_first_token + u / p.w_per_tok;
+                const int r = (int)(u % p.w_per_tok);
+                const int hi = r >> 2, grp = (r & 3) * 4; // K heads then V heads; first of the unit's four groups
+                const int kv = hi >= p.kv_heads, wh = hi - kv * p.kv_heads;
+                const uint4* src =
+                    reinterpret_cast<const uint4*>((kv ? p.v : p.k) + ((t * p.kv_heads + wh) * 16 + grp) * 8);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) quantize_group8(raw[i], &q[i], &sc[i]);
-            const int64_t row = p.addr.row(tok, kv, wh);
-            uint4* dst = reinterpret_cast<uint4*>(p.w_cache + row + grp * 8);
-            dst[0] = make_uint4(q[0].x, q[0].y, q[1].x, q[1].y);
-            dst[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
-            uint32_t packed[2];
-            __builtin_memcpy(packed, sc, 8);
-            uint32_t* sdst = reinterpret_cast<uint32_t*>(p.w_scale + row / kQuantGroup + grp);
-            sdst[0] = packed[0];
-            sdst[1] = packed[1];
+                for (int i = 0; i < 4; ++i) raw[k][i] = src[i];
+            }
+#pragma unroll
+            for (int k = 0; k < kWriteUnits; ++k) {
+                const int64_t u = u0 + 256 * k;
+                if (u >= units) break;
+                const int64_t t = p.w_first_token + u / p.w_per_tok;
+                const int r = (int)(u % p.w_per_tok);
+                const int hi = r >> 2, grp = (r & 3) * 4;
+                const int kv = hi >= p.kv_heads, wh = hi - kv * p.kv_heads;
+                const int64_t t0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(t >> 32)) << 32) |
+                                   (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+                const int wb = __all(t == t0) ? find_sequence_wave(p.seqstarts, p.w_batch, t0)
+                                              : find_sequence(p.seqstarts, p.w_batch, t);
+                const int64_t tok = p.pages.token(wb, p.start_pos[wb] + (t - p.seqstarts[wb]));
+                uint2 q[4];
+                half_t sc[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) quantize_group8(raw[k][i], &q[i], &sc[i]);
+                const int64_t row = p.addr.row(tok, kv, wh);
+                uint4* dst = reinterpret_cast<uint4*>(p.w_cache + row + grp * 8);
+                dst[0] = make_uint4(q[0].x, q[0].y, q[1].x, q[1].y);
+                dst[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
+                uint32_t packed[2];
+                __builtin_memcpy(packed, sc, 8);
+                uint32_t* sdst = reinterpret_cast<uint32_t*>(p.w_scale + row / kQuantGroup + grp);
+                sdst[0] = packed[0];
+                sdst[1] = packed[1];
+            }
         }
     };
-    if (qt >= ntiles) {
+    if (is_wblock) {
         write_share();
         return;
     }
+    if (qt >= ntiles) return;
     const int64_t q0 = (int64_t)qt * kBM;
 
     const int n = lane & 31;
@@ -738,7 +762,6 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
         return a;
     };
 
-    write_share();
     // tile 0 and the queries have to be there before the first MFMA (see prefill_attention_kernel for why the wait
     // is explicit)
     __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -973,8 +996,14 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
         p.w_batch = (int32_t)a->batch;
         p.w_per_tok = 2 * a->num_kv_heads * 4;
     }
-    const int64_t blocks = (int64_t)plan->prefill_num_q_tiles * npre * a->num_heads;
+    int64_t blocks = (int64_t)plan->prefill_num_q_tiles * npre * a->num_heads;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many query tiles in one call");
+    p.attn_blocks = (int32_t)blocks;
+    if (p.w_cache != nullptr && !a->enable_cache_prefill) {
+        const int64_t units = (p.w_end_token - p.w_first_token) * p.w_per_tok;
+        blocks += (units + 256 * kWriteUnits - 1) / (256 * kWriteUnits);
+        if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many tokens in one call");
+    }
     const dim3 grid((unsigned)blocks);
     if (a->enable_cache_prefill)
         hipLaunchKernelGGL(prefill_attention_kernel<true>, grid, dim3(256), 0, stream, p);
@@ -1012,6 +1041,7 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
     const int64_t q_tiles = (a->max_seqlen + kBM - 1) / kBM;
     const int64_t blocks = q_tiles * a->batch * a->num_heads;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many query tiles in one call");
+    p.attn_blocks = (int32_t)blocks;
     hipLaunchKernelGGL(prefill_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("multi_head_attention");
     return PPLHIP_RC_SUCCESS;
