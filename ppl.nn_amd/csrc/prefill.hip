@@ -61,6 +61,8 @@ struct PrefillParams {
     int32_t w_batch; // all sequences of the call (the sequence of a token is looked up in seqstarts)
     int32_t w_per_tok; // 4-group units per token: 2 * kv_heads * 4
     int32_t attn_blocks; // workgroups [0, attn_blocks) map to query tiles; the ones behind them only write tokens
+    int32_t ntiles_max; // query tiles of the longest sequence allowed (from max_seqlen)
+    int32_t compact; // the grid has one workgroup per possible tile instead of per (level, sequence): see the kernel
 };
 
 // A thread's share of a 64-token K/V tile: channels 8*col .. 8*col+7 (col = tid & 15) of the four consecutive tokens
@@ -571,6 +573,8 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef short short8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) short4_t* lds_short4_t;
 
+// the compact tile grid pays a search per workgroup: worth it from about 6 us of empty dispatches on
+constexpr int64_t kCompactMinEmpty = 8192;
 constexpr int kWriteUnits = 2; // units of four quantisation groups per thread of a write-only workgroup
 __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams p) {
     __shared__ __attribute__((aligned(1024))) char lds[4 * kDmaTile];
@@ -583,11 +587,100 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     const uint32_t wblock = blockIdx.x - p.attn_blocks;
     const bool is_wblock = blockIdx.x >= (unsigned)p.attn_blocks;
     const uint32_t ablock = is_wblock ? 0 : blockIdx.x;
-    const int per_tile = p.num_seqs * p.num_heads;
-    const int qt_rev = ablock / per_tile;
-    const int rem = ablock - qt_rev * per_tile;
-    const int b = p.first_seq + rem / p.num_heads;
-    const int hl = rem % p.num_heads;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int b, hl, qt;
+    if (!p.compact || is_wblock) {
+        // dense grid: (tile level, sequence, head); a sequence shorter than the longest has no tile at the top levels
+        const int per_tile = p.num_seqs * p.num_heads;
+        const int qt_rev = ablock / per_tile;
+        const int rem = ablock - qt_rev * per_tile;
+        b = p.first_seq + rem / p.num_heads;
+        hl = rem % p.num_heads;
+        qt = p.ntiles_max - 1 - qt_rev;
+    } else {
+        // Compact grid, for batches whose lengths differ so much that most (level, sequence) pairs are empty (one
+        // long prompt among many short ones: every empty workgroup still costs its dispatch, 0.75 us per thousand):
+        // the grid only has as many workgroups as there can be tiles, and workgroup -> tile is found here. Same order as
+        // the dense grid -- levels from the top, sequences by index within a level -- with the empty pairs left out.
+        const int rank = ablock / p.num_heads;
+        hl = ablock - rank * p.num_heads;
+        constexpr int kRegPasses = 4; // tile counts of the first 256 sequences stay in registers
+        int nreg[kRegPasses];
+#pragma unroll
+        for (int k = 0; k < kRegPasses; ++k) {
+            const int i = 64 * k + lane;
+            nreg[k] = i < p.num_seqs
+                          ? (int)((p.seqstarts[p.first_seq + i + 1] - p.seqstarts[p.first_seq + i] + kBM - 1) / kBM)
+                          : 0;
+        }
+        auto tiles_of = [&](int i) {
+            return i < p.num_seqs
+                       ? (int)((p.seqstarts[p.first_seq + i + 1] - p.seqstarts[p.first_seq + i] + kBM - 1) / kBM)
+                       : 0;
+        };
+        // sum over the lanes of a small non-negative number, bit by bit with ballots (the scalar unit counts the set
+        // bits): a few instructions per bit instead of a cross-lane reduction
+        auto wave_sum = [&](int v, int bits) {
+            int total = 0;
+            for (int bit = 0; bit < bits; ++bit) total += __popcll(__ballot((v >> bit) & 1)) << bit;
+            return total;
+        };
+        const int passes = (p.num_seqs + 63) >> 6;
+        const int pbits = 32 - __builtin_clz((unsigned)passes); // a lane adds up one number per pass
+        const int nbits = 32 - __builtin_clz((unsigned)p.ntiles_max) + pbits;
+        // tiles above level q = sum over the sequences of max(0, tiles - 1 - q)
+        auto tiles_above = [&](int q) {
+            int v = 0;
+#pragma unroll
+            for (int k = 0; k < kRegPasses; ++k) v += nreg[k] - 1 - q > 0 ? nreg[k] - 1 - q : 0;
+            for (int base = 64 * kRegPasses; base < p.num_seqs; base += 64) {
+                const int n = tiles_of(base + lane);
+                v += n - 1 - q > 0 ? n - 1 - q : 0;
+            }
+            return wave_sum(v, nbits);
+        };
+        // the level of this workgroup's rank: the lowest q with (tiles above q) <= rank
+        int lo = 0, hi = p.ntiles_max - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (tiles_above(mid) <= rank)
+                hi = mid;
+            else
+                lo = mid + 1;
+        }
+        const int q = lo;
+        const int cum = tiles_above(q);
+        {
+            int r = 0; // sequences that have a tile at level q
+#pragma unroll
+            for (int k = 0; k < kRegPasses; ++k) r += nreg[k] > q;
+            for (int base = 64 * kRegPasses; base < p.num_seqs; base += 64) r += tiles_of(base + lane) > q;
+            if (rank - cum >= wave_sum(r, pbits)) return; // the grid is an upper bound: no tile left for this workgroup
+        }
+        int idx = rank - cum; // the idx-th sequence (by index) that reaches level q
+        int sel = -1;
+        for (int base = 0; base < p.num_seqs && sel < 0; base += 64) {
+            int n = 0;
+            if (base < 64 * kRegPasses) {
+#pragma unroll
+                for (int k = 0; k < kRegPasses; ++k)
+                    if (base == 64 * k) n = nreg[k];
+            } else {
+                n = tiles_of(base + lane);
+            }
+            const uint64_t reach = __ballot(n > q);
+            const int pc = __popcll(reach);
+            if (idx < pc) {
+                const bool mine = (n > q) && __popcll(reach & ((uint64_t(1) << lane) - 1)) == idx;
+                sel = base + (int)__builtin_ctzll(__ballot(mine));
+            } else {
+                idx -= pc;
+            }
+        }
+        b = p.first_seq + __builtin_amdgcn_readfirstlane(sel);
+        qt = __builtin_amdgcn_readfirstlane(q);
+    }
     const int kvh = hl % p.kv_heads;
     const int head = kvh * p.rep + hl / p.kv_heads;
     const int64_t s0 = p.seqstarts[b];
@@ -596,10 +689,6 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     const int64_t kvlen = p.kvstarts[b + 1] - kv0;
     const int64_t sp = kvlen > L ? kvlen - L : 0;
     const int ntiles = (int)((L + kBM - 1) / kBM);
-    const int ntiles_max = p.attn_blocks / per_tile;
-    const int qt = ntiles_max - 1 - qt_rev;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
     // A write-only workgroup's share of the prompt tokens' quantize-on-write: units of four quantisation groups,
     // kWriteUnits per thread and pass.
@@ -997,6 +1086,17 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
         p.w_per_tok = 2 * a->num_kv_heads * 4;
     }
     int64_t blocks = (int64_t)plan->prefill_num_q_tiles * npre * a->num_heads;
+    p.ntiles_max = plan->prefill_num_q_tiles;
+    p.compact = 0;
+    if (!a->enable_cache_prefill) {
+        // the prompts hold total_new_tokens - decoding_batches tokens: at most that many / kBM + one per sequence tiles
+        const int64_t prompt_tokens = a->total_new_tokens - a->decoding_batches;
+        const int64_t tile_bound = (prompt_tokens / kBM + npre) * a->num_heads;
+        if (blocks - tile_bound >= kCompactMinEmpty) {
+            blocks = tile_bound;
+            p.compact = 1;
+        }
+    }
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many query tiles in one call");
     p.attn_blocks = (int32_t)blocks;
     if (p.w_cache != nullptr && !a->enable_cache_prefill) {
@@ -1042,6 +1142,8 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
     const int64_t blocks = q_tiles * a->batch * a->num_heads;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many query tiles in one call");
     p.attn_blocks = (int32_t)blocks;
+    p.ntiles_max = (int32_t)q_tiles;
+    p.compact = 0; // (the token total that bounds the number of tiles is not among this op's arguments)
     hipLaunchKernelGGL(prefill_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("multi_head_attention");
     return PPLHIP_RC_SUCCESS;

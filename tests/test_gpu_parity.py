@@ -351,3 +351,20 @@ def test_more_decode_sequences_than_ranges(KVH):
     b = workloads.Batch(8, KVH, 128, [1] * 40, hist, 40, name="40 ragged short sequences")
     check(b, workloads.make_tensors(b, seed=23), plans=plans)
     assert plans[-1].decode_num_ranges <= 40
+
+
+def test_one_long_prompt_among_many_short_ones():
+    """Prompt lengths so uneven that the prefill launch switches to its compact tile grid (one workgroup per possible
+    tile, tile found by a search in the kernel): 100 short prompts around one of 1024 tokens (two passes of 64
+    sequences in the search), then 300 short ones around one of 700 (more sequences than the search keeps in registers),
+    with decode sequences in front."""
+    rng = np.random.default_rng(31)
+    lens = rng.integers(1, 41, 100).tolist()
+    lens.insert(37, 1024)
+    b = workloads.Batch(32, 8, 128, [1, 1, 1] + lens, [17, 200, 64] + [0] * 101, 3, name="1 long + 100 short prompts")
+    check(b, workloads.make_tensors(b, seed=32))
+    lens = rng.integers(1, 7, 300).tolist()
+    lens.insert(280, 700)
+    lens[5] = 129
+    b = workloads.Batch(32, 8, 128, lens, [0] * 301, 0, name="1 long + 300 short prompts")
+    check(b, workloads.make_tensors(b, seed=33))
