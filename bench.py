@@ -46,7 +46,7 @@ def parse():
 class DeviceBatch:
     """Device-resident tensors + argument block of one MHCA call; history is quantised by the library itself."""
 
-    def __init__(self, pkg, lib, b, seed, n_slabs, split_k=1):
+    def __init__(self, pkg, lib, b, seed, n_slabs, split_k=1, cache_prefill=0):
         import torch
         from ppl_nn_amd import cabi
         self.pkg, self.lib, self.b, self.cabi = pkg, lib, b, cabi
@@ -100,6 +100,7 @@ class DeviceBatch:
                 setattr(a, kk, vv)
             a.enable_decoding_sharemem_mhca = a.enable_decoding_infinity_mhca = a.enable_decoding_infinity_gqca = 1
             a.specify_decoding_attn_split_k = split_k
+            a.enable_cache_prefill = cache_prefill
             a.d_cache, a.d_scale, a.d_output = ptr(cache), ptr(scale), ptr(self.out)
             a.total_new_tokens = S
             self.args.append(a)
@@ -392,6 +393,18 @@ def main():
                                           "tflops": lfl / (l_ms * 1e-3) / 1e12, "ms": l_ms,
                                           "frac_of_fp16_mfma_peak": lfl / (l_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS}
         del ldb
+        torch.cuda.empty_cache()
+        # chunked prefill: every prompt brings a 512-token chunk on top of 4096 tokens already in the int8 slab
+        cb = workloads.Batch(32, 8, 128, _np.full(8, 512, _np.int64), _np.full(8, 4096, _np.int64), 0, name="chunked prefill")
+        cdb = DeviceBatch(pkg, lib, cb, seed=6, n_slabs=1, cache_prefill=1)
+        _, c_ms = timed(cdb, 10, 2)
+        cfl = cb.prefill_flops()
+        result["chunked_prefill"] = {"workload": "8 prompts x (4096 cached + 512 new tokens), H32/KVH8/Dh128, cache-prefill "
+                                                 "(quantize-on-write, fp16 staging of the cached K/V, attention)",
+                                     "tflops": cfl / (c_ms * 1e-3) / 1e12, "ms": c_ms,
+                                     "frac_of_fp16_mfma_peak": cfl / (c_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
+                                     "staged": int(cdb.plan.prefill_staging)}
+        del cdb
         torch.cuda.empty_cache()
     if args.copy_calibration:
         copy_calibration()

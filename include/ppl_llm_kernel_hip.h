@@ -119,7 +119,11 @@ typedef struct pplhip_mhca_plan {
     int32_t decode_waves_per_block;
     int32_t prefill_q_tile; /* query rows per prefill workgroup */
     int32_t prefill_num_q_tiles; /* ceil(max_seqlen / prefill_q_tile) */
-    int32_t reserved[3];
+    int32_t prefill_staging; /* cache-prefill only: 1 = the prompts' cached K/V are first dequantised into fp16 staging
+                                rows in the workspace (one streaming pass) and attention runs over those; 0 = the
+                                attention kernel dequantises the int8 slab itself (small chunks, or staging too large) */
+    int32_t prefill_staging_offset_256; /* where the staging rows start in the workspace, in units of 256 bytes */
+    int32_t reserved[1];
 } pplhip_mhca_plan;
 
 /* Host-only: validates `args` exactly like the reference wrapper + kernel library would

@@ -50,7 +50,8 @@ class MhcaPlan(C.Structure):
         ("workspace_bytes", C.c_uint64),
         ("decode_num_ranges", _i32), ("decode_heads_per_block", _i32), ("decode_waves_per_block", _i32),
         ("prefill_q_tile", _i32), ("prefill_num_q_tiles", _i32),
-        ("reserved", _i32 * 3),
+        ("prefill_staging", _i32), ("prefill_staging_offset_256", _i32),
+        ("reserved", _i32 * 1),
     ]
 
 

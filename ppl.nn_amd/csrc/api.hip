@@ -187,6 +187,12 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     if (a->batch > a->decoding_batches)
         plan->prefill_num_q_tiles = (int32_t)((a->max_seqlen + plan->prefill_q_tile - 1) / plan->prefill_q_tile);
     plan->workspace_bytes = (plan->workspace_bytes + 255) / 256 * 256;
+    if (const int64_t staged = prefill_staging_tokens(a)) {
+        plan->prefill_staging = 1;
+        plan->prefill_staging_offset_256 = (int32_t)(plan->workspace_bytes / 256);
+        plan->workspace_bytes += (uint64_t)staged * 2 * a->num_kv_heads * a->head_dim * sizeof(uint16_t);
+        plan->workspace_bytes = (plan->workspace_bytes + 255) / 256 * 256;
+    }
     return PPLHIP_RC_SUCCESS;
 }
 
@@ -211,7 +217,7 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     if (rc != PPLHIP_RC_SUCCESS) return rc;
     rc = launch_decode(a, plan, d_workspace, s);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
-    return launch_prefill(a, plan, s);
+    return launch_prefill(a, plan, d_workspace, s);
 }
 
 pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {

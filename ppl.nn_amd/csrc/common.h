@@ -127,13 +127,19 @@ inline int ceil_div(int64_t a, int64_t b) {
 pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token = 0,
                                         int64_t end_token = -1);
 pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream_t stream);
+// cache-prefill: dequantises the cached K/V of sequences [decoding_batches, batch) into packed fp16 rows
+// [kv token - kvstarts[decoding_batches], kv head, head_dim] at `key_out` / `value_out`; `max_tokens` bounds the rows
+pplhip_retcode launch_kv_stage_prefill(const pplhip_mhca_args* a, half_t* key_out, half_t* value_out, int64_t max_tokens,
+                                       hipStream_t stream);
+// whether (and where in the workspace) a cache-prefill call stages its K/V as fp16: see pplhip_mhca_plan
+int64_t prefill_staging_tokens(const pplhip_mhca_args* a);
 int decode_heads_per_block(int kv_heads);
 bool decode_writes_new_tokens(int64_t decoding_batches, int num_ranges);
 bool prefill_writes_new_tokens(const pplhip_mhca_args* a);
 int decode_blocks_per_cu();
 int decode_waves_per_block();
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
-pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, hipStream_t stream);
+pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
 pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream);
 pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream);
 pplhip_retcode launch_position_index(const int64_t* d_seqstarts, const int64_t* d_start_pos, int64_t batch,

@@ -60,6 +60,7 @@ struct PrefillParams {
     int64_t w_first_token, w_end_token; // packed new tokens [first, end)
     int32_t w_batch; // all sequences of the call (the sequence of a token is looked up in seqstarts)
     int32_t w_per_tok; // 4-group units per token: 2 * kv_heads * 4
+    const int64_t* kv_origin; // null, or the packed kv-token index that row 0 of k / v holds (device scalar)
     int32_t attn_blocks; // workgroups [0, attn_blocks) map to query tiles; the ones behind them only write tokens
     int32_t ntiles_max; // query tiles of the longest sequence allowed (from max_seqlen)
     int32_t compact; // the grid has one workgroup per possible tile instead of per (level, sequence): see the kernel
@@ -685,8 +686,9 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     const int head = kvh * p.rep + hl / p.kv_heads;
     const int64_t s0 = p.seqstarts[b];
     const int64_t L = p.seqstarts[b + 1] - s0;
-    const int64_t kv0 = p.kvstarts[b];
-    const int64_t kvlen = p.kvstarts[b + 1] - kv0;
+    const int64_t kv_first = p.kvstarts[b];
+    const int64_t kvlen = p.kvstarts[b + 1] - kv_first;
+    const int64_t kv0 = kv_first - (p.kv_origin ? *p.kv_origin : 0); // row of the sequence's first key in k / v
     const int64_t sp = kvlen > L ? kvlen - L : 0;
     const int ntiles = (int)((L + kBM - 1) / kBM);
 
@@ -1053,10 +1055,11 @@ bool prefill_writes_new_tokens(const pplhip_mhca_args* a) {
     return !a->enable_cache_prefill && a->batch > a->decoding_batches;
 }
 
-pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, hipStream_t stream) {
+pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
     const int npre = (int)(a->batch - a->decoding_batches);
     if (npre <= 0 || plan->prefill_num_q_tiles <= 0) return PPLHIP_RC_SUCCESS;
     PrefillParams p;
+    p.kv_origin = nullptr;
     p.q = (const half_t*)a->d_query;
     p.k = (const half_t*)a->d_current_key;
     p.v = (const half_t*)a->d_current_value;
@@ -1076,6 +1079,21 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     p.is_causal = a->is_causal;
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
     p.num_seqs = npre;
+    // cache-prefill over staged fp16 rows: the slab rows of the prompts (the new tokens are in there by now) are
+    // dequantised in one streaming pass, and attention reads those like it reads current_key / current_value
+    const bool staged = a->enable_cache_prefill && plan->prefill_staging;
+    if (staged) {
+        const int64_t tokens = prefill_staging_tokens(a);
+        if (tokens == 0 || ws == nullptr)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "prefill: plan was not produced by pplhip_mhca_prepare for these arguments");
+        half_t* k_stage = (half_t*)((char*)ws + (uint64_t)plan->prefill_staging_offset_256 * 256);
+        half_t* v_stage = k_stage + tokens * a->num_kv_heads * a->head_dim;
+        pplhip_retcode rc = launch_kv_stage_prefill(a, k_stage, v_stage, tokens, stream);
+        if (rc != PPLHIP_RC_SUCCESS) return rc;
+        p.k = k_stage;
+        p.v = v_stage;
+        p.kv_origin = a->d_kvstarts + a->decoding_batches; // staging row 0 = the first prompt's first cached token
+    }
     p.w_cache = nullptr;
     if (prefill_writes_new_tokens(a)) {
         p.w_cache = (int8_t*)a->d_cache;
@@ -1088,7 +1106,7 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     int64_t blocks = (int64_t)plan->prefill_num_q_tiles * npre * a->num_heads;
     p.ntiles_max = plan->prefill_num_q_tiles;
     p.compact = 0;
-    if (!a->enable_cache_prefill) {
+    if (!a->enable_cache_prefill || staged) {
         // the prompts hold total_new_tokens - decoding_batches tokens: at most that many / kBM + one per sequence tiles
         const int64_t prompt_tokens = a->total_new_tokens - a->decoding_batches;
         const int64_t tile_bound = (prompt_tokens / kBM + npre) * a->num_heads;
@@ -1099,13 +1117,13 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     }
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many query tiles in one call");
     p.attn_blocks = (int32_t)blocks;
-    if (p.w_cache != nullptr && !a->enable_cache_prefill) {
+    if (p.w_cache != nullptr) {
         const int64_t units = (p.w_end_token - p.w_first_token) * p.w_per_tok;
         blocks += (units + 256 * kWriteUnits - 1) / (256 * kWriteUnits);
         if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many tokens in one call");
     }
     const dim3 grid((unsigned)blocks);
-    if (a->enable_cache_prefill)
+    if (a->enable_cache_prefill && !staged)
         hipLaunchKernelGGL(prefill_attention_kernel<true>, grid, dim3(256), 0, stream, p);
     else
         hipLaunchKernelGGL(prefill_f16_kernel, grid, dim3(256), 0, stream, p);
@@ -1136,6 +1154,7 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream) {
     p.is_causal = a->is_causal;
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
     p.num_seqs = (int32_t)a->batch;
+    p.kv_origin = nullptr;
     p.w_cache = nullptr; // MultiHeadAttention has no cache to write
     p.w_scale = nullptr;
     const int64_t q_tiles = (a->max_seqlen + kBM - 1) / kBM;

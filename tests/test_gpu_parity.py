@@ -368,3 +368,33 @@ def test_one_long_prompt_among_many_short_ones():
     lens[5] = 129
     b = workloads.Batch(32, 8, 128, lens, [0] * 301, 0, name="1 long + 300 short prompts")
     check(b, workloads.make_tensors(b, seed=33))
+
+
+def test_cache_prefill_over_staged_rows():
+    """Chunks large enough that the plan stages the prompts' cached K/V as fp16 rows (one dequantisation pass) and
+    runs attention over those: contiguous slab, paged slab, cache_layout 3, with decode sequences in front; the three
+    must agree bit for bit with each other and match the oracle."""
+    b = workloads.Batch(8, 2, 128, [1, 1, 300, 700, 260, 5], [77, 1500, 100, 0, 513, 31], 2, num_layer=2, layer_idx=1,
+                        name="staged_cache_prefill")
+    t = workloads.make_tensors(b, seed=61)
+    plans = []
+    _, ref, flat = check(b, t, cache_prefill=1, plans=plans)
+    assert plans[-1].prefill_staging == 1
+    paged = harness.PagedLayout(b, page_size=128, seed=5)
+    got = harness.run_device(b, t, cache_prefill=1, paged=paged)
+    assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
+    lay3 = harness.run_device(b, t, cache_prefill=1, layout=3)
+    assert np.array_equal(lay3["output"].view(np.uint16), flat["output"].view(np.uint16))
+    # small chunks keep the kernel that dequantises the slab itself
+    b = workloads.Batch(8, 2, 128, [1, 20, 130, 7], [12, 30, 100, 0], 1, name="small_chunks")
+    plans = []
+    check(b, workloads.make_tensors(b, seed=62), cache_prefill=1, plans=plans)
+    assert plans[-1].prefill_staging == 0
+    # uneven chunks: staged rows and the compact tile grid together
+    rng = np.random.default_rng(63)
+    lens = [1024] + rng.integers(200, 300, 40).tolist()
+    hist = [256] + rng.integers(0, 50, 40).tolist()
+    b = workloads.Batch(32, 8, 128, lens, hist, 0, name="staged_uneven_chunks")
+    plans = []
+    check(b, workloads.make_tensors(b, seed=64), cache_prefill=1, plans=plans)
+    assert plans[-1].prefill_staging == 1
