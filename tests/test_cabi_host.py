@@ -112,6 +112,34 @@ def test_decode_plan_fills_one_round_of_workgroup_slots(hiplib, kvh):
     assert (plan.decode_num_ranges + 8) * groups > 512  # and no more than one step of 8 below it
 
 
+def test_cache_prefill_plan_stages_large_chunks_only(hiplib):
+    """Cache-prefill: chunks of >= 1024 / (query heads per kv head) new tokens per prompt on average make the plan stage
+    the prompts' cached K/V as fp16 rows behind the decode part of the workspace (worst case: every prompt max_kvlen
+    long); small chunks, more than 1 GiB of staging rows, or no cache-prefill leave the workspace as it was."""
+    fake = lambda t: C.c_void_p(0x1000)
+
+    def plan_of(seqlens, hist, nd, cache_prefill):
+        b = workloads.Batch(32, 8, 128, seqlens, hist, nd)
+        a = cabi.MhcaArgs()
+        harness.fill_mhca_args(a, b, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, ptr=fake, split_k=1, cache_prefill=cache_prefill)
+        plan = cabi.MhcaPlan()
+        assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+        return b, plan
+
+    b, base = plan_of([1, 1, 512, 300], [100, 900, 4096, 0], 2, 0)
+    assert base.prefill_staging == 0
+    b, staged = plan_of([1, 1, 512, 300], [100, 900, 4096, 0], 2, 1)
+    assert staged.prefill_staging == 1
+    assert staged.prefill_staging_offset_256 * 256 == base.workspace_bytes
+    rows = 2 * b.max_kvlen  # two prompts
+    assert staged.workspace_bytes == base.workspace_bytes + rows * 2 * 8 * 128 * 2
+    _, small = plan_of([1, 1, 100, 200], [100, 900, 4096, 0], 2, 1)  # 150 new tokens per prompt on average x 4 < 1024
+    _, small0 = plan_of([1, 1, 100, 200], [100, 900, 4096, 0], 2, 0)
+    assert small.prefill_staging == 0 and small.workspace_bytes == small0.workspace_bytes
+    _, huge = plan_of([1, 1, 512, 300] + [300] * 30, [100, 900, 16384, 0] + [0] * 30, 2, 1)  # 32 x 16896 rows x 4 KB > 1 GiB
+    assert huge.prefill_staging == 0
+
+
 def test_prepare_accepts_paged_cache(hiplib):
     a, plan = _valid_args(), cabi.MhcaPlan()
     a.cache_mode, a.cachestart_stride_b, a.page_size = 1, 4, 128
