@@ -83,7 +83,17 @@ struct DecodeParams {
     float score_scale; // log2(e) / sqrt(Dh)
 };
 
-// Tokens per range: the total is only known on the device. At least 128 so that tiny batches are not shredded.
+// Every sequence boundary inside a range costs the range's workgroup about one stage more (the sequence before the
+// boundary ends with a partly filled stage, the one behind it starts a new one), and the launch lasts as long as the
+// range with the most boundaries. The ranges are therefore cut on a virtual axis on which every sequence is followed by
+// kBoundaryTokens positions that hold no token: sequence i starts at kvstarts[i] + i * kBoundaryTokens. Equal virtual
+// ranges give a range with many boundaries fewer tokens.
+#ifndef PPLHIP_BOUNDARY_TOKENS
+#define PPLHIP_BOUNDARY_TOKENS 32
+#endif
+constexpr int kBoundaryTokens = PPLHIP_BOUNDARY_TOKENS;
+
+// Positions per range: the total is only known on the device. At least 128 so that tiny batches are not shredded.
 __device__ inline int64_t range_tokens(int64_t total, int num_ranges) {
     int64_t r = (total + num_ranges - 1) / num_ranges;
     r = (r + 31) & ~(int64_t)31;
@@ -422,7 +432,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     const int64_t j = blockIdx.x >> 3;
     const int hg = (int)(j % groups);
     const int64_t s_idx = (j / groups) * 8 + xcd; // range index
-    const int64_t total = p.kvstarts[p.nd];
+    // (virtual positions: see kBoundaryTokens)
+    const int64_t total = p.kvstarts[p.nd] + (int64_t)p.nd * kBoundaryTokens;
     const int64_t R = range_tokens(total, p.num_ranges);
     const int64_t r0 = s_idx * R;
     if (r0 >= total) return;
@@ -455,11 +466,19 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     int b = 0;
     for (int base = 0; base < p.nd; base += kWave) {
         const int i = base + lane;
-        const bool ends_before = i < p.nd && p.kvstarts[i + 1] <= r0;
+        const bool ends_before = i < p.nd && p.kvstarts[i + 1] + (int64_t)(i + 1) * kBoundaryTokens <= r0;
         b += __builtin_popcountll(__ballot(ends_before));
     }
     b = __builtin_amdgcn_readfirstlane(b);
     if (hg == 0 && threadIdx.x == 0) p.range_first[s_idx] = b; // saves the merge kernel the same search
+    int64_t pos = r0;
+    if (r0 - (p.kvstarts[b] + (int64_t)b * kBoundaryTokens) >= p.kvstarts[b + 1] - p.kvstarts[b]) {
+        // the range starts in the empty positions behind sequence b: its first token is the next sequence's first
+        ++b;
+        if (b >= p.nd) return;
+        pos = p.kvstarts[b] + (int64_t)b * kBoundaryTokens;
+        if (pos >= r1) return;
+    }
 
     // A segment = the part of one sequence inside this range; this wave's share of it is tokens [t_begin, t_end).
     struct Segment {
@@ -474,12 +493,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         bool has_new;
     };
     const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
-    int64_t pos = r0;
-    auto next_segment = [&](Segment& g) { // consumes sequence b from position pos on
+    auto next_segment = [&](Segment& g) { // consumes sequence b from (virtual) position pos on
         const int64_t seq_lo = p.kvstarts[b], seq_hi = p.kvstarts[b + 1];
-        const int64_t seg_begin = pos - seq_lo;
+        const int64_t vlo = seq_lo + (int64_t)b * kBoundaryTokens; // virtual position of the sequence's first token
+        const int64_t seg_begin = pos - vlo; // < the sequence's length
         g.b = b;
-        g.seg_end = (int32_t)(((r1 < seq_hi) ? r1 : seq_hi) - seq_lo);
+        g.seg_end = (int32_t)((r1 - vlo < seq_hi - seq_lo) ? r1 - vlo : seq_hi - seq_lo);
         g.whole_sequence = seg_begin == 0 && g.seg_end == seq_hi - seq_lo;
         g.page_row = PAGED ? p.cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
         g.qrow = (int32_t)p.seqstarts[b];
@@ -498,7 +517,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         g.has_new = FUSED_WRITE && g.n_stages > 0 && t_end == seq_hi - seq_lo;
         const int64_t row0 = (PAGED ? 0 : (p.cachestarts[b] + (int64_t)g.t_begin) * (int64_t)stride) + head_off;
         g.cbase = reinterpret_cast<const char*>(p.cache) + row0;
-        pos = seq_lo + g.seg_end;
+        // where the range goes on: inside this sequence (then pos = r1), or at the next sequence's first token
+        pos = vlo + g.seg_end + (g.seg_end == seq_hi - seq_lo ? kBoundaryTokens : 0);
         ++b;
     };
     // enqueues stage idx of segment g into stage buffer `slot`
@@ -768,19 +788,22 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
     const int head = blockIdx.x;
     const int g = threadIdx.x >> 5;
     const int d4 = (threadIdx.x & 31) * 4;
-    const int64_t R = range_tokens(p.kvstarts[p.nd], p.num_ranges);
+    const int64_t total = p.kvstarts[p.nd] + (int64_t)p.nd * kBoundaryTokens; // virtual positions, as in the decode kernel
+    const int64_t R = range_tokens(total, p.num_ranges);
     // blockIdx.y is a sequence, or (when there are more sequences than ranges) a boundary between two ranges: only
     // a sequence that straddles a boundary has anything to merge, and it is handled by the first boundary it crosses
     int b;
     if (p.merge_by_boundary) {
         const int64_t edge = ((int64_t)blockIdx.y + 1) * R; // first token of range blockIdx.y + 1
-        if (edge >= p.kvstarts[p.nd]) return;
-        b = p.range_first[blockIdx.y + 1]; // the sequence that holds token `edge` (found by the decode kernel)
-        if (p.kvstarts[b] >= edge || p.kvstarts[b] / R != blockIdx.y) return; // starts there, or crossed one before
+        if (edge >= total) return;
+        b = p.range_first[blockIdx.y + 1]; // the sequence that holds position `edge` (found by the decode kernel)
+        const int64_t vb = p.kvstarts[b] + (int64_t)b * kBoundaryTokens;
+        if (vb >= edge || vb / R != blockIdx.y) return; // starts there, or crossed a boundary before this one
     } else {
         b = blockIdx.y;
     }
-    const int64_t s_lo = p.kvstarts[b] / R, s_hi = (p.kvstarts[b + 1] - 1) / R;
+    const int64_t vlo = p.kvstarts[b] + (int64_t)b * kBoundaryTokens;
+    const int64_t s_lo = vlo / R, s_hi = (vlo + (p.kvstarts[b + 1] - p.kvstarts[b]) - 1) / R;
     if (s_lo == s_hi) return;
     float mx = -INFINITY, l = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
