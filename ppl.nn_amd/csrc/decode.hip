@@ -39,6 +39,7 @@
 // consecutive (range, sequence) segments get consecutive slots -- and `decode_merge_kernel` combines the slots of a
 // sequence with the usual log-sum-exp weights.
 #include <atomic>
+#include <type_traits>
 #include "common.h"
 
 namespace pplhip {
@@ -100,6 +101,11 @@ __device__ inline int64_t range_tokens(int64_t total, int num_ranges) {
     return r < 128 ? 128 : r;
 }
 
+// The sequence tables are read through the constant address space: a wave-uniform read from there is always a scalar
+// load. Through a plain global pointer the compiler only uses scalar loads while the kernel has not stored anything;
+// after the first result store the look-ups of the next sequence became vector loads, whose result is only there
+// once every transfer in flight has landed (one counter, in order): each sequence boundary drained the pipeline.
+typedef const int64_t __attribute__((address_space(4)))* const_tab_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
@@ -202,19 +208,31 @@ __device__ inline void lds_write_b16(uint32_t addr, uint32_t v) {
 
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at "no wait"), gfx9 encoding
 #define PPLHIP_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | 0x0f70)
-// the same with `extra` (0, 2, 4, 6, 10 or 12: the result stores of the previous segment) younger operations more left
-// in flight; the immediate has to be a constant
-#define PPLHIP_WAIT_VMCNT_PLUS(n, extra)              \
-    do {                                              \
-        switch (extra) {                              \
-            case 2: PPLHIP_WAIT_VMCNT((n) + 2); break;   \
-            case 4: PPLHIP_WAIT_VMCNT((n) + 4); break;   \
-            case 6: PPLHIP_WAIT_VMCNT((n) + 6); break;   \
-            case 10: PPLHIP_WAIT_VMCNT((n) + 10); break; \
-            case 12: PPLHIP_WAIT_VMCNT((n) + 12); break; \
-            default: PPLHIP_WAIT_VMCNT(n); break;        \
-        }                                             \
+// the same with `extra` (0, 4 or 8: result stores of the previous segment) younger operations more left in flight; the
+// immediate has to be a constant
+#define PPLHIP_WAIT_VMCNT_PLUS(n, extra)            \
+    do {                                            \
+        switch (extra) {                            \
+            case 4: PPLHIP_WAIT_VMCNT((n) + 4); break; \
+            case 8: PPLHIP_WAIT_VMCNT((n) + 8); break; \
+            default: PPLHIP_WAIT_VMCNT(n); break;      \
+        }                                           \
     } while (0)
+// A 16-byte global load the compiler does not track: its waitcnt pass merges what it knows about loads in flight at
+// every loop header, and for the query registers (loaded once per sequence, read by every stage) that put a
+// vmcnt(0) in front of the first MFMA of EVERY stage and another in front of every stage's transfers -- the wave never
+// computed while one of its own transfers was in flight. The waits for these loads are the explicit ones in the
+// stage loop (they are older than the stage they are used with) and the one in front of the hand-over to the next
+// segment. The destination must be the variable the value lives in until such a wait: a copy made earlier would copy
+// registers the data has not reached.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+// and must not be carried around a loop before that wait (the copies of a loop-carried value are made at once).
+__device__ inline void load16_untracked(half8_t& dst, const void* ptr) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+}
+__device__ inline void load16_untracked(u32x4_t& dst, const void* ptr) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+}
 constexpr int kDmaPerStage = 2 * (kStageTokens / 8) + 2; // 4 K + 4 V + K scales + V scales
 
 // Per-lane source offsets of the stage DMA (relative to the wave-uniform stage base).
@@ -433,7 +451,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     const int hg = (int)(j % groups);
     const int64_t s_idx = (j / groups) * 8 + xcd; // range index
     // (virtual positions: see kBoundaryTokens)
-    const int64_t total = p.kvstarts[p.nd] + (int64_t)p.nd * kBoundaryTokens;
+    const const_tab_t kvstarts = (const_tab_t)p.kvstarts, seqstarts = (const_tab_t)p.seqstarts,
+                      cachestarts = (const_tab_t)p.cachestarts;
+    const int64_t total = kvstarts[p.nd] + (int64_t)p.nd * kBoundaryTokens;
     const int64_t R = range_tokens(total, p.num_ranges);
     const int64_t r0 = s_idx * R;
     if (r0 >= total) return;
@@ -472,11 +492,11 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     b = __builtin_amdgcn_readfirstlane(b);
     if (hg == 0 && threadIdx.x == 0) p.range_first[s_idx] = b; // saves the merge kernel the same search
     int64_t pos = r0;
-    if (r0 - (p.kvstarts[b] + (int64_t)b * kBoundaryTokens) >= p.kvstarts[b + 1] - p.kvstarts[b]) {
+    if (r0 - (kvstarts[b] + (int64_t)b * kBoundaryTokens) >= kvstarts[b + 1] - kvstarts[b]) {
         // the range starts in the empty positions behind sequence b: its first token is the next sequence's first
         ++b;
         if (b >= p.nd) return;
-        pos = p.kvstarts[b] + (int64_t)b * kBoundaryTokens;
+        pos = kvstarts[b] + (int64_t)b * kBoundaryTokens;
         if (pos >= r1) return;
     }
 
@@ -485,7 +505,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         int b;
         int32_t seg_end, qrow, t_begin; // positions inside a sequence and packed token rows fit 32 bits
         bool whole_sequence;
-        const int64_t* page_row; // paged slab: the sequence's row of the page table
+        const_tab_t page_row; // paged slab: the sequence's row of the page table
         const char* cbase; // contiguous slab: K row of token t_begin (this kv head) in the cache tensor
         int n_stages, tail_rows_mem, tail_rows_valid;
         // this wave's chunk ends with the sequence's NEW token (its last one), which the wave quantises into the slab
@@ -494,14 +514,14 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     };
     const int64_t head_off = p.addr.row(0, 0, kvh); // layer and kv head, K plane
     auto next_segment = [&](Segment& g) { // consumes sequence b from (virtual) position pos on
-        const int64_t seq_lo = p.kvstarts[b], seq_hi = p.kvstarts[b + 1];
+        const int64_t seq_lo = kvstarts[b], seq_hi = kvstarts[b + 1];
         const int64_t vlo = seq_lo + (int64_t)b * kBoundaryTokens; // virtual position of the sequence's first token
         const int64_t seg_begin = pos - vlo; // < the sequence's length
         g.b = b;
         g.seg_end = (int32_t)((r1 - vlo < seq_hi - seq_lo) ? r1 - vlo : seq_hi - seq_lo);
         g.whole_sequence = seg_begin == 0 && g.seg_end == seq_hi - seq_lo;
-        g.page_row = PAGED ? p.cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
-        g.qrow = (int32_t)p.seqstarts[b];
+        g.page_row = PAGED ? cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
+        g.qrow = (int32_t)seqstarts[b];
         int64_t sub = (g.seg_end - seg_begin + tsplits - 1) / tsplits;
         sub = (sub + kStageTokens - 1) / kStageTokens * kStageTokens;
         g.t_begin = (int32_t)(seg_begin + (int64_t)ts * sub);
@@ -515,7 +535,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         g.tail_rows_valid = (int)(t_end - last_stage_t0);
         const int64_t seq_len = seq_hi - seq_lo;
         g.has_new = FUSED_WRITE && g.n_stages > 0 && t_end == seq_hi - seq_lo;
-        const int64_t row0 = (PAGED ? 0 : (p.cachestarts[b] + (int64_t)g.t_begin) * (int64_t)stride) + head_off;
+        const int64_t row0 = (PAGED ? 0 : (cachestarts[b] + (int64_t)g.t_begin) * (int64_t)stride) + head_off;
         g.cbase = reinterpret_cast<const char*>(p.cache) + row0;
         // where the range goes on: inside this sequence (then pos = r1), or at the next sequence's first token
         pos = vlo + g.seg_end + (g.seg_end == seq_hi - seq_lo ? kBoundaryTokens : 0);
@@ -565,22 +585,27 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     // four query pieces (+ the lane's group of the sequence's new token)
     constexpr int kQueryLoads = FUSED_WRITE ? 5 : 4;
     // lanes 0..15: groups of the new token's K row (this kv head), lanes 16..31: of its V row (upper half-wave mirrors)
-    auto load_query = [&](const Segment& g, half8_t (&q)[2][2], uint4& newtok) {
+    // untracked: by load16_untracked, for the hand-over inside a range (the caller waits); otherwise by ordinary
+    // loads that are waited for on the spot (first segment of a range, token-split workgroups)
+    auto load_query = [&](const Segment& g, half8_t (&q)[2][2], u32x4_t& newtok, auto untracked) {
         if (FUSED_WRITE) {
             const half_t* src = ((lane & 16) ? p.cur_value : p.cur_key) +
                                 ((int64_t)g.qrow * p.kv_heads + kvh) * kDh + 8 * (lane & 15);
-            newtok = *reinterpret_cast<const uint4*>(src);
+            if (untracked) load16_untracked(newtok, src);
+            else newtok = *reinterpret_cast<const u32x4_t*>(src);
         }
-        const bool live = m < p.rep;
-        const half_t* qp = p.q + (((int64_t)g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (live ? m : 0)) * kDh;
+        // Columns m >= rep of the MFMA have no query head: they carry a copy of head 0 of the group, whose results
+        // are never stored.
+        const half_t* qp = p.q + (((int64_t)g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (m < p.rep ? m : 0)) * kDh;
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                uint4 x = *reinterpret_cast<const uint4*>(qp + 32 * kq + 16 * jj + 8 * i);
-                if (!live) x = make_uint4(0, 0, 0, 0);
-                __builtin_memcpy(&q[jj][i], &x, 16);
+                if (untracked) load16_untracked(q[jj][i], qp + 32 * kq + 16 * jj + 8 * i);
+                else q[jj][i] = *reinterpret_cast<const half8_t*>(qp + 32 * kq + 16 * jj + 8 * i);
             }
+        if (!untracked) // the wait for these loads happens HERE, not in front of every stage's first MFMA
+            asm volatile("" : "+v"(q[0][0]), "+v"(q[0][1]), "+v"(q[1][0]), "+v"(q[1][1]), "+v"(newtok));
     };
 
     // When every wave owns a whole kv head (no token split inside the workgroup) nothing is combined through LDS, the
@@ -598,9 +623,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     bool cur_in_flight = false; // stage 0 of `cur` already enqueued by the previous segment's last iteration
     // store instructions issued behind the stage-0 transfers of a segment that was put in flight early (see the waits)
     int pending_stores = 0;
-    half8_t qB[2][2], qN[2][2];
-    uint4 newB, newN;
-    load_query(cur, qB, newB);
+    half8_t qB[2][2];
+    u32x4_t newB = {0, 0, 0, 0};
+    load_query(cur, qB, newB, std::false_type{});
     for (;;) {
         SoftmaxState ss;
 #pragma unroll
@@ -609,32 +634,43 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         ss.l_part = 0.f;
 
         bool has_next = false;
+        half8_t qN[2][2];
+        u32x4_t newN = {0, 0, 0, 0};
         if (cur.n_stages > 0) {
             if (!cur_in_flight) issue(cur, 0, slot0);
-            for (int it = 0; it < cur.n_stages; ++it) {
+            const int last = cur.n_stages - 1;
+            // ---- every stage but the last. The buffer the next stage lands in was last read by the stage before this
+            // one, which has finished in program order.
+            for (int it = 0; it < last; ++it) {
                 const int slot = (slot0 + it) & 1;
-                // the buffer the next stage lands in was last read by compute(it-1), which has finished in program order
-                if (it + 1 < cur.n_stages) {
-                    if (!deep || it == 0) issue(cur, it + 1, slot ^ 1);
-                    // everything older than the transfers just enqueued has landed: stage `it`, and at it == 0 the
-                    // query loads. The previous segment's result stores were issued AFTER this segment's stage 0 (which
-                    // was put in flight ahead of them), so they may stay in flight: waiting for their acknowledgement
-                    // here cost 2 us per sequence boundary.
-                    PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage, pending_stores);
+                if (!deep || it == 0) issue(cur, it + 1, slot ^ 1);
+                // everything older than the transfers just enqueued has landed: stage `it`. The previous segment's
+                // result stores were issued AFTER this segment's stage 0 (which was put in flight ahead of them), so
+                // they may stay in flight: waiting for their acknowledgement here cost 2 us per sequence boundary.
+                PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage, pending_stores);
+                pending_stores = 0;
+                __builtin_amdgcn_sched_barrier(0);
+                compute_stage(wave_lds_addr + slot * kStageBytes, ro, ss, qB, kq, kStageTokens, p.score_scale, [&]() {
+                    if (deep && it + 2 < cur.n_stages) issue(cur, it + 2, slot);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- the last stage, outside the loop: the next segment's queries are loaded around it, and what the
+            // compiler knows about loads in flight must not travel around the loop above
+            {
+                const int slot = (slot0 + last) & 1;
+                has_next = direct && pos < r1;
+                if (has_next) {
+                    next_segment(nxt);
+                    load_query(nxt, qN, newN, std::true_type{}); // older than the transfers below
+                    issue(nxt, 0, slot ^ 1);
+                    PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage + kQueryLoads, pending_stores); // the last stage only
                 } else {
-                    has_next = direct && pos < r1;
-                    if (has_next) {
-                        next_segment(nxt);
-                        load_query(nxt, qN, newN); // older than the transfers below: landed before they are waited for
-                        issue(nxt, 0, slot ^ 1);
-                        PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage + kQueryLoads, pending_stores); // stage `it` only
-                    } else {
-                        PPLHIP_WAIT_VMCNT_PLUS(0, pending_stores);
-                    }
+                    PPLHIP_WAIT_VMCNT_PLUS(0, pending_stores);
                 }
                 pending_stores = 0;
                 __builtin_amdgcn_sched_barrier(0);
-                if (FUSED_WRITE && it + 1 == cur.n_stages && cur.has_new) {
+                if (FUSED_WRITE && cur.has_new) {
                     // The stage has landed with whatever the slab held in the new token's row: the row is replaced in
                     // the stage buffer by the freshly quantised token (LDS operations of one wave execute in order, so
                     // the reads below see it), and the same bytes go to the slab.
@@ -642,7 +678,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                         const int grp = lane & 15, isv = lane >> 4, r = cur.tail_rows_valid - 1;
                         uint2 qv;
                         half_t sc;
-                        quantize_group8(newB, &qv, &sc);
+                        quantize_group8(make_uint4(newB[0], newB[1], newB[2], newB[3]), &qv, &sc);
                         const uint32_t st = wave_lds_addr + slot * kStageBytes;
                         uint16_t sbits;
                         __builtin_memcpy(&sbits, &sc, 2);
@@ -665,14 +701,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                         row += isv ? (int64_t)kv_off : 0;
                         *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
                         p.scale[row / kQuantGroup + grp] = sc;
-                        // (counted below: two store instructions)
+                        // (two more stores behind the next stage 0; the waits count only the result rows)
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                compute_stage(wave_lds_addr + slot * kStageBytes, ro, ss, qB, kq,
-                              it + 1 == cur.n_stages ? cur.tail_rows_valid : kStageTokens, p.score_scale, [&]() {
-                                  if (deep && it + 2 < cur.n_stages) issue(cur, it + 2, slot);
-                              });
+                compute_stage(wave_lds_addr + slot * kStageBytes, ro, ss, qB, kq, cur.tail_rows_valid, p.score_scale,
+                              []() {});
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -757,9 +791,13 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         }
 
         if (has_next) { // its stage 0 is already in flight, in the buffer the last stage did not use
-            // (has_next implies the register epilogue: 4 stores of a finished row, or 8 + 2 of a partial result, and
-            // two more where the wave wrote its sequence's new token)
-            pending_stores = (cur.whole_sequence ? 4 : 10) + ((FUSED_WRITE && cur.has_new) ? 2 : 0);
+            // (has_next implies the register epilogue: 4 16-byte stores of a finished row, or 8 of a partial result.
+            // The count is a lower bound on the store instructions behind the next segment's stage 0 -- the small
+            // ones, which the compiler may merge, are left out -- so a wait that allows this many more operations in
+            // flight still covers stage 0 and everything older.)
+            pending_stores = cur.whole_sequence ? 4 : 8;
+            // the next segment's queries (and new token) are older than its stage 0: landed after this wait
+            PPLHIP_WAIT_VMCNT_PLUS(kDmaPerStage, pending_stores);
             slot0 = (slot0 + cur.n_stages) & 1;
             cur = nxt;
 #pragma unroll
@@ -771,7 +809,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         } else {
             if (pos >= r1) break;
             next_segment(cur);
-            load_query(cur, qB, newB);
+            load_query(cur, qB, newB, std::false_type{});
             slot0 = 0;
             cur_in_flight = false;
         }
