@@ -620,7 +620,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     Segment cur, nxt;
     next_segment(cur);
     int slot0 = 0; // stage buffer of the current segment's stage 0
-    bool cur_in_flight = false; // stage 0 of `cur` already enqueued by the previous segment's last iteration
+    // stage 0 of `cur` is already enqueued: by the previous segment's last stage, or here, AHEAD of the query loads,
+    // whose wait (in load_query) would otherwise pass before the first transfer is even requested
+    bool cur_in_flight = cur.n_stages > 0;
+    if (cur_in_flight) issue(cur, 0, 0);
     // store instructions issued behind the stage-0 transfers of a segment that was put in flight early (see the waits)
     int pending_stores = 0;
     half8_t qB[2][2];
@@ -809,9 +812,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
         } else {
             if (pos >= r1) break;
             next_segment(cur);
-            load_query(cur, qB, newB, std::false_type{});
             slot0 = 0;
-            cur_in_flight = false;
+            cur_in_flight = cur.n_stages > 0;
+            if (cur_in_flight) issue(cur, 0, 0);
+            load_query(cur, qB, newB, std::false_type{});
         }
     }
 }
