@@ -299,8 +299,8 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (the attention path has no collective; see DESIGN.md for how it "
-              "would shard by kv head). Re-run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU (the attention path has no collective: it would shard by kv head, "
+              "every GPU holding its heads' slice of the cache). Re-run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     import torch
     pkg = entry.load_package()
