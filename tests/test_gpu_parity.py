@@ -398,3 +398,42 @@ def test_cache_prefill_over_staged_rows():
     plans = []
     check(b, workloads.make_tensors(b, seed=64), cache_prefill=1, plans=plans)
     assert plans[-1].prefill_staging == 1
+
+
+@pytest.mark.parametrize("cache_prefill", [0, 1])
+def test_forward_replays_from_a_hip_graph(cache_prefill):
+    """pplhip_mhca_forward only enqueues kernels: captured into a HIP graph on a side stream, every replay (with the
+    program's own eager work and synchronisations between replays, new queries each time) gives bit for bit what the
+    eager call gives. With cache_prefill the chunks are large enough for the staged route (one more kernel)."""
+    import torch
+    import bench
+    lib = harness.pkg.load_library()
+    if cache_prefill:
+        b = workloads.Batch(8, 2, 128, [1, 1, 300, 700], [77, 1500, 100, 0], 2, name="graph_staged")
+    else:
+        b = workloads.Batch(8, 2, 128, [1, 1, 1, 150, 40], [300, 17, 1000, 0, 0], 3, name="graph_mixed")
+    db = bench.DeviceBatch(harness.pkg, lib, b, seed=3, n_slabs=1, cache_prefill=cache_prefill)
+    assert int(db.plan.prefill_staging) == cache_prefill
+    default_stream = db.stream
+    db.step(0)  # also takes the one-time per-device set-up out of the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        db.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        db.step(0)
+    db.stream = default_stream
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    for rep in range(3):
+        db.q.copy_(torch.randn(db.q.shape, generator=gen, dtype=torch.float16, device="cuda"))
+        db.out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = db.out.clone()
+        db.out.zero_()
+        db.step(0)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), db.out.view(torch.int16)), f"replay {rep} differs from the eager call"
+        assert bool(got.float().abs().sum() > 0)
