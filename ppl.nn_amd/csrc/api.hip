@@ -208,11 +208,10 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     hipStream_t s = (hipStream_t)stream;
     pplhip_kv_write_args w;
     write_args_from_mhca(a, &w);
-    // when the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens)
-    // into the slab itself, the launch below covers the prompt tokens only
-    // and the prompt tokens are left to the prefill launch unless it reads them back from the slab (cache-prefill)
-    const bool fused = decode_writes_new_tokens(a->decoding_batches, plan->decode_num_ranges);
-    pplhip_retcode rc = launch_kv_quantize_write(&w, s, fused ? a->decoding_batches : 0,
+    // the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens) into the
+    // slab itself, and the prompt tokens are left to the prefill launch unless it reads them back from the slab
+    // (cache-prefill): on the default path this launches nothing
+    pplhip_retcode rc = launch_kv_quantize_write(&w, s, a->decoding_batches,
                                                  prefill_writes_new_tokens(a) ? a->decoding_batches : -1);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
     rc = launch_decode(a, plan, d_workspace, s);

@@ -134,7 +134,6 @@ pplhip_retcode launch_kv_stage_prefill(const pplhip_mhca_args* a, half_t* key_ou
 // whether (and where in the workspace) a cache-prefill call stages its K/V as fp16: see pplhip_mhca_plan
 int64_t prefill_staging_tokens(const pplhip_mhca_args* a);
 int decode_heads_per_block(int kv_heads);
-bool decode_writes_new_tokens(int64_t decoding_batches, int num_ranges);
 bool prefill_writes_new_tokens(const pplhip_mhca_args* a);
 int decode_blocks_per_cu();
 int decode_waves_per_block();

@@ -62,7 +62,7 @@ constexpr int kDecodeLdsBytes = kDecodeWaves * kWaveLdsBytes; // 81920: two work
 
 struct DecodeParams {
     const half_t* q; // [S, H, Dh]
-    const half_t* cur_key; // [S, KVH, Dh] new tokens; null: the slab already holds them
+    const half_t* cur_key; // [S, KVH, Dh] new tokens: the decode sequences' are quantised into the slab by this launch
     const half_t* cur_value;
     int8_t* cache;
     half_t* scale;
@@ -436,11 +436,11 @@ __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, 
     }
 }
 
-// FUSED_WRITE: the wave that owns the tail of a sequence quantises the sequence's new token into the slab (and into
-// its stage buffer) itself; otherwise the slab already holds it.
+// The wave that owns the tail of a sequence quantises the sequence's new token into the slab (and into its stage
+// buffer) itself.
 // DIRECT: every wave owns a whole kv head (hpb == waves per workgroup); otherwise the waves split the tokens of a kv
 // head and combine through LDS.
-template <bool PAGED, bool FUSED_WRITE, bool DIRECT>
+template <bool PAGED, bool DIRECT>
 __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63;
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
             (int)(((int64_t)g.seg_end - last_stage_t0) < kStageTokens ? ((int64_t)g.seg_end - last_stage_t0) : kStageTokens);
         g.tail_rows_valid = (int)(t_end - last_stage_t0);
         const int64_t seq_len = seq_hi - seq_lo;
-        g.has_new = FUSED_WRITE && g.n_stages > 0 && t_end == seq_hi - seq_lo;
+        g.has_new = g.n_stages > 0 && t_end == seq_hi - seq_lo;
         const int64_t row0 = (PAGED ? 0 : (cachestarts[b] + (int64_t)g.t_begin) * (int64_t)stride) + head_off;
         g.cbase = reinterpret_cast<const char*>(p.cache) + row0;
         // where the range goes on: inside this sequence (then pos = r1), or at the next sequence's first token
@@ -583,12 +583,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
 
     // Q^T as the B operand, kept for a whole segment: q[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
     // four query pieces (+ the lane's group of the sequence's new token)
-    constexpr int kQueryLoads = FUSED_WRITE ? 5 : 4;
+    constexpr int kQueryLoads = 5;
     // lanes 0..15: groups of the new token's K row (this kv head), lanes 16..31: of its V row (upper half-wave mirrors)
     // untracked: by load16_untracked, for the hand-over inside a range (the caller waits); otherwise by ordinary
     // loads that are waited for on the spot (first segment of a range, token-split workgroups)
     auto load_query = [&](const Segment& g, half8_t (&q)[2][2], u32x4_t& newtok, auto untracked) {
-        if (FUSED_WRITE) {
+        {
             const half_t* src = ((lane & 16) ? p.cur_value : p.cur_key) +
                                 ((int64_t)g.qrow * p.kv_heads + kvh) * kDh + 8 * (lane & 15);
             if (untracked) load16_untracked(newtok, src);
@@ -673,7 +673,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
                 }
                 pending_stores = 0;
                 __builtin_amdgcn_sched_barrier(0);
-                if (FUSED_WRITE && cur.has_new) {
+                if (cur.has_new) {
                     // The stage has landed with whatever the slab held in the new token's row: the row is replaced in
                     // the stage buffer by the freshly quantised token (LDS operations of one wave execute in order, so
                     // the reads below see it), and the same bytes go to the slab.
@@ -920,14 +920,6 @@ int decode_heads_per_block(int kv_heads) {
     return hpb;
 }
 
-// Whether the decode kernel quantises the decode sequences' new tokens itself. It saves the separate launch, but
-// the tail of every sequence then costs its owner extra work on the launch's critical path: worth it as long as at
-// most half of the workgroups own a tail (measured: 120 sequences over 256 ranges -2.7 %, 8 over 512 -7 %, 64 over
-// 64 +3 %).
-bool decode_writes_new_tokens(int64_t decoding_batches, int num_ranges) {
-    return decoding_batches > 0 && 2 * decoding_batches <= (int64_t)num_ranges;
-}
-
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
     const int nd = (int)a->decoding_batches;
     if (nd == 0) return PPLHIP_RC_SUCCESS;
@@ -968,14 +960,10 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
         PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: no current device");
     if (!(lds_opted_in.load(std::memory_order_relaxed) >> dev & 1)) {
-        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, false, true>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true, true>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false, true>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true, true>)}) {
+        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true>),
+                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true>)}) {
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
             if (e != hipSuccess)
                 PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
@@ -983,25 +971,16 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
         }
         lds_opted_in.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
     }
-    const bool fused = decode_writes_new_tokens(nd, p.num_ranges);
     const dim3 grid((unsigned)blocks), block(kDecodeWaves * kWave);
     const bool direct = p.hpb == kDecodeWaves;
-#define PPLHIP_LAUNCH_DECODE(PAGED, FUSED)                                                                          \
-    do {                                                                                                            \
-        if (direct)                                                                                                 \
-            hipLaunchKernelGGL((decode_int8kv_kernel<PAGED, FUSED, true>), grid, block, lds_bytes, stream, p);      \
-        else                                                                                                        \
-            hipLaunchKernelGGL((decode_int8kv_kernel<PAGED, FUSED, false>), grid, block, lds_bytes, stream, p);     \
-    } while (0)
-    if (p.page_shift && fused)
-        PPLHIP_LAUNCH_DECODE(true, true);
+    if (p.page_shift && direct)
+        hipLaunchKernelGGL((decode_int8kv_kernel<true, true>), grid, block, lds_bytes, stream, p);
     else if (p.page_shift)
-        PPLHIP_LAUNCH_DECODE(true, false);
-    else if (fused)
-        PPLHIP_LAUNCH_DECODE(false, true);
+        hipLaunchKernelGGL((decode_int8kv_kernel<true, false>), grid, block, lds_bytes, stream, p);
+    else if (direct)
+        hipLaunchKernelGGL((decode_int8kv_kernel<false, true>), grid, block, lds_bytes, stream, p);
     else
-        PPLHIP_LAUNCH_DECODE(false, false);
-#undef PPLHIP_LAUNCH_DECODE
+        hipLaunchKernelGGL((decode_int8kv_kernel<false, false>), grid, block, lds_bytes, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
     // the sequences that need merging are those that straddle a range boundary: at most num_ranges - 1 of them,
     // however many sequences there are (2048 short sequences launched 65k workgroups that all left at once: 35 us)
