@@ -608,21 +608,12 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
         hl = ablock - rank * p.num_heads;
         constexpr int kRegPasses = 4; // tile counts of the first 256 sequences stay in registers
         int nreg[kRegPasses];
-        {
-            // every lane loads, past the end the last sequence again, and all four passes are requested before the
-            // first is used (the empty asm keeps the compiler from putting each load back under its lane mask, where
-            // it is waited for on its own: four round trips instead of one)
-            int64_t len[kRegPasses];
 #pragma unroll
-            for (int k = 0; k < kRegPasses; ++k) {
-                const int i = 64 * k + lane;
-                const int ic = i < p.num_seqs ? i : p.num_seqs - 1;
-                len[k] = p.seqstarts[p.first_seq + ic + 1] - p.seqstarts[p.first_seq + ic];
-            }
-            static_assert(kRegPasses == 4, "the operand list below names four passes");
-            asm volatile("" : "+v"(len[0]), "+v"(len[1]), "+v"(len[2]), "+v"(len[3]));
-#pragma unroll
-            for (int k = 0; k < kRegPasses; ++k) nreg[k] = 64 * k + lane < p.num_seqs ? (int)((len[k] + kBM - 1) / kBM) : 0;
+        for (int k = 0; k < kRegPasses; ++k) {
+            const int i = 64 * k + lane;
+            nreg[k] = i < p.num_seqs
+                          ? (int)((p.seqstarts[p.first_seq + i + 1] - p.seqstarts[p.first_seq + i] + kBM - 1) / kBM)
+                          : 0;
         }
         auto tiles_of = [&](int i) {
             return i < p.num_seqs
