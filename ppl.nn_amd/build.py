@@ -8,7 +8,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "decode.hip", "prefill.hip", "pack.hip", "rope.hip"]
+# attention.hip is decode.hip + prefill.hip in one translation unit (it includes them: a call with decode sequences and
+# prompts runs both kinds of workgroup in one launch)
+KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "attention.hip", "pack.hip", "rope.hip"]
+KERNEL_INCLUDED = ["decode.hip", "prefill.hip"]
 
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
@@ -30,7 +33,7 @@ def build_kernels(force=False, verbose=False):
     os.makedirs(LIBDIR, exist_ok=True)
     out = os.path.join(LIBDIR, "libppl_llm_kernel_hip.so")
     srcs = [os.path.join(CSRC, s) for s in KERNEL_SOURCES]
-    deps = srcs + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "exports.map"),
+    deps = srcs + [os.path.join(CSRC, s) for s in KERNEL_INCLUDED] + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "exports.map"),
                    os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip.h")]
     if not force and not _newer(out, deps):
         return out

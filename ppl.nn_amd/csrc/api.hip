@@ -214,9 +214,7 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     pplhip_retcode rc = launch_kv_quantize_write(&w, s, a->decoding_batches,
                                                  prefill_writes_new_tokens(a) ? a->decoding_batches : -1);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
-    rc = launch_decode(a, plan, d_workspace, s);
-    if (rc != PPLHIP_RC_SUCCESS) return rc;
-    return launch_prefill(a, plan, d_workspace, s);
+    return launch_decode_and_prefill(a, plan, d_workspace, s);
 }
 
 pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {

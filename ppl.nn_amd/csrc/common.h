@@ -139,6 +139,9 @@ int decode_blocks_per_cu();
 int decode_waves_per_block();
 pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
 pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
+// both, in one launch where the call has decode sequences and prompts
+pplhip_retcode launch_decode_and_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws,
+                                         hipStream_t stream);
 pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream);
 pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream);
 pplhip_retcode launch_position_index(const int64_t* d_seqstarts, const int64_t* d_start_pos, int64_t batch,

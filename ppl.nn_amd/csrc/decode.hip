@@ -39,6 +39,7 @@
 // consecutive (range, sequence) segments get consecutive slots -- and `decode_merge_kernel` combines the slots of a
 // sequence with the usual log-sum-exp weights.
 #include <atomic>
+#include <initializer_list>
 #include <type_traits>
 #include "common.h"
 
@@ -440,14 +441,15 @@ __device__ inline void compute_stage(uint32_t lds_stage, const ReadOffsets& ro, 
 // buffer) itself.
 // DIRECT: every wave owns a whole kv head (hpb == waves per workgroup); otherwise the waves split the tokens of a kv
 // head and combine through LDS.
+// `block`: the workgroup's index among the decode workgroups of the launch (they come first in the grid); `smem`: the
+// launch's dynamic LDS, kDecodeLdsBytes of it.
 template <bool PAGED, bool DIRECT>
-__global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+__device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t block, char* smem) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
     const int groups = p.kv_heads / p.hpb;
-    const int xcd = blockIdx.x & 7;
-    const int64_t j = blockIdx.x >> 3;
+    const int xcd = block & 7;
+    const int64_t j = block >> 3;
     const int hg = (int)(j % groups);
     const int64_t s_idx = (j / groups) * 8 + xcd; // range index
     // (virtual positions: see kBoundaryTokens)
@@ -820,6 +822,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
     }
 }
 
+template <bool PAGED, bool DIRECT>
+__global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(const DecodeParams p) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    decode_workgroup<PAGED, DIRECT>(p, blockIdx.x, smem);
+}
+
 // One workgroup of 256 lanes per (decode sequence, query head): 8 groups of 32 lanes stride over the partial slots of
 // the sequence (one per range it touches), each lane owning 4 channels; the groups' running (max, sum, acc) are combined
 // through LDS. out[d] = sum_s w_s acc_s[d] / sum_s w_s l_s with w_s = exp2(m_s - max_s m_s). Sequences that lie inside a
@@ -920,9 +928,27 @@ int decode_heads_per_block(int kv_heads) {
     return hpb;
 }
 
-pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
+// More than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in per kernel, once per device (the attribute is
+// kept per device by the runtime); setting it twice from two threads is harmless, so a relaxed bit mask is enough.
+static pplhip_retcode reserve_decode_lds(std::atomic<uint64_t>& done, std::initializer_list<const void*> kernels) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: no current device");
+    if (done.load(std::memory_order_relaxed) >> dev & 1) return PPLHIP_RC_SUCCESS;
+    for (const void* fn : kernels) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLdsBytes);
+        if (e != hipSuccess)
+            PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %d bytes of LDS per workgroup: %s",
+                        kDecodeLdsBytes, hipGetErrorString(e));
+    }
+    done.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
+    return PPLHIP_RC_SUCCESS;
+}
+
+// Fills the launch parameters of the decode sequences' attention; *blocks: workgroups of the launch.
+static pplhip_retcode decode_setup(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, DecodeParams* out,
+                                   int64_t* out_blocks) {
     const int nd = (int)a->decoding_batches;
-    if (nd == 0) return PPLHIP_RC_SUCCESS;
     DecodeParams p;
     p.q = (const half_t*)a->d_query;
     p.cur_key = (const half_t*)a->d_current_key;
@@ -952,25 +978,34 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     p.range_first = (int32_t*)((char*)ws + slots * p.num_heads * (kDh + 2) * sizeof(float));
     const int64_t blocks = (int64_t)p.num_ranges * (p.kv_heads / p.hpb);
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many tasks");
+    p.merge_by_boundary = nd > p.num_ranges - 1;
+    *out = p;
+    *out_blocks = blocks;
+    return PPLHIP_RC_SUCCESS;
+}
+
+// the sequences that need merging are those that straddle a range boundary: at most num_ranges - 1 of them, however
+// many sequences there are (2048 short sequences launched 65k workgroups that all left at once: 35 us)
+static pplhip_retcode launch_decode_merge(const DecodeParams& p, hipStream_t stream) {
+    hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, p.merge_by_boundary ? p.num_ranges - 1 : p.nd), dim3(256),
+                       0, stream, p);
+    PPLHIP_CHECK_LAUNCH("decode_merge");
+    return PPLHIP_RC_SUCCESS;
+}
+
+pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
+    if (a->decoding_batches == 0) return PPLHIP_RC_SUCCESS;
+    DecodeParams p;
+    int64_t blocks;
+    pplhip_retcode rc = decode_setup(a, plan, ws, &p, &blocks);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
     const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
-    // more than 64 KiB of dynamic LDS per workgroup needs an explicit opt-in, once per device (the attribute is kept
-    // per device by the runtime); setting it twice from two threads is harmless, so a relaxed bit mask is enough
     static std::atomic<uint64_t> lds_opted_in{0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
-        PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: no current device");
-    if (!(lds_opted_in.load(std::memory_order_relaxed) >> dev & 1)) {
-        for (const void* fn : {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, false>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<false, true>),
-                               reinterpret_cast<const void*>(decode_int8kv_kernel<true, true>)}) {
-            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess)
-                PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "decode: cannot reserve %zu bytes of LDS per workgroup: %s",
-                            lds_bytes, hipGetErrorString(e));
-        }
-        lds_opted_in.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
-    }
+    rc = reserve_decode_lds(lds_opted_in, {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false>),
+                                           reinterpret_cast<const void*>(decode_int8kv_kernel<true, false>),
+                                           reinterpret_cast<const void*>(decode_int8kv_kernel<false, true>),
+                                           reinterpret_cast<const void*>(decode_int8kv_kernel<true, true>)});
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
     const dim3 grid((unsigned)blocks), block(kDecodeWaves * kWave);
     const bool direct = p.hpb == kDecodeWaves;
     if (p.page_shift && direct)
@@ -982,13 +1017,7 @@ pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* 
     else
         hipLaunchKernelGGL((decode_int8kv_kernel<false, false>), grid, block, lds_bytes, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_int8kv");
-    // the sequences that need merging are those that straddle a range boundary: at most num_ranges - 1 of them,
-    // however many sequences there are (2048 short sequences launched 65k workgroups that all left at once: 35 us)
-    p.merge_by_boundary = nd > p.num_ranges - 1;
-    hipLaunchKernelGGL(decode_merge_kernel, dim3(p.num_heads, p.merge_by_boundary ? p.num_ranges - 1 : nd), dim3(256), 0,
-                       stream, p);
-    PPLHIP_CHECK_LAUNCH("decode_merge");
-    return PPLHIP_RC_SUCCESS;
+    return launch_decode_merge(p, stream);
 }
 
 } // namespace pplhip

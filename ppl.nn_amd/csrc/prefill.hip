@@ -577,17 +577,17 @@ typedef __attribute__((address_space(3))) short4_t* lds_short4_t;
 // the compact tile grid pays a search per workgroup: worth it from about 6 us of empty dispatches on
 constexpr int64_t kCompactMinEmpty = 8192;
 constexpr int kWriteUnits = 2; // units of four quantisation groups per thread of a write-only workgroup
-__global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams p) {
-    __shared__ __attribute__((aligned(1024))) char lds[4 * kDmaTile];
-
+// `block` of `nblocks`: the workgroup's index among the prefill workgroups of the launch; `lds`: 4 * kDmaTile bytes,
+// 1024-byte aligned.
+__device__ __forceinline__ void prefill_workgroup(const PrefillParams& p, uint32_t block, uint32_t nblocks, char* lds) {
     // Workgroups [0, attn_blocks) map to query tiles. The ones behind them quantise the prompt tokens into the slab
     // and leave: they are dispatched last, into the slots that the launch's tail leaves idle. (Measured against the
     // alternatives on 8 prompts of 64..1024 tokens: the same work as a share of every tile workgroup's prologue 67 us,
     // behind the tiles 62 us; dealt evenly INTO the grid 70 us, because that shifts the tiles' workgroup -> XCD
     // assignment and with it the L2 reuse of K/V among the query heads of a kv head.)
-    const uint32_t wblock = blockIdx.x - p.attn_blocks;
-    const bool is_wblock = blockIdx.x >= (unsigned)p.attn_blocks;
-    const uint32_t ablock = is_wblock ? 0 : blockIdx.x;
+    const uint32_t wblock = block - p.attn_blocks;
+    const bool is_wblock = block >= (unsigned)p.attn_blocks;
+    const uint32_t ablock = is_wblock ? 0 : block;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int b, hl, qt;
@@ -699,7 +699,7 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
         const int64_t units = (p.w_end_token - p.w_first_token) * p.w_per_tok;
         // kWriteUnits units per thread per pass, their 64-byte loads all issued before the first is used
         for (int64_t u0 = (int64_t)wblock * (256 * kWriteUnits) + threadIdx.x; u0 < units;
-             u0 += (int64_t)(gridDim.x - p.attn_blocks) * (256 * kWriteUnits)) {
+             u0 += (int64_t)(nblocks - p.attn_blocks) * (256 * kWriteUnits)) {
             uint4 raw[kWriteUnits][4];
 #pragma unroll
             for (int k = 0; k < kWriteUnits; ++k) {
@@ -1049,15 +1049,22 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams
     }
 }
 
+__global__ __launch_bounds__(256, 2) void prefill_f16_kernel(const PrefillParams p) {
+    __shared__ __attribute__((aligned(1024))) char lds[4 * kDmaTile];
+    prefill_workgroup(p, blockIdx.x, gridDim.x, lds);
+}
+
 // Whether the prefill launch quantises the prompt tokens into the slab itself (instead of a separate launch before
 // it): whenever it reads K/V from the fp16 inputs, i.e. does not depend on the slab holding them.
 bool prefill_writes_new_tokens(const pplhip_mhca_args* a) {
     return !a->enable_cache_prefill && a->batch > a->decoding_batches;
 }
 
-pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
+// Fills the launch parameters of the prompts' attention (and enqueues the staging pass where the plan has one).
+// *blocks: workgroups of the launch; *from_slab: the kernel that dequantises the int8 slab itself has to run it.
+static pplhip_retcode prefill_setup(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream,
+                                    PrefillParams* out, int64_t* out_blocks, bool* from_slab) {
     const int npre = (int)(a->batch - a->decoding_batches);
-    if (npre <= 0 || plan->prefill_num_q_tiles <= 0) return PPLHIP_RC_SUCCESS;
     PrefillParams p;
     p.kv_origin = nullptr;
     p.q = (const half_t*)a->d_query;
@@ -1122,8 +1129,21 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
         blocks += (units + 256 * kWriteUnits - 1) / (256 * kWriteUnits);
         if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "prefill: too many tokens in one call");
     }
+    *out = p;
+    *out_blocks = blocks;
+    *from_slab = a->enable_cache_prefill && !staged;
+    return PPLHIP_RC_SUCCESS;
+}
+
+pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
+    if (a->batch <= a->decoding_batches || plan->prefill_num_q_tiles <= 0) return PPLHIP_RC_SUCCESS;
+    PrefillParams p;
+    int64_t blocks;
+    bool from_slab;
+    const pplhip_retcode rc = prefill_setup(a, plan, ws, stream, &p, &blocks, &from_slab);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
     const dim3 grid((unsigned)blocks);
-    if (a->enable_cache_prefill && !staged)
+    if (from_slab)
         hipLaunchKernelGGL(prefill_attention_kernel<true>, grid, dim3(256), 0, stream, p);
     else
         hipLaunchKernelGGL(prefill_f16_kernel, grid, dim3(256), 0, stream, p);
