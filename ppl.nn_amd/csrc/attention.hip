@@ -1,12 +1,13 @@
 // MultiHeadCacheAttention's kernels in one translation unit: the decode sequences' attention (decode.hip), the prompts'
 // attention (prefill.hip), and -- for a call that has both -- ONE launch that carries the workgroups of both.
 //
-// Why one launch: the decode workgroups all run in a single round and finish between 80 % and 100 % of the launch's
-// duration (workgroups of identical work differ that much, and the launch lasts as long as the slowest), so for the
-// last fifth of it most CUs have nothing to do. The prompts' tile workgroups sit behind the decode workgroups in the
-// same grid and take the slots as they become free. Two streams give the same overlap (both parts done 179 us after
-// the decode launch started, against 198 us back to back, on the Llama-3-8B mixed batch), but the fork and the join are
-// two dependencies between hardware queues and cost the 17 us again; kernels of one stream never overlap.
+// Why one launch: kernels of one stream never overlap and every launch boundary costs a few microseconds of idle chip;
+// two streams overlap the two parts, but the fork and the join are two dependencies between hardware queues that cost
+// more than the overlap gains (Llama-3-8B mixed batch: 17 us). In one grid the decode workgroups come first and all run
+// at once; the prompts' tile workgroups sit behind them and take the slots as they become free. Measured on that batch:
+// 187 us per call instead of 199 (the launch itself takes about as long as the two kernels one after the other -- the
+// tile workgroups that move in share their CUs' memory pipes with the decode workgroups still running -- what is saved is
+// two launches and their gaps).
 #include "decode.hip"
 #include "prefill.hip"
 
