@@ -1,4 +1,5 @@
-// Decode attention over the int8 group-8 KV slab (one new token per sequence), split along the cached tokens.
+// Decode attention over the int8 group-8 KV slab (one new token per sequence, which the kernel also quantises into
+// the slab), split along the cached tokens.
 //
 // Roofline: HBM. Each cached token costs 2 * KVH * (Dh + Dh/4) bytes and is read exactly once; arithmetic
 // intensity is 1.6 .. 12.8 flop/B. Three things have to stay below the HBM time for the kernel to sit on that
@@ -12,7 +13,8 @@
 //     read once whatever the grouping, and the contraction costs two dozen MFMAs per 32 tokens.
 //
 // Work decomposition (balanced on the device, no host knowledge of the lengths): the cached tokens of all decode
-// sequences, laid end to end (kvstarts is exactly that prefix sum), are cut into S equal ranges. One workgroup owns one
+// sequences, laid end to end (kvstarts is exactly that prefix sum), are cut into S ranges of equal cost (equal length
+// on an axis that charges every sequence boundary a few positions: see kBoundaryTokens). One workgroup owns one
 // range for a group of up to 4 kv heads; where its range crosses sequence boundaries it handles the pieces ("segments")
 // one after the other. Every workgroup therefore streams the same number of bytes, whatever the raggedness of the batch,
 // and there is no tail of long sequences. Inside a workgroup each wave owns one kv head (the workgroup then reads

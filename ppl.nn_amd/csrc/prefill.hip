@@ -1,27 +1,29 @@
 // Causal prefill attention over ragged packed sequences (flash-attention style, fp16 MFMA, fp32 online softmax).
 //
 // Roofline: fp16 MFMA. One workgroup (4 wavefronts) owns 128 query rows of one (sequence, query head); each wave
-// owns 32 of them. K/V tiles of 64 tokens are staged in LDS once per workgroup and shared by the 4 waves (two buffers,
-// one barrier per tile), with the next tile's global loads in flight (held in registers) while the current tile is
-// computed; grouped query heads map to their kv head by integer division. Everything is computed transposed so that
-// probabilities never leave registers:
+// owns 32 of them. K/V tiles of 64 tokens are staged in LDS once per workgroup and shared by the 4 waves; grouped query
+// heads map to their kv head by integer division. Everything is computed transposed so that probabilities never leave
+// registers:
 //   S^T = K * Q^T    v_mfma_f32_32x32x16_f16, A = K tile from LDS (16 B per lane per MFMA), B = Q^T held in registers
 //                    -> lane (n = lane & 31, hb = lane >> 5) owns query row n and kv tokens {8*(r/4) + 4*hb + r%4}
-//   O^T += V^T * P^T A = V^T from LDS: the tile is transposed ONCE per workgroup on its way into LDS (4 tokens x 8
-//                    channels per thread, v_perm), laid out [channel][token position] with the positions permuted so
-//                    that the 8 tokens a lane owns in P^T are one 16-byte read; B = P^T is exactly the layout the score
-//                    registers already have.
-// Softmax statistics are per lane column, so rescaling O^T needs no cross-lane traffic; one shuffle per tile
-// combines the two half-waves' maxima. The reference maximum of a row is only moved when the running maximum has
-// outgrown it by more than 2^kRescaleLog2 (probabilities then stay below that factor, well inside fp16), which
-// removes the accumulator rescale from almost every tile. Tiles entirely above the causal diagonal are skipped.
-// Workgroups are numbered heaviest query tile first across ALL sequences and heads (longest-processing-time order,
-// which keeps the tail of the launch short for causal work), and the query heads of one kv head are spaced 8 apart so
-// that they run on the same XCD and share its L2 copy of the K/V rows. The output tile goes through LDS so that global
-// stores are full rows.
+//   O^T += V^T * P^T A = V^T from LDS, B = P^T, which is exactly the layout the score registers already have.
+// Softmax statistics are per lane column, so rescaling O^T needs no cross-lane traffic. The reference maximum of a row
+// is only moved when the running maximum has outgrown it by more than 2^kRescaleLog2 (probabilities then stay below
+// that factor, well inside fp16), which removes the accumulator rescale from almost every tile. Tiles entirely above
+// the causal diagonal are skipped. Workgroups are numbered heaviest query tile first across ALL sequences and heads
+// (longest-processing-time order, which keeps the tail of the launch short for causal work), and the query heads of
+// one kv head are spaced 8 apart so that they run on the same XCD and share its L2 copy of the K/V rows. The output
+// tile goes through LDS so that global stores are full rows.
 //
-// K/V source: the fp16 current_key/current_value of the sequence (default), or the int8 slab dequantised on the way
-// into LDS (cache-prefill: supports start_pos > 0, i.e. chunked prefill / prompt cache).
+// Two kernels:
+//   prefill_workgroup / prefill_f16_kernel   K/V are fp16 rows (current_key / current_value, MultiHeadAttention's
+//       key / value, or the staged rows of a cache-prefill call): tiles travel global -> LDS by DMA, unpadded and
+//       swizzled; V stays row-major and its transposed operands come from ds_read_b64_tr_b16; the scores of tile t+1
+//       are issued between the exponentials of tile t. Its grid also carries the workgroups that quantise the prompt
+//       tokens into the slab.
+//   prefill_attention_kernel<true>            K/V are the int8 slab (cache-prefill with small chunks): the next
+//       tile's global loads are held in registers while the current tile is computed, and are dequantised -- V also
+//       transposed (4 tokens x 8 channels per thread, v_perm) -- on their way into LDS.
 #include "common.h"
 
 namespace pplhip {
