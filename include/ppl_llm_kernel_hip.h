@@ -121,7 +121,8 @@ typedef struct pplhip_mhca_plan {
     int32_t prefill_num_q_tiles; /* ceil(max_seqlen / prefill_q_tile) */
     int32_t prefill_staging; /* cache-prefill only: 1 = the prompts' cached K/V are first dequantised into fp16 staging
                                 rows in the workspace (one streaming pass) and attention runs over those; 0 = the
-                                attention kernel dequantises the int8 slab itself (small chunks, or staging too large) */
+                                attention kernel dequantises the int8 slab itself (small chunks, or staging too large).
+                                The caller may clear it before forward to stay on the second route. */
     int32_t prefill_staging_offset_256; /* where the staging rows start in the workspace, in units of 256 bytes */
     int32_t reserved[1];
 } pplhip_mhca_plan;

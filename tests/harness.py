@@ -141,8 +141,9 @@ def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0):
-    """Same call through the C ABI on cuda:0."""
+def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0, staging=None):
+    """Same call through the C ABI on cuda:0. staging=0 clears plan.prefill_staging (the caller's way to keep a
+    cache-prefill call on the kernel that reads the int8 slab itself)."""
     import torch
     lib = pkg.load_library()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -164,6 +165,9 @@ def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layo
     plan = cabi.MhcaPlan()
     pkg.check(lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)), "mhca_prepare")
     ws = torch.empty(max(int(plan.workspace_bytes), 256), dtype=torch.uint8, device="cuda")
+    if staging is not None:
+        assert staging == 0, "a plan can only be taken OFF the staged route"
+        plan.prefill_staging = 0
     pkg.check(lib.pplhip_mhca_forward(C.byref(a), C.byref(plan), dev_ptr(ws), stream), "mhca_forward")
     torch.cuda.synchronize()
     if plan_out is not None:

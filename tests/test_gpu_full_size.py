@@ -39,3 +39,22 @@ def test_cfg3_long_context_reduced_and_property():
         want = vals.mean(axis=0)
         for h in range(8):
             assert np.abs(got["output"][i, h].astype(np.float64) - want).max() <= 2e-3 + 1e-2 * np.abs(want).max()
+
+
+def test_chunked_prefill_both_routes_at_full_size():
+    """Chunks of 512 tokens on top of 0 .. 4096 cached tokens (H32 / KVH8), with decode sequences in front: the staged
+    route (fp16 staging rows + the fp16 kernel, what the plan chooses) against the oracle, and against the route that
+    reads the int8 slab in the attention kernel (the caller cleared plan.prefill_staging): same slab bytes, outputs
+    within the attention tolerance of each other."""
+    b = workloads.Batch(32, 8, 128, [1, 1, 512, 512, 512, 512], [3000, 500, 2048, 4096, 1000, 0], 2,
+                        name="chunked_prefill_full")
+    t = workloads.make_tensors(b, seed=7)
+    plans = []
+    _, ref, staged = check(b, t, cache_prefill=1, plans=plans)
+    assert plans[-1].prefill_staging == 1
+    direct = harness.run_device(b, t, cache_prefill=1, staging=0)
+    assert np.array_equal(direct["cache"], staged["cache"])
+    assert np.array_equal(direct["scale"].view(np.uint16), staged["scale"].view(np.uint16))
+    harness.assert_attn_close(direct["output"], ref["output_f64"])
+    diff = np.abs(direct["output"].astype(np.float64) - staged["output"].astype(np.float64))
+    assert diff.max() <= 2 * (2e-3 + 1e-2 * np.abs(ref["output_f64"]).max())
