@@ -437,3 +437,25 @@ def test_forward_replays_from_a_hip_graph(cache_prefill):
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), db.out.view(torch.int16)), f"replay {rep} differs from the eager call"
         assert bool(got.float().abs().sum() > 0)
+
+
+def test_degenerate_batches():
+    """An empty call; decode sequences whose cache is empty (their new token is their only key); one-token prompts; a
+    single sequence of each kind."""
+    import torch
+    lib = harness.pkg.load_library()
+    a, plan = cabi.MhcaArgs(), cabi.MhcaPlan()
+    b0 = workloads.Batch(8, 2, 128, [], [], 0, name="empty")
+    harness.fill_mhca_args(a, b0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, ptr=lambda t: C.c_void_p(0x1000))
+    assert lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+    assert lib.pplhip_mhca_forward(C.byref(a), C.byref(plan), None, None) == cabi.RC_SUCCESS
+    torch.cuda.synchronize()
+    for kvh in (2, 8):
+        b = workloads.Batch(8, kvh, 128, [1, 1, 1], [0, 5, 0], 3, name="decode_with_empty_cache")
+        check(b, workloads.make_tensors(b, seed=71))
+        b = workloads.Batch(8, kvh, 128, [1, 1, 1, 1], [0, 33, 0, 0], 2, name="one_token_prompts")
+        check(b, workloads.make_tensors(b, seed=72))
+        b = workloads.Batch(8, kvh, 128, [1], [0], 1, name="single_decode_empty_cache")
+        check(b, workloads.make_tensors(b, seed=73))
+        b = workloads.Batch(8, kvh, 128, [1], [0], 0, name="single_one_token_prompt")
+        check(b, workloads.make_tensors(b, seed=74))
