@@ -459,3 +459,14 @@ def test_degenerate_batches():
         check(b, workloads.make_tensors(b, seed=73))
         b = workloads.Batch(8, kvh, 128, [1], [0], 0, name="single_one_token_prompt")
         check(b, workloads.make_tensors(b, seed=74))
+
+
+@pytest.mark.parametrize("KVH", [8, 1])
+def test_hundreds_of_decode_sequences(KVH):
+    """300 decode sequences (five passes of the 64-wide table search), some with an empty cache, a few long ones that
+    span many ranges among them, and prompts behind them."""
+    rng = np.random.default_rng(81)
+    hist = rng.integers(0, 60, 300)
+    hist[[7, 150, 299]] = [3000, 1777, 2500]
+    b = workloads.Batch(8, KVH, 128, [1] * 300 + [40, 3], hist.tolist() + [0, 0], 300, name="300 decode sequences")
+    check(b, workloads.make_tensors(b, seed=82))
