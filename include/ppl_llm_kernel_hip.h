@@ -45,6 +45,11 @@ const char* pplhip_last_error(void);
 /* Library/ABI version: major*10000 + minor*100 + patch. */
 int32_t pplhip_version(void);
 
+/* Optional, once per process with the GPU current (the reference engine's counterpart is the device set-up in
+ * src/ppl/nn/engines/llm_cuda/llm_cuda_device.cc:60-100): reads the current device's compute-unit count, which sizes
+ * the decode plan. Without it pplhip_mhca_prepare plans for the 256 compute units of MI355X. Touches the device. */
+pplhip_retcode pplhip_init(void);
+
 /*
  * Argument block of MultiHeadCacheAttention: one field per argument the reference passes to `heuristic_prepare`
  * (multi_head_cache_attention_kernel.cc:170-212), in the same order and with the same meaning.
@@ -130,7 +135,8 @@ typedef struct pplhip_mhca_plan {
 /* Host-only: validates `args` exactly like the reference wrapper + kernel library would
  * (unsupported attrs -> PPLHIP_RC_UNSUPPORTED, inconsistent sizes -> PPLHIP_RC_INVALID_VALUE),
  * picks the split-k decomposition (how many equal token ranges) and reports the workspace size. Replaces `heuristic_prepare`
- * (multi_head_cache_attention_kernel.cc:170). Does not touch the device. */
+ * (multi_head_cache_attention_kernel.cc:170). Makes no HIP call and reads no environment: the plan depends on `args`
+ * and on the compute-unit count recorded by pplhip_init() (256 before it) only. */
 pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* args, pplhip_mhca_plan* plan);
 
 /* Enqueues: quantize-on-write of the new K/V tokens, decode attention (+ split-k merge) for the first

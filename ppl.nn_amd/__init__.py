@@ -106,6 +106,9 @@ def load_engine_library():
             "pplnn_hip_tensor_copy_to_host": (u32, [vp, vp]),
             "pplnn_hip_tensor_use_host_device": (None, [vp]),
             "pplnn_hip_selftest_registry": (u32, []),
+            "pplnn_x86_engine_create": (vp, []),
+            "pplnn_x86_set_num_threads": (None, [ctypes.c_int]),
+            "pplnn_x86_get_num_threads": (ctypes.c_int, []),
             "pplnn_hip_arena_create_host": (vp, [u64, u64]),
             "pplnn_hip_arena_alloc": (u32, [vp, u64, ctypes.POINTER(vp), ctypes.POINTER(u64)]),
             "pplnn_hip_arena_free": (None, [vp, vp]),

@@ -116,6 +116,7 @@ class PackArgs(C.Structure):
 PROTOTYPES = {
     "pplhip_last_error": (C.c_char_p, []),
     "pplhip_version": (_i32, []),
+    "pplhip_init": (_i32, []),
     "pplhip_mhca_prepare": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan)]),
     "pplhip_mhca_forward": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan), _p, _p]),
     "pplhip_mha_forward": (_i32, [C.POINTER(MhaArgs), _p]),

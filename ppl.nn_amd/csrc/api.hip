@@ -1,6 +1,7 @@
 // C ABI entry points: argument validation (same outcomes as the reference wrapper's checks), the split-k
 // heuristic, and the launch sequence write -> decode(+merge) -> prefill on the caller's stream.
 #include <stdarg.h>
+#include <atomic>
 #include <stdlib.h>
 #include <string.h>
 
@@ -17,16 +18,10 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+// Compute units the decode plan is sized for: MI355X's 256 until pplhip_init() has read the current device's count.
+static std::atomic<int> g_cu_count{256};
 static int device_cu_count() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256; // MI355X
-    }
-    return cus;
+    return g_cu_count.load(std::memory_order_relaxed);
 }
 
 static pplhip_retcode validate_common(int num_kv_heads, int head_dim, int num_layer, int layer_idx,
@@ -42,6 +37,10 @@ static pplhip_retcode validate_common(int num_kv_heads, int head_dim, int num_la
         PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support quantized cache but scale not found");
     if (stride_s <= 0 || stride_s % 16 || stride_l % 16 || stride_h % 16 || stride_kv % 16)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache strides must be positive multiples of 16 elements");
+    // the kernels keep the offsets inside a stage of 32 (decode) or a tile of 64 (prefill) tokens in 32 bits
+    if (stride_s >= (int64_t(1) << 25))
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "cache_stride_s %lld: at most 2^25 - 16 elements between tokens",
+                    (long long)stride_s);
     if (((uintptr_t)cache & 15) || ((uintptr_t)scale & 15))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache and scale must be 16-byte aligned");
     return PPLHIP_RC_SUCCESS;
@@ -112,7 +111,16 @@ const char* pplhip_last_error(void) {
 }
 
 int32_t pplhip_version(void) {
-    return 100; // 0.1.0
+    return 200; // 0.2.0
+}
+
+pplhip_retcode pplhip_init(void) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+        PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "init: no current HIP device");
+    if (prop.multiProcessorCount > 0) g_cu_count.store(prop.multiProcessorCount, std::memory_order_relaxed);
+    return PPLHIP_RC_SUCCESS;
 }
 
 pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* plan) {
@@ -162,10 +170,7 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         const int64_t slots = (int64_t)device_cu_count() * decode_blocks_per_cu();
         // halves of a slot: every workgroup streams the same number of bytes, so one workgroup per slot (a single,
         // perfectly filled round) measures best; the knob moves it to half or twice that
-        int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
-        if (const char* env = getenv("PPLHIP_DECODE_TASKS_PER_SLOT")) { // tuning aid, in workgroups per slot
-            if (atoll(env) > 0) half_slots = 2 * atoll(env);
-        }
+        const int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
         // ranges x groups workgroups must not spill over the slots (a second, nearly empty round doubles the time:
         // 40 kv heads = 10 groups took 56 ranges = 560 workgroups on 512 slots), so everything rounds DOWN to the
         // multiple of 8 the XCD-aware numbering needs

@@ -48,10 +48,7 @@
 namespace pplhip {
 
 constexpr int kDh = 128; // head_dim this kernel is specialised for
-#ifndef PPLHIP_DECODE_WAVES
-#define PPLHIP_DECODE_WAVES 4
-#endif
-constexpr int kDecodeWaves = PPLHIP_DECODE_WAVES; // waves per workgroup; each owns a 20 KiB double-buffered LDS region
+constexpr int kDecodeWaves = 4; // waves per workgroup; each owns a 20 KiB double-buffered LDS region
 constexpr int kStageTokens = 32; // tokens per pipeline stage (2 MFMA sub-blocks of 16)
 constexpr int kSubBlocks = kStageTokens / 16;
 // LDS bytes of one stage of one wave, and where its four arrays start
@@ -92,10 +89,7 @@ struct DecodeParams {
 // range with the most boundaries. The ranges are therefore cut on a virtual axis on which every sequence is followed by
 // kBoundaryTokens positions that hold no token: sequence i starts at kvstarts[i] + i * kBoundaryTokens. Equal virtual
 // ranges give a range with many boundaries fewer tokens.
-#ifndef PPLHIP_BOUNDARY_TOKENS
-#define PPLHIP_BOUNDARY_TOKENS 32
-#endif
-constexpr int kBoundaryTokens = PPLHIP_BOUNDARY_TOKENS;
+constexpr int kBoundaryTokens = 32;
 
 // Positions per range: the total is only known on the device. At least 128 so that tiny batches are not shredded.
 __device__ inline int64_t range_tokens(int64_t total, int num_ranges) {
@@ -265,15 +259,18 @@ __device__ inline void make_dma_offsets(DmaOffsets& o, int lane, uint32_t stride
 // Enqueues the 10 global->LDS transfers of one stage. cbase/sbase: K row 0 of the stage in the cache / scale tensors;
 // kv_off / kv_off_s: distance from a K row to the V row of the same token.
 __device__ inline void dma_stage(char* lds_stage, const char* cbase, const char* sbase, const DmaOffsets& o,
-                                 uint32_t kv_off, uint32_t kv_off_s) {
+                                 int64_t kv_off, int64_t kv_off_s) {
+    // the K -> V distance is folded into the wave-uniform base (it exceeds 32 bits in a large cache_layout 3 slab)
+    const char* vbase = cbase + kv_off;
+    const char* vsbase = sbase + kv_off_s;
 #pragma unroll
     for (int i = 0; i < kStageTokens / 8; ++i) {
         __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + o.kv[i]), (lds_ptr_t)(lds_stage + kLdsK + 1024 * i), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(cbase + kv_off + o.kv[i]), (lds_ptr_t)(lds_stage + kLdsV + 1024 * i),
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(vbase + o.kv[i]), (lds_ptr_t)(lds_stage + kLdsV + 1024 * i),
                                          16, 0, 0);
     }
     __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + o.sc), (lds_ptr_t)(lds_stage + kLdsKs), 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(sbase + kv_off_s + o.sc), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(vsbase + o.sc), (lds_ptr_t)(lds_stage + kLdsVs), 16, 0, 0);
 }
 
 // The same 10 transfers when a stage may straddle two pages of a paged slab: rows below `split` come from page A
@@ -281,8 +278,8 @@ __device__ inline void dma_stage(char* lds_stage, const char* cbase, const char*
 // would precede page B's first row by `split` rows, so the same per-row offsets apply). The base is then per lane,
 // so these transfers take the 64-bit vector-address form.
 __device__ inline void dma_stage_paged(char* lds_stage, const char* cbase_a, const char* cbase_b, const char* sbase_a,
-                                       const char* sbase_b, int split, const DmaOffsets& o, uint32_t kv_off,
-                                       uint32_t kv_off_s) {
+                                       const char* sbase_b, int split, const DmaOffsets& o, int64_t kv_off,
+                                       int64_t kv_off_s) {
 #pragma unroll
     for (int i = 0; i < kStageTokens / 8; ++i) {
         const char* cb = (o.kv_row[i] < split ? cbase_a : cbase_b) + o.kv[i];
@@ -470,10 +467,12 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
     const int m = lane & 15;
     const int kq = lane >> 4;
 
-    const uint32_t stride = (uint32_t)p.addr.stride_s; // bytes between tokens (int8 elements)
+    // bytes between tokens (int8 elements); the entry points reject strides of 2^25 and more, so the offsets of a
+    // 32-token stage (and of a 64-token prefill tile) fit 32 bits
+    const uint32_t stride = (uint32_t)p.addr.stride_s;
     const uint32_t sstride_b = (uint32_t)(p.addr.stride_s / kQuantGroup) * 2u;
-    const uint32_t kv_off = (uint32_t)p.addr.stride_kv;
-    const uint32_t kv_off_s = (uint32_t)(p.addr.stride_kv / kQuantGroup) * 2u;
+    const int64_t kv_off = p.addr.stride_kv; // up to KVH * MaxT * Dh in cache_layout 3: not a 32-bit quantity
+    const int64_t kv_off_s = p.addr.stride_kv / kQuantGroup * 2;
     const int64_t step_c = (int64_t)kStageTokens * stride, step_s = (int64_t)kStageTokens * sstride_b;
     DmaOffsets full;
     make_dma_offsets(full, lane, stride, sstride_b, kStageTokens);
@@ -705,7 +704,7 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
                         } else {
                             row = (cur.cbase - reinterpret_cast<const char*>(p.cache)) + tl * (int64_t)stride;
                         }
-                        row += isv ? (int64_t)kv_off : 0;
+                        row += isv ? kv_off : 0;
                         *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
                         p.scale[row / kQuantGroup + grp] = sc;
                         // (two more stores behind the next stage 0; the waits count only the result rows)

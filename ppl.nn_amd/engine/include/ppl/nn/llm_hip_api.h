@@ -244,6 +244,32 @@ public:
 
 }} // namespace llm::hip
 
+// The x86 engine that runs the fp32 ONNX attention subgraph (MatMul / Mul / Add / Softmax / Transpose) on the host
+// cores: the CPU baseline behind the same boundary.
+//   EngineOptions / ENGINE_CONF_* / MM_*   include/ppl/nn/engines/x86/{engine_options.h:26-30, options.h:26-63}
+//   EngineFactory                          include/ppl/nn/engines/x86/engine_factory.h
+//   SetGlobalOmpNumThreads                 used by tools/pplnn.cc:377-380 for --num-threads
+namespace x86 {
+
+enum { ENGINE_CONF_GRAPH_FUSION = 0, ENGINE_CONF_TENSOR_DEBUG = 1, ENGINE_CONF_DEBUG_DATA_DIR = 2, ENGINE_CONF_MAX };
+enum { MM_COMPACT = 0, MM_MRU = 1, MM_PLAIN = 2 };
+
+struct EngineOptions final {
+    uint32_t mm_policy = MM_COMPACT;
+    bool disable_avx512 = false; // accepted; the kernels pick their instruction set at load time
+    bool disable_avx_fma3 = false;
+};
+
+class EngineFactory final {
+public:
+    static Engine* Create(const EngineOptions&);
+};
+
+void SetGlobalOmpNumThreads(int num_threads);
+int GetGlobalOmpNumThreads();
+
+} // namespace x86
+
 }} // namespace ppl::nn
 
 #endif

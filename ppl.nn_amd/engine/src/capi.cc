@@ -33,6 +33,11 @@ uint32_t pplnn_hip_engine_configure_str(void* e, uint32_t option, const char* va
 }
 void pplnn_hip_engine_destroy(void* e) { delete static_cast<Engine*>(e); }
 
+// ---- x86 engine (the CPU baseline behind the same builder / runtime calls)
+void* pplnn_x86_engine_create(void) { return x86::EngineFactory::Create(x86::EngineOptions()); }
+void pplnn_x86_set_num_threads(int n) { x86::SetGlobalOmpNumThreads(n); }
+int pplnn_x86_get_num_threads(void) { return x86::GetGlobalOmpNumThreads(); }
+
 // ---- builder
 void* pplnn_hip_builder_create(void) { return onnx::RuntimeBuilderFactory::Create(); }
 uint32_t pplnn_hip_builder_load_model(void* b, const char* buf, uint64_t len) {

@@ -49,6 +49,10 @@ public:
             return RC_NOT_FOUND;
         }
         if (hipSetDevice(device_id) != hipSuccess) return RC_DEVICE_RUNTIME_ERROR;
+        if (pplhip_init() != PPLHIP_RC_SUCCESS) { // the kernel library plans its decode split for this device
+            LOG(ERROR) << "kernel library init failed: " << pplhip_last_error();
+            return RC_DEVICE_RUNTIME_ERROR;
+        }
         if (stream) {
             stream_ = (hipStream_t)stream;
         } else {

@@ -74,6 +74,7 @@ struct PbAttr final {
     int64_t i = 0;
     float f = 0;
     std::string s;
+    std::vector<int64_t> ints;
     bool has_i = false, has_f = false;
 };
 
@@ -92,6 +93,8 @@ bool ParseAttr(Reader r, PbAttr* a) {
         else if (f == 2 && wt == 5) { uint32_t u = (uint32_t)v; memcpy(&a->f, &u, 4); a->has_f = true; }
         else if (f == 3 && wt == 0) { a->i = (int64_t)v; a->has_i = true; }
         else if (f == 4 && wt == 2) a->s = sub.Str();
+        else if (f == 8 && wt == 2) { while (!sub.Done()) a->ints.push_back((int64_t)sub.Varint()); } // packed ints
+        else if (f == 8 && wt == 0) a->ints.push_back((int64_t)v);
     }
     return r.ok;
 }
@@ -234,10 +237,11 @@ bool GetNodeAttr(const PbNode& n, const char* key, T* value, T dft) {
 
 struct ParserInfo final {
     std::function<std::shared_ptr<ir::Attr>()> create_param; // may be empty for ops without attributes
-    std::function<RetCode(const PbNode&, const std::string& node_name, ir::Attr*)> parse_param;
+    std::function<RetCode(const PbNode&, const ir::Node&, ir::Attr*)> parse_param;
 };
 
-RetCode ParseMultiHeadCacheAttentionParam(const PbNode& pb, const std::string& node_name, ir::Attr* arg) {
+RetCode ParseMultiHeadCacheAttentionParam(const PbNode& pb, const ir::Node& node, ir::Attr* arg) {
+    const std::string& node_name = node.name;
     auto param = static_cast<opmx::MultiHeadCacheAttentionParam*>(arg);
     if (!GetNodeAttr(pb, "num_heads", &param->num_heads, -1)) { LOG(ERROR) << node_name << ": missing num_heads"; return RC_INVALID_VALUE; }
     if (!GetNodeAttr(pb, "head_dim", &param->head_dim, -1)) { LOG(ERROR) << node_name << ": missing head_dim"; return RC_INVALID_VALUE; }
@@ -257,7 +261,8 @@ RetCode ParseMultiHeadCacheAttentionParam(const PbNode& pb, const std::string& n
     return RC_SUCCESS;
 }
 
-RetCode ParseKeyValueCacheParam(const PbNode& pb, const std::string& node_name, ir::Attr* arg) {
+RetCode ParseKeyValueCacheParam(const PbNode& pb, const ir::Node& node, ir::Attr* arg) {
+    const std::string& node_name = node.name;
     auto param = static_cast<opmx::KeyValueCacheParam*>(arg);
     if (!GetNodeAttr(pb, "num_layer", &param->num_layer, -1)) { LOG(ERROR) << node_name << ": missing num_layer"; return RC_INVALID_VALUE; }
     if (!GetNodeAttr(pb, "layer_idx", &param->layer_idx, -1)) { LOG(ERROR) << node_name << ": missing layer_idx"; return RC_INVALID_VALUE; }
@@ -271,7 +276,8 @@ RetCode ParseKeyValueCacheParam(const PbNode& pb, const std::string& node_name, 
 }
 
 // models/onnx/parsers/opmx/parse_multi_head_attention_param.cc:10-31
-RetCode ParseMultiHeadAttentionParam(const PbNode& pb, const std::string& node_name, ir::Attr* arg) {
+RetCode ParseMultiHeadAttentionParam(const PbNode& pb, const ir::Node& node, ir::Attr* arg) {
+    const std::string& node_name = node.name;
     auto param = static_cast<opmx::MultiHeadAttentionParam*>(arg);
     if (!GetNodeAttr(pb, "num_heads", &param->num_heads, -1)) { LOG(ERROR) << node_name << ": missing num_heads"; return RC_INVALID_VALUE; }
     if (!GetNodeAttr(pb, "head_dim", &param->head_dim, -1)) { LOG(ERROR) << node_name << ": missing head_dim"; return RC_INVALID_VALUE; }
@@ -285,7 +291,8 @@ RetCode ParseMultiHeadAttentionParam(const PbNode& pb, const std::string& node_n
 }
 
 // models/onnx/parsers/opmx/parse_rotary_position_embedding_param.cc:10-41
-RetCode ParseRotaryPositionEmbeddingParam(const PbNode& pb, const std::string& node_name, ir::Attr* arg) {
+RetCode ParseRotaryPositionEmbeddingParam(const PbNode& pb, const ir::Node& node, ir::Attr* arg) {
+    const std::string& node_name = node.name;
     auto param = static_cast<opmx::RotaryPositionEmbeddingParam*>(arg);
     if (!GetNodeAttr(pb, "theta", &param->theta, -1.0f)) { LOG(ERROR) << node_name << ": missing theta"; return RC_INVALID_VALUE; }
     GetNodeAttr(pb, "bypass_key", &param->bypass_key, 0);
@@ -305,6 +312,21 @@ RetCode ParseRotaryPositionEmbeddingParam(const PbNode& pb, const std::string& n
         LOG(ERROR) << "unsupported scaling_type: " << scaling_type;
         return RC_UNSUPPORTED;
     }
+    return RC_SUCCESS;
+}
+
+// models/onnx/parsers/onnx/parse_softmax_param.cc:26-32: the default axis depends on the opset
+RetCode ParseSoftmaxParam(const PbNode& pb, const ir::Node& node, ir::Attr* arg) {
+    auto param = static_cast<ppl::nn::onnx::SoftmaxParam*>(arg);
+    GetNodeAttr(pb, "axis", &param->axis, node.type.version >= 13 ? -1 : 1);
+    return RC_SUCCESS;
+}
+
+// models/onnx/parsers/onnx/parse_transpose_param.cc: `perm`, empty = reverse the dimensions
+RetCode ParseTransposeParam(const PbNode& pb, const ir::Node&, ir::Attr* arg) {
+    auto param = static_cast<ppl::nn::onnx::TransposeParam*>(arg);
+    for (auto& a : pb.attrs)
+        if (a.name == "perm") param->perm.assign(a.ints.begin(), a.ints.end());
     return RC_SUCCESS;
 }
 
@@ -328,6 +350,12 @@ utils::OpInfoManager<ParserInfo>& ParamParserManager() {
         reg("opmx.dynamic_batching", "RotaryPositionEmbedding", 1, 1,
             {[] { return std::make_shared<opmx::RotaryPositionEmbeddingParam>(); }, ParseRotaryPositionEmbeddingParam});
         reg("opmx.dynamic_batching", "PositionIndex", 1, 1, {nullptr, nullptr}); // no attributes
+        // the ONNX ops of the attention subgraph the x86 engine runs (param_parser_manager.cc: same version ranges)
+        reg("", "Softmax", 1, 16, {[] { return std::make_shared<ppl::nn::onnx::SoftmaxParam>(); }, ParseSoftmaxParam});
+        reg("", "Transpose", 1, 16, {[] { return std::make_shared<ppl::nn::onnx::TransposeParam>(); }, ParseTransposeParam});
+        reg("", "MatMul", 1, 16, {nullptr, nullptr});
+        reg("", "Mul", 7, 16, {nullptr, nullptr});
+        reg("", "Add", 7, 16, {nullptr, nullptr});
     });
     return mgr;
 }
@@ -438,7 +466,7 @@ RetCode ParseModel(const char* buf, uint64_t size, ir::Graph* graph) {
         auto info = ParamParserManager().Find(node.type.domain, node.type.name, node.type.version);
         if (info && info->create_param) {
             auto param = info->create_param();
-            const RetCode rc = info->parse_param(pb, node.name, param.get());
+            const RetCode rc = info->parse_param(pb, node, param.get());
             if (rc != RC_SUCCESS) {
                 LOG(ERROR) << "parse attr of node[" << node.name << "] failed: " << GetRetCodeStr(rc);
                 return rc;

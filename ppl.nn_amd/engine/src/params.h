@@ -3,6 +3,7 @@
 //   src/ppl/nn/params/opmx/key_value_cache_param.h:10-30
 //   src/ppl/nn/params/opmx/multi_head_attention_param.h:10-26
 //   src/ppl/nn/params/opmx/rotary_position_embedding_param.h:10-36
+//   src/ppl/nn/params/onnx/softmax_param.h, transpose_param.h (the ONNX ops of the x86 attention subgraph)
 #ifndef PPLNN_LLM_HIP_PARAMS_H_
 #define PPLNN_LLM_HIP_PARAMS_H_
 
@@ -78,5 +79,19 @@ struct RotaryPositionEmbeddingParam final : public ir::Attr {
 };
 
 }}} // namespace ppl::nn::opmx
+
+namespace ppl { namespace nn { namespace onnx {
+
+struct SoftmaxParam final : public ir::Attr {
+    int32_t axis = 1;
+    bool operator==(const SoftmaxParam& p) const { return axis == p.axis; }
+};
+
+struct TransposeParam final : public ir::Attr {
+    std::vector<int32_t> perm;
+    bool operator==(const TransposeParam& p) const { return perm == p.perm; }
+};
+
+}}} // namespace ppl::nn::onnx
 
 #endif

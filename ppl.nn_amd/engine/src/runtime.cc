@@ -238,6 +238,11 @@ public:
         for (auto e : topo->constants) {
             auto t = make(e);
             auto& c = info->graph.data->constants[e];
+            if (c.data.size() < t->GetShape()->CalcBytesIncludingPadding()) { // dims promise more than the payload holds
+                LOG(ERROR) << "initializer[" << t->GetName() << "] holds " << c.data.size() << " bytes, its shape needs "
+                           << t->GetShape()->CalcBytesIncludingPadding();
+                return RC_INVALID_VALUE;
+            }
             auto rc = t->CopyFromHost(c.data.data());
             if (rc != RC_SUCCESS) return rc;
         }

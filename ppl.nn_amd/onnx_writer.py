@@ -1,7 +1,8 @@
 """Minimal ONNX ModelProto writer (protobuf wire format by hand; no onnx / protobuf package needed).
 Field numbers follow onnx.proto: ModelProto{ir_version=1, graph=7, opset_import=8}, GraphProto{node=1, name=2,
 input=11, output=12}, NodeProto{input=1, output=2, name=3, op_type=4, attribute=5, domain=7},
-AttributeProto{name=1, f=2, i=3, type=20}, ValueInfoProto{name=1, type=2}."""
+AttributeProto{name=1, f=2, i=3, s=4, ints=8, type=20}, ValueInfoProto{name=1, type=2}, GraphProto.initializer=5 with
+TensorProto{dims=1, data_type=2, name=8, raw_data=9}."""
 import struct
 
 FLOAT, INT8, INT64, FLOAT16 = 1, 3, 7, 10
@@ -42,6 +43,15 @@ def attr_float(name, v):
     return _str(1, name) + _key(2, 5) + struct.pack("<f", v) + _int(20, 1)
 
 
+def attr_ints(name, vs):
+    return _str(1, name) + b"".join(_int(8, v) for v in vs) + _int(20, 7)
+
+
+def initializer(name, elem_type, dims, raw):
+    """TensorProto with raw little-endian data."""
+    return b"".join(_int(1, d) for d in dims) + _int(2, elem_type) + _str(8, name) + _ld(9, bytes(raw))
+
+
 def value_info(name, elem_type, dims):
     """dims: ints, or strings for symbolic dimensions."""
     shape = b"".join(_ld(1, _int(1, d) if isinstance(d, int) else _str(2, d)) for d in dims)
@@ -59,9 +69,9 @@ def node(op_type, inputs, outputs, name="", domain="", attrs=()):
     return b
 
 
-def model(nodes, inputs, outputs, opsets, graph_name="g"):
-    graph = b"".join(_ld(1, n) for n in nodes) + _str(2, graph_name) + b"".join(_ld(11, i) for i in inputs) + \
-        b"".join(_ld(12, o) for o in outputs)
+def model(nodes, inputs, outputs, opsets, graph_name="g", initializers=()):
+    graph = b"".join(_ld(1, n) for n in nodes) + _str(2, graph_name) + b"".join(_ld(5, t) for t in initializers) + \
+        b"".join(_ld(11, i) for i in inputs) + b"".join(_ld(12, o) for o in outputs)
     m = _int(1, 8) + _ld(7, graph)
     for domain, version in opsets:
         m += _ld(8, (_str(1, domain) if domain else b"") + _int(2, version))
@@ -184,3 +194,25 @@ def position_index_model():
     names = ["sequence", "seqstarts", "start_pos", "max_seqlen"]
     n = node("PositionIndex", names, ["position_idx"], name="posidx", domain=DB)
     return model([n], _inputs(names), [value_info("position_idx", INT64, ["s"])], [("", 11), (DB, 1)])
+
+
+def attention_fp32_model(head_dim, rank=3, opset=11):
+    """The attention subgraph the x86 engine runs per sequence, fp32: Transpose(K) -> MatMul(Q, K^T) -> Mul by the
+    initializer 1/sqrt(head_dim) -> Add of an additive mask -> Softmax over the keys -> MatMul with V.
+    rank 3: query / key / value [heads, L, head_dim]; rank 4: [kv_heads, heads per kv head | 1, L, head_dim] (MatMul's
+    batch broadcasting shares a kv head among its query heads). mask [Lq, Lk], -inf where a query must not look."""
+    lead = ["h"] if rank == 3 else ["g", "r"]
+    perm = list(range(rank - 2)) + [rank - 1, rank - 2]
+    nodes = [
+        node("Transpose", ["key"], ["key_t"], name="transpose_k", attrs=[attr_ints("perm", perm)]),
+        node("MatMul", ["query", "key_t"], ["scores"], name="qk"),
+        node("Mul", ["scores", "scale"], ["scaled"], name="scale_scores"),
+        node("Add", ["scaled", "mask"], ["masked"], name="add_mask"),
+        node("Softmax", ["masked"], ["probs"], name="softmax", attrs=[attr_int("axis", -1)]),
+        node("MatMul", ["probs", "value"], ["attn_output"], name="pv"),
+    ]
+    ins = [value_info("query", FLOAT, lead + ["lq", head_dim]), value_info("key", FLOAT, lead + ["lk", head_dim]),
+           value_info("value", FLOAT, lead + ["lk", head_dim]), value_info("mask", FLOAT, ["lq", "lk"])]
+    outs = [value_info("attn_output", FLOAT, lead + ["lq", head_dim])]
+    scale = initializer("scale", FLOAT, [], struct.pack("<f", 1.0 / (head_dim ** 0.5)))
+    return model(nodes, ins, outs, [("", opset)], graph_name="attention_fp32", initializers=[scale])

@@ -83,6 +83,8 @@ def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
     (lambda a: setattr(a, "layer_idx", 5), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "decoding_batches", 3), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "cache_stride_s", 100), cabi.RC_INVALID_VALUE),
+    # offsets inside a stage / tile are 32-bit in the kernels: a token stride of 2^25 elements or more is refused
+    (lambda a: setattr(a, "cache_stride_s", 1 << 25), cabi.RC_UNSUPPORTED),
     (lambda a: setattr(a, "d_query", None), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "specify_decoding_attn_split_k", 7), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "specify_decoding_attn_tpb", 128), cabi.RC_INVALID_VALUE),
@@ -138,6 +140,17 @@ def test_cache_prefill_plan_stages_large_chunks_only(hiplib):
     assert small.prefill_staging == 0 and small.workspace_bytes == small0.workspace_bytes
     _, huge = plan_of([1, 1, 512, 300] + [300] * 30, [100, 900, 16384, 0] + [0] * 30, 2, 1)  # 32 x 16896 rows x 4 KB > 1 GiB
     assert huge.prefill_staging == 0
+
+
+def test_prepare_accepts_plane_strides_beyond_32_bits(hiplib):
+    """cache_layout 3 puts KVH * MaxT * Dh elements between the K and the V plane (multi_head_cache_attention_kernel.cc:
+    149-155): more than 4 GiB with a large slab. The kernels carry that distance in 64 bits, so prepare accepts it;
+    only the distance between two tokens is limited."""
+    a, plan = _valid_args(), cabi.MhcaPlan()
+    a.cache_stride_kv, a.cache_stride_l, a.cache_stride_h, a.cache_stride_s = 1 << 33, 1 << 34, 1 << 30, 128
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
+    a.cache_stride_s = (1 << 25) - 16
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS
 
 
 def test_prepare_accepts_paged_cache(hiplib):

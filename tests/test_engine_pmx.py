@@ -11,7 +11,7 @@ import struct
 import pytest
 
 import harness
-import onnx_writer as ow
+from ppl_nn_amd import onnx_writer as ow
 from harness import cabi
 
 # union OpParamType tags and field lists (name, kind) in schema order: llm_cuda_op_params.fbs:14-23, 31-37, 60-67, 75-88

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import harness
-import onnx_writer as ow
+from ppl_nn_amd import onnx_writer as ow
 from harness import cabi, workloads
 
 pytestmark = pytest.mark.gpu
