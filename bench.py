@@ -133,14 +133,44 @@ def timed(db, steps, warmup):
     return wall, e0.elapsed_time(e1) / steps
 
 
-def cpu_baseline(db, min_seconds=10.0, max_prepare=24):
-    """The decode part run through the x86-engine-semantics attention (fp32 MatMul/Mul/Softmax/MatMul, OpenMP over
-    heads) on the host cores, on dequantised K/V copied from the slab. A bounded sample: the first `max_prepare`
-    decode sequences, repeated until about `min_seconds` of CPU work has been timed."""
-    import oracle
-    L = oracle.lib()
+def timed_robust(step, min_warmup=20, min_iters=100, min_ms=200.0, batches=10):
+    """For the secondary figures: at least `min_warmup` untimed calls, then at least `min_iters` calls and `min_ms` of
+    device time whatever --steps says, timed with events on the launch stream in `batches` equal batches.
+    Returns (mean ms per call, median over the batches of ms per call, calls timed)."""
+    import torch
+    for i in range(min_warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    probe = max(min_iters // batches, 1)
+    e0.record()
+    for i in range(probe):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    per_call = max(e0.elapsed_time(e1) / probe, 1e-4)
+    per_batch = max(-(-min_iters // batches), int(min_ms / per_call / batches) + 1)
+    times = []
+    k = 0
+    for _ in range(batches):
+        e0.record()
+        for _ in range(per_batch):
+            step(k)
+            k += 1
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) / per_batch)
+    return float(np.mean(times)), float(np.median(times)), per_batch * batches
+
+
+def cpu_baseline(db, threads, min_seconds=10.0, max_prepare=24):
+    """The decode part run through the x86 engine on the host cores: per sequence the fp32 ONNX attention subgraph
+    (Transpose, MatMul, Mul, Add of a mask, Softmax, MatMul) over the sequence's dequantised K/V, loaded by the engine
+    library's ONNX reader -- PPLNN-x86-semantics baseline with this build's own kernels (the reference's x86 arithmetic
+    lives in its un-vendored ppl.kernel.cpu). A bounded sample: the first `max_prepare` decode sequences, repeated
+    until about `min_seconds` of CPU work has been timed, once with `threads` OpenMP threads and once with 1."""
+    from ppl_nn_amd import x86_baseline
     b = db.b
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
     cache, scale = db.slabs[0]
     n = min(b.decoding_batches, max_prepare)
     cases = []
@@ -152,23 +182,51 @@ def cpu_baseline(db, min_seconds=10.0, max_prepare=24):
         v = deq[:, 1].permute(1, 0, 2).contiguous().cpu().numpy()
         s0 = int(b.seqstarts[i])
         q = db.q[s0:s0 + 1].float().permute(1, 0, 2).contiguous().cpu().numpy()  # [H, 1, Dh]
-        cases.append((q, k, v, np.empty_like(q), kv))
-    done_tokens, spent, passes = 0, 0.0, 0
-    while spent < min_seconds:
-        t0 = time.perf_counter()
-        for q, k, v, out, kv in cases:
-            rc = L.oracle_x86_attention(q.ctypes.data, k.ctypes.data, v.ctypes.data, None, out.ctypes.data,
-                                        b.num_heads, b.num_kv_heads, 1, kv, b.head_dim, cores)
-            assert rc == 0
-        dt = time.perf_counter() - t0
-        if passes > 0:  # the first pass warms caches and the OpenMP pool
-            spent += dt
-            done_tokens += len(cases)
-        passes += 1
-    return dict(value=done_tokens / spent, unit="tokens/s", cores=cores, kind="port",
-                sample=f"first {n} of {b.decoding_batches} decode sequences of the workload x {passes - 1} passes, "
-                       f"fp32 x86-engine-semantics attention (MatMul-Mul-Softmax-MatMul, OpenMP over heads) on "
-                       f"dequantised K/V resident in host memory, {spent:.1f} s of CPU work")
+        cases.append((q, k, v, x86_baseline.causal_mask(1, kv)))
+
+    def measure(nthreads, seconds):
+        ab = x86_baseline.AttentionBaseline(b.head_dim, num_threads=nthreads)
+        done, spent, passes = 0, 0.0, 0
+        while spent < seconds:
+            t0 = time.perf_counter()
+            for q, k, v, m in cases:
+                ab.run(q, k, v, m)
+            dt = time.perf_counter() - t0
+            if passes > 0:  # the first pass warms caches and the OpenMP pool
+                spent += dt
+                done += len(cases)
+            passes += 1
+        used = ab.num_threads
+        ab.close()
+        return done / spent, used, passes - 1, spent
+
+    rate, used, passes, spent = measure(threads, min_seconds)
+    rate1, _, passes1, spent1 = measure(1, min_seconds / 2)
+    return dict(value=rate, unit="tokens/s", cores=used, kind="port", value_1_thread=rate1,
+                host_cpus=os.cpu_count(), engine="x86 (own fp32 kernels behind the engine boundary)",
+                sample=f"first {n} of {b.decoding_batches} decode sequences of the workload x {passes} passes "
+                       f"({spent:.1f} s) with {used} threads, x {passes1} passes ({spent1:.1f} s) with 1 thread; per "
+                       f"sequence the ONNX subgraph Transpose-MatMul-Mul-Add-Softmax-MatMul in fp32 on dequantised K/V "
+                       f"resident in host memory")
+
+
+def mfma_sustained(lib, pkg):
+    """TFLOP/s of a bare v_mfma_f32_32x32x16_f16 loop on the whole chip, with all-zero and with random fp16 operands:
+    the clock the chip holds depends on how many operand bits toggle."""
+    import torch
+    out = {}
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    dst = torch.empty(1024 * 256, dtype=torch.float32, device="cuda")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    for name, ops in (("zeros", torch.zeros(2048 * 8, dtype=torch.float16, device="cuda")),
+                      ("random_normal", torch.randn(2048 * 8, generator=g, dtype=torch.float16, device="cuda"))):
+        flops = C.c_double()
+        call = lambda i: pkg.check(lib.pplhip_probe_mfma_f16(C.c_void_p(ops.data_ptr()), C.c_void_p(dst.data_ptr()),
+                                                              1024, 2000, C.byref(flops), stream), "probe")
+        mean_ms, med_ms, _ = timed_robust(call, min_warmup=3, min_iters=10, min_ms=100.0, batches=5)
+        out[name] = flops.value / (med_ms * 1e-3) / 1e12
+    return out
 
 
 PROFILE_TRAFFIC = os.path.join(ROOT, "profiles", "decode_int8kv_cfg2_hbm_traffic.txt")
@@ -283,6 +341,8 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
+    # the table rebuild alone (same slot state every call; one workgroup, latency-bound)
+    pack_mean, pack_med, _ = timed_robust(lambda i: lib.pplhip_pack_tables(C.byref(calls[-1][0]), stream), min_ms=50.0)
     timed = host[warm_steps:]
     dec_tokens = sum(h["nd"] for h in timed)
     dec_bytes = sum(h["dec_kv"] for h in timed) * 2.5 * KVH * Dh
@@ -291,7 +351,8 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
     assert np.array_equal(slot_kv.cpu().numpy(), host[-1]["kv"] + host[-1]["nl"]), "slot state diverged"
     return {"workload": "cfg4 churn: 256 slots x %d steps, H=KVH=40, Dh 128, retire p=0.02, prompts U[32,512], tables "
                         "rebuilt on the GPU every step" % steps,
-            "ms_per_step": ms, "decode_tokens_per_s": dec_tokens / (ms * steps * 1e-3),
+            "ms_per_step": ms, "pack_tables_us": {"mean": pack_mean * 1e3, "median": pack_med * 1e3},
+            "decode_tokens_per_s": dec_tokens / (ms * steps * 1e-3),
             "decode_kv_GB_per_step": dec_bytes / steps / 1e9, "prefill_GFLOP_per_step": flops / steps / 1e9,
             "decode_GBps_if_step_were_decode_only": dec_bytes / (ms * steps * 1e-3) / 1e9}
 
@@ -326,6 +387,7 @@ def main():
 
     dec = DeviceBatch(pkg, lib, dec_b, seed=1, n_slabs=N_SLABS, split_k=args.split_k)
     wall_ms, ev_ms = timed(dec, args.steps, args.warmup)
+    _, dec_med_ms, dec_n = timed_robust(dec.step)
     nd = dec_b.decoding_batches
     dec_bytes = dec_b.decode_bytes()
     gbs = dec_bytes / (ev_ms * 1e-3) / 1e9
@@ -348,36 +410,55 @@ def main():
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": recorded_traffic(args.workload),
                      "kernel": "decode_int8kv_kernel (reads the int8 slab once, quantises the new tokens into it) + decode_merge in the same call",
-                     "algorithmic_bytes_per_launch": dec_bytes, "event_ms_per_launch": ev_ms},
+                     "algorithmic_bytes_per_launch": dec_bytes, "event_ms_per_launch": ev_ms,
+                     "median_ms_per_launch_long_run": dec_med_ms, "long_run_calls": dec_n,
+                     "traffic_source": "recorded rocprofv3 --pmc summary under profiles/ (not re-measured in this run)"},
     }
+    def frac(tflops):
+        return tflops / MFMA_FP16_PEAK_TFLOPS
+
+    sustained = mfma_sustained(lib, pkg) if pre_b is not None else None
+    if sustained:
+        result["mfma_f16_sustained_tflops"] = dict(
+            sustained, note="bare v_mfma_f32_32x32x16_f16 loop on all CUs, measured in this run; the published peak is "
+                            "%.0f" % MFMA_FP16_PEAK_TFLOPS)
+
+    def prefill_entry(db, bb, extra=None):
+        mean_ms, med_ms, n = timed_robust(db.step)
+        fl = bb.prefill_flops()
+        tf = fl / (med_ms * 1e-3) / 1e12
+        e = {"tflops": tf, "ms": med_ms, "ms_mean": mean_ms, "calls_timed": n, "flops": fl,
+             "frac_of_fp16_mfma_peak": frac(tf), "peak_tflops": MFMA_FP16_PEAK_TFLOPS}
+        if sustained:
+            e["frac_of_sustained_mfma_random_operands"] = tf / sustained["random_normal"]
+        e.update(extra or {})
+        return e
+
     if pre_b is not None:
         pre = DeviceBatch(pkg, lib, pre_b, seed=2, n_slabs=1)
-        _, pre_ms = timed(pre, max(args.steps // 2, 10), max(args.warmup // 2, 3))
-        fl = pre_b.prefill_flops()
-        result["prefill"] = {"tflops": fl / (pre_ms * 1e-3) / 1e12, "ms": pre_ms, "flops": fl,
-                             "frac_of_fp16_mfma_peak": fl / (pre_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
-                             "peak_tflops": MFMA_FP16_PEAK_TFLOPS, "prefill_seqs": pre_b.batch,
-                             "prefill_tokens": pre_b.total_new_tokens}
+        result["prefill"] = prefill_entry(pre, pre_b, {"prefill_seqs": pre_b.batch, "prefill_tokens": pre_b.total_new_tokens})
         del pre
         mixed = DeviceBatch(pkg, lib, full, seed=3, n_slabs=N_SLABS)
-        _, mix_ms = timed(mixed, max(args.steps // 2, 10), max(args.warmup // 2, 3))
-        result["fused_mixed_call_ms"] = mix_ms
+        mix_mean, mix_med, _ = timed_robust(mixed.step)
+        result["fused_mixed_call_ms"] = mix_med
+        result["fused_mixed_call_ms_mean"] = mix_mean
         del mixed
     if args.workload == "cfg2" and not args.no_churn:
         del dec.slabs[1:], dec.args[1:]
         torch.cuda.empty_cache()
         result["churn_cfg4"] = churn_cfg4(pkg, lib)
     if args.workload == "cfg2" and not args.no_other_configs:
-        # the other decode configurations at their full sizes, same timing loop, shorter runs
+        # the other decode configurations at their full sizes
         others = {}
         for name, ob in (("cfg1 Llama-2-7B pure decode (H32/KVH32/Dh128): 64 seqs kv~U[128,2048]",
                           workloads.cfg1_llama2_7b_decode()),
                          ("cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]",
                           workloads.cfg3_long_context())):
             odb = DeviceBatch(pkg, lib, ob, seed=4, n_slabs=N_SLABS)
-            o_wall, o_ev = timed(odb, max(args.steps // 2, 10), max(args.warmup // 2, 3))
-            o_gbs = ob.decode_bytes() / (o_ev * 1e-3) / 1e9
-            others[name] = {"tokens_per_s": ob.decoding_batches / (o_wall * 1e-3), "ms_per_step": o_wall,
+            o_mean, o_med, o_n = timed_robust(odb.step)
+            o_gbs = ob.decode_bytes() / (o_med * 1e-3) / 1e9
+            others[name] = {"tokens_per_s": ob.decoding_batches / (o_med * 1e-3), "ms_per_step": o_med,
+                            "ms_per_step_mean": o_mean, "calls_timed": o_n,
                             "achieved_GBs": o_gbs, "frac_of_hbm_peak": o_gbs / HBM_PEAK_GBS,
                             "kv_tokens": int(ob.kvlens.sum()), "decode_ranges": int(odb.plan.decode_num_ranges)}
             del odb
@@ -387,29 +468,24 @@ def main():
         import numpy as _np
         lb = workloads.Batch(32, 8, 128, _np.full(4, 8192, _np.int64), _np.zeros(4, _np.int64), 0, name="4x8192 prefill")
         ldb = DeviceBatch(pkg, lib, lb, seed=5, n_slabs=1)
-        _, l_ms = timed(ldb, 5, 2)
-        lfl = lb.prefill_flops()
-        result["prefill_long_prompts"] = {"workload": "4 prompts x 8192 tokens, H32/KVH8/Dh128, causal, incl. quantize-on-write",
-                                          "tflops": lfl / (l_ms * 1e-3) / 1e12, "ms": l_ms,
-                                          "frac_of_fp16_mfma_peak": lfl / (l_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS}
+        result["prefill_long_prompts"] = prefill_entry(
+            ldb, lb, {"workload": "4 prompts x 8192 tokens, H32/KVH8/Dh128, causal, incl. quantize-on-write"})
         del ldb
         torch.cuda.empty_cache()
         # chunked prefill: every prompt brings a 512-token chunk on top of 4096 tokens already in the int8 slab
         cb = workloads.Batch(32, 8, 128, _np.full(8, 512, _np.int64), _np.full(8, 4096, _np.int64), 0, name="chunked prefill")
         cdb = DeviceBatch(pkg, lib, cb, seed=6, n_slabs=1, cache_prefill=1)
-        _, c_ms = timed(cdb, 10, 2)
-        cfl = cb.prefill_flops()
-        result["chunked_prefill"] = {"workload": "8 prompts x (4096 cached + 512 new tokens), H32/KVH8/Dh128, cache-prefill "
-                                                 "(quantize-on-write, fp16 staging of the cached K/V, attention)",
-                                     "tflops": cfl / (c_ms * 1e-3) / 1e12, "ms": c_ms,
-                                     "frac_of_fp16_mfma_peak": cfl / (c_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
-                                     "staged": int(cdb.plan.prefill_staging)}
+        result["chunked_prefill"] = prefill_entry(
+            cdb, cb, {"workload": "8 prompts x (4096 cached + 512 new tokens), H32/KVH8/Dh128, cache-prefill "
+                                  "(quantize-on-write, fp16 staging of the cached K/V, attention)",
+                      "staged": int(cdb.plan.prefill_staging)})
         del cdb
         torch.cuda.empty_cache()
     if args.copy_calibration:
         copy_calibration()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(dec)
+        threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        result["cpu_baseline"] = cpu_baseline(dec, threads)
     print(json.dumps(result))
 
 

@@ -326,6 +326,16 @@ pplhip_retcode pplhip_pack_tables(const pplhip_pack_args* args, void* stream);
 pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot_newlen, int32_t num_slots,
                                     void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): enqueues `workgroups` x 4 wavefronts that each issue
+ * `iterations` x 16 independent v_mfma_f32_32x32x16_f16 on the operands at `d_operands` (2048 x 16 bytes of fp16,
+ * device, 16-byte aligned) and write one float per lane to `d_out` (workgroups x 256 floats). `*flops` (host, may be
+ * NULL) receives the floating-point operations of the launch. Timing it gives the matrix-core rate this chip sustains
+ * for THAT operand data: with random operands the clock is held well below the one the published peak assumes.
+ */
+pplhip_retcode pplhip_probe_mfma_f16(const void* d_operands, void* d_out, int32_t workgroups, int32_t iterations,
+                                     double* flops, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

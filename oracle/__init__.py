@@ -41,7 +41,5 @@ def lib():
         L.oracle_kv_cache_forward.restype = C.c_int
         L.oracle_pack_tables.argtypes = [vp]
         L.oracle_pack_tables.restype = C.c_int
-        L.oracle_x86_attention.argtypes = [vp, vp, vp, vp, vp, C.c_int, C.c_int, i64, i64, C.c_int, C.c_int]
-        L.oracle_x86_attention.restype = C.c_int
         _LIB = L
     return _LIB

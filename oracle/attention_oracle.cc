@@ -26,7 +26,6 @@
 //   oracle_position_index  pinned by a Python loop.
 //   oracle_kv_cache_forward pinned by |dequant(quant(x)) - x| <= scale/2 and row-order checks.
 //   oracle_pack_tables     pinned against a brute-force Python loop written from generation_state.cc.
-//   oracle_x86_attention   pinned against the same float64 textbook routine.
 
 #include "../include/ppl_llm_kernel_hip.h"
 #include "fp16_soft.h"
@@ -423,54 +422,6 @@ int oracle_pack_tables(const pplhip_pack_args* a) {
     a->d_header[3] = max_kv;
     a->d_header[4] = a->d_seqstarts[b];
     a->d_header[5] = a->d_kvstarts[b];
-    return PPLHIP_RC_SUCCESS;
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// CPU baseline with the x86 engine's op semantics: the ONNX subgraph
-//     MatMul(Q, K^T) -> Mul(1/sqrt(d)) -> Add(mask) -> Softmax(axis -1) -> MatMul(., V)
-// in fp32 NDARRAY, one head at a time ([heads, Lq, d] x [heads, d, Lk]); wrappers being restated:
-// src/ppl/nn/engines/x86/kernels/onnx/matmul_kernel.cc:44-52, add_kernel.cc:64-71, softmax_kernel.cc:41-56
-// (axis -1 default for opset >= 13: src/ppl/nn/models/onnx/parsers/onnx/parse_softmax_param.cc:29). The arithmetic
-// of those ops is in the un-vendored ppl.kernel.cpu; these are plain loops, threaded over heads with OpenMP the way
-// `pplnn --num-threads` threads the x86 engine (tools/pplnn.cc:332,377-380).
-// q [heads, Lq, d], k [kv_heads, Lk, d], v [kv_heads, Lk, d], mask [Lq, Lk] additive (may be NULL), out [heads, Lq, d].
-int oracle_x86_attention(const float* q, const float* k, const float* v, const float* mask, float* out, int heads,
-                         int kv_heads, int64_t Lq, int64_t Lk, int d, int num_threads) {
-    if (heads % kv_heads) return PPLHIP_RC_INVALID_VALUE;
-    const int rep = heads / kv_heads;
-    const float sm = 1.0f / sqrtf((float)d);
-    (void)num_threads;
-#pragma omp parallel for num_threads(num_threads > 0 ? num_threads : 1) schedule(dynamic, 1)
-    for (int h = 0; h < heads; ++h) {
-        const float* qh = q + (int64_t)h * Lq * d;
-        const float* kh = k + (int64_t)(h / rep) * Lk * d;
-        const float* vh = v + (int64_t)(h / rep) * Lk * d;
-        float* oh = out + (int64_t)h * Lq * d;
-        std::vector<float> s((size_t)Lk);
-        for (int64_t i = 0; i < Lq; ++i) {
-            float m = -INFINITY;
-            for (int64_t j = 0; j < Lk; ++j) { // MatMul + Mul + Add
-                float acc = 0.f;
-                for (int c = 0; c < d; ++c) acc += qh[i * d + c] * kh[j * d + c];
-                acc *= sm;
-                if (mask) acc += mask[i * Lk + j];
-                s[j] = acc;
-                m = std::max(m, acc);
-            }
-            float l = 0.f; // Softmax along the last axis
-            for (int64_t j = 0; j < Lk; ++j) {
-                s[j] = expf(s[j] - m);
-                l += s[j];
-            }
-            const float inv = 1.0f / l;
-            for (int c = 0; c < d; ++c) oh[i * d + c] = 0.f;
-            for (int64_t j = 0; j < Lk; ++j) { // MatMul with V
-                const float pj = s[j] * inv;
-                for (int c = 0; c < d; ++c) oh[i * d + c] += pj * vh[j * d + c];
-            }
-        }
-    }
     return PPLHIP_RC_SUCCESS;
 }
 
