@@ -241,9 +241,15 @@ pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* args, void* stream);
  * src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/rotary_position_embedding_kernel.cc:110-132.
  *   query / rotated_query  fp16 [total_tokens, num_heads, head_dim]
  *   key   / rotated_key    fp16 [total_tokens, num_key_heads, head_dim]     (outputs may alias the inputs)
- * Token t of sequence b has position start_pos[b] + (t - seqstarts[b]); channel pair (2i, 2i+1), 2i < rotary_dim,
- * is rotated by position * theta^(-2i / rotary_dim):
- *     y[2i] = x[2i] cos - x[2i+1] sin,   y[2i+1] = x[2i+1] cos + x[2i] sin;
+ * Token t of sequence b has position start_pos[b] + (t - seqstarts[b]); pair i (0 <= i < rotary_dim / 2) of a head row
+ * is rotated by the angle position * theta^(-2i / rotary_dim):
+ *     y[lo] = x[lo] cos - x[hi] sin,   y[hi] = x[hi] cos + x[lo] sin.
+ * Which two channels form pair i is `pair_layout` (the reference's CUDA kernel is not in its tree, so neither
+ * convention can be pinned against it; an integrator picks the one the model was exported for):
+ *     PPLHIP_ROPE_PAIRS_INTERLEAVED  (lo, hi) = (2i, 2i + 1)               -- complex-number layout of the original
+ *                                                                              LLaMA weights
+ *     PPLHIP_ROPE_PAIRS_HALF_SPLIT   (lo, hi) = (i, i + rotary_dim / 2)    -- "rotate_half" layout of weights whose
+ *                                                                              q/k projections were permuted for it
  * channels >= rotary_dim are copied; `bypass_key` copies the key unrotated. rotary_dim 0 means head_dim.
  * scaling_type: the values of RotaryPositionEmbeddingParam (src/ppl/nn/params/opmx/rotary_position_embedding_param.h:
  * 12-16). LINEAR divides the position by scaling_factor. DYNAMIC, for a sequence whose total length
@@ -252,8 +258,14 @@ pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* args, void* stream);
  * (The reference wrapper maps the three values through an inverted `!=` chain at
  * rotary_position_embedding_kernel.cc:99-108, which sends NONE to LINEAR and everything else to NONE; this library
  * takes the value at its name.)
- * head_dim and rotary_dim must be multiples of 8, head_dim <= 2048.
+ * head_dim and rotary_dim must be multiples of 8, head_dim <= 2048; the half-split layout needs rotary_dim to be a
+ * multiple of 16 and head_dim <= 512.
  */
+enum {
+    PPLHIP_ROPE_PAIRS_INTERLEAVED = 0,
+    PPLHIP_ROPE_PAIRS_HALF_SPLIT = 1
+};
+
 enum {
     PPLHIP_ROPE_SCALING_NONE = 0,
     PPLHIP_ROPE_SCALING_LINEAR = 1,
@@ -268,7 +280,7 @@ typedef struct pplhip_rope_args {
     float theta;
     int32_t bypass_key;
     int32_t rotary_dim;
-    int32_t reserved;
+    int32_t pair_layout; /* PPLHIP_ROPE_PAIRS_* */
     int64_t batch;
     int64_t total_tokens; /* = seqstarts[batch] = dim 0 of query and key */
     int32_t num_heads;

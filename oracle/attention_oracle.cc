@@ -301,12 +301,16 @@ int oracle_mha_forward(const pplhip_mha_args* a, double* out_f64) {
 
 // RotaryPositionEmbedding over a ragged batch, float64 throughout, one rounding to binary16 at the end.
 // Argument meaning follows src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/
-// rotary_position_embedding_kernel.cc:110-132; the pair convention (consecutive channels rotate together, angle
-// position * theta^(-2i/rotary_dim)) and the linear / dynamic-NTK position scaling restate the published
-// algorithm of the absent kernel library: parity unpinned against its exact bits.
+// rotary_position_embedding_kernel.cc:110-132; the angle position * theta^(-2i/rotary_dim) of pair i and the linear /
+// dynamic-NTK position scaling restate the published algorithm of the absent kernel library; which channels form a
+// pair (consecutive, or i with i + rotary_dim/2) is the caller's pair_layout: parity unpinned against the absent
+// kernel's exact bits and against its choice of layout.
 int oracle_rope_forward(const pplhip_rope_args* a) {
     const int Dh = a->head_dim, rd = a->rotary_dim == 0 ? Dh : a->rotary_dim;
     if (Dh <= 0 || rd % 2 || rd > Dh) return PPLHIP_RC_INVALID_VALUE;
+    if (a->pair_layout != PPLHIP_ROPE_PAIRS_INTERLEAVED && a->pair_layout != PPLHIP_ROPE_PAIRS_HALF_SPLIT)
+        return PPLHIP_RC_INVALID_VALUE;
+    const bool half_split = a->pair_layout == PPLHIP_ROPE_PAIRS_HALF_SPLIT;
     const uint16_t* Q = (const uint16_t*)a->d_query;
     const uint16_t* K = (const uint16_t*)a->d_key;
     uint16_t* QO = (uint16_t*)a->d_rotated_query;
@@ -331,18 +335,16 @@ int oracle_rope_forward(const pplhip_rope_args* a) {
                 const bool bypass = which && a->bypass_key;
                 for (int h = 0; h < heads; ++h) {
                     const int64_t off = ((s0 + t) * heads + h) * Dh;
-                    for (int i = 0; i < Dh / 2; ++i) {
-                        const uint16_t r0 = src[off + 2 * i], r1 = src[off + 2 * i + 1];
-                        if (bypass || 2 * i >= rd) {
-                            dst[off + 2 * i] = r0;
-                            dst[off + 2 * i + 1] = r1;
-                            continue;
-                        }
+                    for (int c = 0; c < Dh; ++c) dst[off + c] = src[off + c]; // channels past rotary_dim, bypassed keys
+                    if (bypass) continue;
+                    for (int i = 0; i < rd / 2; ++i) {
+                        // pair i: consecutive channels, or channel i with channel i + rotary_dim / 2
+                        const int lo = half_split ? i : 2 * i, hi = half_split ? i + rd / 2 : 2 * i + 1;
                         const double ang = pos * pow(theta, -2.0 * i / (double)rd);
                         const double c = cos(ang), sn = sin(ang);
-                        const double x0 = half_to_float(r0), x1 = half_to_float(r1);
-                        dst[off + 2 * i] = float_to_half((float)(x0 * c - x1 * sn));
-                        dst[off + 2 * i + 1] = float_to_half((float)(x1 * c + x0 * sn));
+                        const double x0 = half_to_float(src[off + lo]), x1 = half_to_float(src[off + hi]);
+                        dst[off + lo] = float_to_half((float)(x0 * c - x1 * sn));
+                        dst[off + hi] = float_to_half((float)(x1 * c + x0 * sn));
                     }
                 }
             }

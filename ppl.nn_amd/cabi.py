@@ -91,7 +91,7 @@ class MhaArgs(C.Structure):
 class RopeArgs(C.Structure):
     _fields_ = [
         ("d_query", _p), ("d_key", _p), ("d_start_pos", _p), ("d_seqstarts", _p),
-        ("theta", C.c_float), ("bypass_key", _i32), ("rotary_dim", _i32), ("reserved", _i32),
+        ("theta", C.c_float), ("bypass_key", _i32), ("rotary_dim", _i32), ("pair_layout", _i32),
         ("batch", _i64), ("total_tokens", _i64),
         ("num_heads", _i32), ("num_key_heads", _i32), ("head_dim", _i32), ("max_position_embeddings", _i32),
         ("max_seqlen", _i64),
@@ -100,6 +100,7 @@ class RopeArgs(C.Structure):
     ]
 
 
+ROPE_PAIRS_INTERLEAVED, ROPE_PAIRS_HALF_SPLIT = 0, 1
 ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_DYNAMIC = 0, 1, 2
 
 

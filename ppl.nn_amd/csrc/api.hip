@@ -250,11 +250,19 @@ pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* a, void* stream) {
         a->scaling_type != PPLHIP_ROPE_SCALING_DYNAMIC)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "invalid scaling type: %d", a->scaling_type);
     const int rotary_dim = a->rotary_dim == 0 ? a->head_dim : a->rotary_dim;
+    if (a->pair_layout != PPLHIP_ROPE_PAIRS_INTERLEAVED && a->pair_layout != PPLHIP_ROPE_PAIRS_HALF_SPLIT)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "invalid pair layout: %d", a->pair_layout);
     if (a->head_dim <= 0 || a->head_dim % 8 || a->head_dim > 2048)
         PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 8, at most 2048", a->head_dim);
     if (rotary_dim < 0 || rotary_dim % 8 || rotary_dim > a->head_dim)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "rotary_dim %d: must be a multiple of 8 within head_dim %d", rotary_dim,
                     a->head_dim);
+    if (a->pair_layout == PPLHIP_ROPE_PAIRS_HALF_SPLIT && rotary_dim % 16)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "rotary_dim %d: must be a multiple of 16 for the half-split pair layout",
+                    rotary_dim);
+    // (the two halves of a pair are read and written by lanes of one wavefront, which keeps in-place rotation safe)
+    if (a->pair_layout == PPLHIP_ROPE_PAIRS_HALF_SPLIT && a->head_dim > 512)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: at most 512 for the half-split pair layout", a->head_dim);
     if (a->num_heads <= 0 || a->num_key_heads <= 0)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d / num_key_heads %d", a->num_heads, a->num_key_heads);
     if (!(a->theta > 0.f)) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "theta must be positive");

@@ -4,8 +4,8 @@
 // Both are streaming kernels (HBM roofline): RotaryPositionEmbedding reads and writes every query and key element
 // once, 16 bytes per lane; the angle of a (position, channel pair) is formed in float64 (position * theta^(-2i/d),
 // reduced mod 2*pi before it is narrowed), because a float32 product loses the low bits of a 100k-token position.
-// Pair convention: consecutive channels (x[2i], x[2i+1]) rotate together by position * theta^(-2i / rotary_dim);
-// channels >= rotary_dim pass through.
+// Pair i rotates by position * theta^(-2i / rotary_dim); its two channels are (2i, 2i + 1) or (i, i + rotary_dim / 2),
+// the caller's pair_layout; channels >= rotary_dim pass through.
 #include "common.h"
 
 namespace pplhip {
@@ -21,6 +21,7 @@ struct RopeParams {
     int32_t num_heads, num_key_heads;
     int32_t head_dim, rotary_dim;
     int32_t bypass_key;
+    int32_t half_split; // pairs are (i, i + rotary_dim / 2) instead of (2i, 2i + 1)
     int32_t scaling_type;
     int32_t max_position_embeddings;
     double log2_theta;
@@ -51,18 +52,25 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
             log2_theta += log2(grow) * ((double)p.rotary_dim / (double)(p.rotary_dim - 2));
         }
     }
-    // this lane's 4 channel pairs: 4*chunk .. 4*chunk+3
-    float cs[4], sn[4];
+    // The lane owns the 8 channels 8*chunk .. +7 of every head row it visits. Interleaved layout: they are the 4 whole
+    // pairs 4*chunk .. +3. Half-split layout: they are one half of the 8 pairs (8*chunk mod rotary_dim/2) .. +7, whose
+    // other halves sit rotary_dim/2 channels away (the lane reads them as well; the row is in cache).
     const bool rotate = 8 * chunk < p.rotary_dim; // rotary_dim is a multiple of 8: a chunk is rotated whole or not at all
+    const int half = p.rotary_dim / 2;
+    const bool upper = p.half_split && 8 * chunk >= half;
+    const int npairs = p.half_split ? 8 : 4;
+    const int pair0 = p.half_split ? 8 * chunk - (upper ? half : 0) : 4 * chunk;
+    float cs[8], sn[8];
     if (rotate) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int pair = 4 * chunk + j;
-            const double inv_freq = exp2(-(2.0 * pair / (double)p.rotary_dim) * log2_theta);
-            double a = pos * inv_freq;
-            a -= kTwoPi * rint(a / kTwoPi);
-            cs[j] = cosf((float)a);
-            sn[j] = sinf((float)a);
+        for (int j = 0; j < 8; ++j) {
+            if (j < npairs) {
+                const double inv_freq = exp2(-(2.0 * (pair0 + j) / (double)p.rotary_dim) * log2_theta);
+                double a = pos * inv_freq;
+                a -= kTwoPi * rint(a / kTwoPi);
+                cs[j] = cosf((float)a);
+                sn[j] = sinf((float)a);
+            }
         }
     }
     const int rows = p.num_heads + p.num_key_heads;
@@ -70,16 +78,29 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
         const bool is_key = r >= p.num_heads;
         const int head = is_key ? r - p.num_heads : r;
         const int64_t off = ((t * (is_key ? p.num_key_heads : p.num_heads) + head) * (int64_t)p.head_dim) + 8 * chunk;
-        const uint4 raw = *reinterpret_cast<const uint4*>((is_key ? p.k : p.q) + off);
+        const half_t* src = is_key ? p.k : p.q;
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + off);
         uint4 res = raw;
         if (rotate && !(is_key && p.bypass_key)) {
             half_t x[8], y[8];
             __builtin_memcpy(x, &raw, 16);
+            if (p.half_split) {
+                half_t o[8]; // the other halves of this lane's pairs
+                const uint4 other = *reinterpret_cast<const uint4*>(src + off + (upper ? -half : half));
+                __builtin_memcpy(o, &other, 16);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float x0 = (float)x[2 * j], x1 = (float)x[2 * j + 1];
-                y[2 * j] = (half_t)(x0 * cs[j] - x1 * sn[j]);
-                y[2 * j + 1] = (half_t)(x1 * cs[j] + x0 * sn[j]);
+                for (int j = 0; j < 8; ++j) {
+                    const float mine = (float)x[j], part = (float)o[j];
+                    // lower half: y = x cos - partner sin; upper half: y = x cos + partner sin
+                    y[j] = (half_t)(upper ? mine * cs[j] + part * sn[j] : mine * cs[j] - part * sn[j]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float x0 = (float)x[2 * j], x1 = (float)x[2 * j + 1];
+                    y[2 * j] = (half_t)(x0 * cs[j] - x1 * sn[j]);
+                    y[2 * j + 1] = (half_t)(x1 * cs[j] + x0 * sn[j]);
+                }
             }
             __builtin_memcpy(&res, y, 16);
         }
@@ -111,6 +132,7 @@ pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream) {
     p.head_dim = a->head_dim;
     p.rotary_dim = a->rotary_dim == 0 ? a->head_dim : a->rotary_dim;
     p.bypass_key = a->bypass_key;
+    p.half_split = a->pair_layout == PPLHIP_ROPE_PAIRS_HALF_SPLIT;
     p.scaling_type = a->scaling_type;
     p.max_position_embeddings = a->max_position_embeddings;
     p.log2_theta = log2((double)a->theta);

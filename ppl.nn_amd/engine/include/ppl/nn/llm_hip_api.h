@@ -212,6 +212,10 @@ enum {
     ENGINE_CONF_DECODING_ATTN_SPLIT_K = 1003,
     ENGINE_CONF_DECODING_ATTN_TPB = 1004,
     ENGINE_CONF_CACHE_PREFILL = 1005,
+    /** uint32_t, llm_hip only: which channels RotaryPositionEmbedding rotates together. 0 (default) = consecutive
+        channels (2i, 2i+1); 1 = channel i with channel i + rotary_dim/2 ("rotate_half"). The op has no attribute for
+        it and the reference's kernel is not in its tree, so the integrator states what the checkpoint was exported for */
+    ENGINE_CONF_ROPE_PAIR_LAYOUT = 1006,
     ENGINE_CONF_INTERNAL_MAX,
 };
 

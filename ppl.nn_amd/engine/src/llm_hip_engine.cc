@@ -32,6 +32,9 @@ struct EngineConfig final { // src/ppl/nn/engines/llm_cuda/engine_config.h:25-36
     bool enable_decoding_infinity_gqca = true;
     int32_t specify_decoding_attn_split_k = 1;
     int32_t specify_decoding_attn_tpb = 0;
+    // which channels RotaryPositionEmbedding rotates together (PPLHIP_ROPE_PAIRS_*): not an attribute of the op, so
+    // the integrator states it per engine for the checkpoint family being served
+    int32_t rope_pair_layout = PPLHIP_ROPE_PAIRS_INTERLEAVED;
 };
 
 // ---------------------------------------------------------------- device
@@ -680,6 +683,7 @@ protected:
         a.max_seqlen = max_seqlen_val;
         a.scaling_type = scaling_type;
         a.scaling_factor = param_->scaling_factor;
+        a.pair_layout = GetEngineConfig().rope_pair_layout;
         a.d_rotated_query = rotated_query->GetBufferPtr();
         a.d_rotated_key = rotated_key->GetBufferPtr();
         return (RetCode)CheckKernelRc(pplhip_rope_forward(&a, GetStream()), GetName());
@@ -967,6 +971,16 @@ public:
                 break;
             }
             case ENGINE_CONF_CACHE_PREFILL: config_.enable_cache_prefill = va_arg(args, uint32_t) ? true : false; break;
+            case ENGINE_CONF_ROPE_PAIR_LAYOUT: {
+                const uint32_t v = va_arg(args, uint32_t);
+                if (v != PPLHIP_ROPE_PAIRS_INTERLEAVED && v != PPLHIP_ROPE_PAIRS_HALF_SPLIT) {
+                    LOG(ERROR) << "ENGINE_CONF_ROPE_PAIR_LAYOUT only accept 0/1 but get " << v;
+                    rc = RC_INVALID_VALUE;
+                } else {
+                    config_.rope_pair_layout = (int32_t)v;
+                }
+                break;
+            }
             default:
                 LOG(ERROR) << "invalid option[" << option << "] >= [" << (uint32_t)ENGINE_CONF_INTERNAL_MAX << "]";
                 rc = RC_INVALID_VALUE;

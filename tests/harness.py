@@ -224,7 +224,7 @@ def run_device_mha(b, q, key, value):
 
 
 def fill_rope_args(a, q, k, seqlens, start_pos, q_out, k_out, theta=10000.0, rotary_dim=0, bypass_key=0,
-                   scaling_type=0, scaling_factor=1.0, max_pos=2048, ptr=_ptr, tables=None):
+                   scaling_type=0, scaling_factor=1.0, max_pos=2048, ptr=_ptr, tables=None, pair_layout=0):
     seqlens = np.asarray(seqlens, np.int64)
     ss = np.concatenate([[0], np.cumsum(seqlens)]).astype(np.int64)
     sp = np.asarray(start_pos, np.int64)
@@ -233,7 +233,7 @@ def fill_rope_args(a, q, k, seqlens, start_pos, q_out, k_out, theta=10000.0, rot
     else:
         ss_arg, sp_arg = ss, sp
     a.d_query, a.d_key, a.d_start_pos, a.d_seqstarts = ptr(q), ptr(k), ptr(sp_arg), ptr(ss_arg)
-    a.theta, a.bypass_key, a.rotary_dim = theta, bypass_key, rotary_dim
+    a.theta, a.bypass_key, a.rotary_dim, a.pair_layout = theta, bypass_key, rotary_dim, pair_layout
     a.batch, a.total_tokens = len(seqlens), int(ss[-1])
     a.num_heads, a.num_key_heads, a.head_dim = int(q.shape[1]), int(k.shape[1]), int(q.shape[2])
     a.max_position_embeddings, a.max_seqlen = max_pos, int(seqlens.max()) if len(seqlens) else 0

@@ -121,7 +121,10 @@ def test_engine_configure_like_the_reference(eng):
     assert eng.pplnn_hip_engine_configure_u32(e, 1004, 128) == cabi.RC_INVALID_VALUE
     assert eng.pplnn_hip_engine_configure_u32(e, 0, 0) == cabi.RC_UNSUPPORTED  # NCCL comm: one GPU only
     assert eng.pplnn_hip_engine_configure_u32(e, 77, 0) == cabi.RC_INVALID_VALUE
-    assert eng.pplnn_hip_engine_configure_u32(e, 1006, 0) == cabi.RC_INVALID_VALUE
+    # 1006 = ENGINE_CONF_ROPE_PAIR_LAYOUT (this engine's own): 0 consecutive channels, 1 half-split
+    assert eng.pplnn_hip_engine_configure_u32(e, 1006, 1) == 0 and eng.pplnn_hip_engine_configure_u32(e, 1006, 0) == 0
+    assert eng.pplnn_hip_engine_configure_u32(e, 1006, 2) == cabi.RC_INVALID_VALUE
+    assert eng.pplnn_hip_engine_configure_u32(e, 1007, 0) == cabi.RC_INVALID_VALUE
     eng.pplnn_hip_engine_destroy(e)
     assert not eng.pplnn_hip_engine_create(0, 99)  # unknown mm_policy: factories return nullptr on failure
 

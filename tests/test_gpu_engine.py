@@ -233,6 +233,33 @@ def test_rope_then_mhca_graph(hiplib, olib):
     s.close()
 
 
+@pytest.mark.parametrize("layout", [0, 1])
+def test_rope_graph_with_the_engine_pair_layout_option(hiplib, olib, layout):
+    """A RotaryPositionEmbedding node alone: ENGINE_CONF_ROPE_PAIR_LAYOUT (1006) selects consecutive-channel or
+    half-split pairs for every such node of the engine; each must match the oracle run with the same layout."""
+    eng = harness.pkg.load_engine_library()
+    rng = np.random.default_rng(43)
+    seqlens, start = np.array([1, 9, 130], np.int64), np.array([4000, 0, 77], np.int64)
+    T = int(seqlens.sum())
+    q = rng.standard_normal((T, 8, 128)).astype(np.float16)
+    k = rng.standard_normal((T, 2, 128)).astype(np.float16)
+    qo, ko = np.zeros_like(q), np.zeros_like(k)
+    a = harness.fill_rope_args(cabi.RopeArgs(), q, k, seqlens, start, qo, ko, theta=500000.0, pair_layout=layout)
+    assert olib.oracle_rope_forward(C.byref(a)) == 0
+    s = Session(eng, ow.rope_model(ow.rope_attrs(500000.0)), configure=[(1006, layout)])
+    s.set_device_tensor(0, harness.to_dev(q))
+    s.set_device_tensor(1, harness.to_dev(k))
+    s.set_table(2, np.concatenate([[0], np.cumsum(seqlens)]).astype(np.int64))
+    s.set_table(3, start)
+    s.set_host_scalar(4, int(seqlens.max()))
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    for i, want in enumerate((qo, ko)):
+        got = s.output(i, np.float16)
+        ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float64)
+        assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= ulp + 1e-6).all()
+    s.close()
+
+
 def test_kv_cache_then_mha_graph_equals_mhca(hiplib):
     import torch
     eng = harness.pkg.load_engine_library()

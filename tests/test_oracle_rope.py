@@ -10,12 +10,12 @@ from harness import cabi
 
 
 def rope_oracle(olib, q, k, seqlens, start_pos, theta=10000.0, rotary_dim=0, bypass_key=0, scaling_type=0,
-                scaling_factor=1.0, max_pos=2048):
+                scaling_factor=1.0, max_pos=2048, pair_layout=0):
     q, k = np.ascontiguousarray(q), np.ascontiguousarray(k)
     qo, ko = np.zeros_like(q), np.zeros_like(k)
     a = harness.fill_rope_args(cabi.RopeArgs(), q, k, seqlens, start_pos, qo, ko, theta=theta, rotary_dim=rotary_dim,
                                bypass_key=bypass_key, scaling_type=scaling_type, scaling_factor=scaling_factor,
-                               max_pos=max_pos)
+                               max_pos=max_pos, pair_layout=pair_layout)
     assert olib.oracle_rope_forward(C.byref(a)) == 0
     return qo, ko
 
@@ -53,6 +53,52 @@ def test_vs_complex_multiply(olib, rotary_dim, Dh):
         want = numpy_rope(x, pos, 500000.0, rd)
         assert close_f16(got, want)  # float64 on both sides, one rounding
         assert np.array_equal(got[..., rd:], x[..., rd:])  # pass-through channels untouched
+
+
+def numpy_rope_half_split(x, pos, theta, rotary_dim):
+    """The "rotate_half" restatement: y = x * cos + rotate_half(x) * sin over the first rotary_dim channels, with
+    rotate_half(x) = concat(-x[rd/2:], x[:rd/2]) and the angle table repeated for both halves."""
+    x = x.astype(np.float64)
+    out = x.copy()
+    rd = rotary_dim
+    inv = theta ** (-np.arange(0, rd, 2, dtype=np.float64) / rd)
+    ang = pos[:, None].astype(np.float64) * inv[None, :]
+    emb = np.concatenate([ang, ang], axis=-1)[:, None, :]
+    xr = x[..., :rd]
+    rot = np.concatenate([-xr[..., rd // 2:], xr[..., :rd // 2]], axis=-1)
+    out[..., :rd] = xr * np.cos(emb) + rot * np.sin(emb)
+    return out
+
+
+@pytest.mark.parametrize("rotary_dim,Dh", [(0, 128), (64, 128), (0, 64), (32, 80)])
+def test_half_split_layout_vs_rotate_half(olib, rotary_dim, Dh):
+    rng = np.random.default_rng(15)
+    seqlens, start = np.array([1, 5, 1, 17]), np.array([100000, 0, 3, 250])
+    T = int(seqlens.sum())
+    q = rng.standard_normal((T, 6, Dh)).astype(np.float16)
+    k = rng.standard_normal((T, 2, Dh)).astype(np.float16)
+    qo, ko = rope_oracle(olib, q, k, seqlens, start, theta=500000.0, rotary_dim=rotary_dim,
+                         pair_layout=cabi.ROPE_PAIRS_HALF_SPLIT)
+    pos = np.concatenate([s + np.arange(n) for n, s in zip(seqlens, start)])
+    rd = rotary_dim or Dh
+    for got, x in ((qo, q), (ko, k)):
+        assert close_f16(got, numpy_rope_half_split(x, pos, 500000.0, rd))
+        assert np.array_equal(got[..., rd:], x[..., rd:])
+    # the two layouts are the same rotation up to a fixed permutation of the rotated channels:
+    # half-split(x) = P^-1 interleaved(P x), P gathering channels (0, rd/2, 1, rd/2+1, ...)
+    perm = np.arange(rd).reshape(2, rd // 2).T.reshape(-1)
+    qp = q.copy()
+    qp[..., :rd] = q[..., perm]
+    inter, _ = rope_oracle(olib, qp, k, seqlens, start, theta=500000.0, rotary_dim=rotary_dim)
+    back = inter.copy()
+    back[..., perm] = inter[..., :rd]
+    assert np.array_equal(back, qo)
+    # and they differ as functions of an unpermuted input, so a wrong choice cannot pass unnoticed
+    plain, _ = rope_oracle(olib, q, k, seqlens, start, theta=500000.0, rotary_dim=rotary_dim)
+    assert not np.array_equal(plain, qo)
+    # an unknown layout value is refused
+    a = harness.fill_rope_args(cabi.RopeArgs(), q, k, seqlens, start, np.zeros_like(q), np.zeros_like(k), pair_layout=2)
+    assert olib.oracle_rope_forward(C.byref(a)) == cabi.RC_INVALID_VALUE
 
 
 def test_invariants(olib):
