@@ -38,7 +38,13 @@ enum OpParamType : uint8_t {
     OpParamType_MultiHeadCacheAttentionParam = 10,
 };
 
-// ---- writer: one member table of 4-byte and 1-byte scalar fields, wrapped in OpParam
+// ---- writer: one member table of 4-byte and 1-byte scalar fields, wrapped in OpParam. The bytes are laid out the
+// way the reference's serialisers lay them out, i.e. the way flatbuffers::FlatBufferBuilder does when driven by the
+// generated Create*Param / CreateOpParam / FinishOpParamBuffer functions (pmx/generated/
+// llm_cuda_op_params_generated.h:1042-1070, 1545-1553, 1654-1658): the buffer grows downwards; the 4-byte fields are
+// added in reverse schema order, then the 1-byte fields in reverse order; a scalar equal to its default is not
+// written; every write is aligned to its size counted from the END of the buffer; a table ends with its soffset and a
+// vtable just long enough for the highest field present; the root offset comes last, i.e. first in memory.
 class TableWriter final {
 public:
     void AddI32(int field, int32_t v) { if (v != 0) Add(field, &v, 4); }
@@ -46,52 +52,66 @@ public:
     void AddF32(int field, float v) { if (v != 0.0f) Add(field, &v, 4); }
     void AddBool(int field, bool v) { if (v) { uint8_t b = 1; Add(field, &b, 1); } }
 
-    // [root uoffset][OpParam vtable][OpParam table][member vtable][member table]
-    std::string Finish(OpParamType type, int num_fields) const {
-        std::string out;
-        auto put16 = [&](uint16_t v) { out.append((const char*)&v, 2); };
-        auto put32 = [&](uint32_t v) { out.append((const char*)&v, 4); };
-        auto align4 = [&] { while (out.size() & 3) out.push_back(0); };
-        put32(0); // root offset, patched below
-        // OpParam: field 0 = value_type (u8), field 1 = value (uoffset32)
-        const size_t root_vt = out.size();
-        put16(8);
-        put16(12);
-        put16(8); // value_type at table + 8
-        put16(4); // value at table + 4
-        align4();
-        const size_t root_tab = out.size();
-        put32((uint32_t)(int32_t)(root_tab - root_vt));
-        const size_t value_pos = out.size();
-        put32(0); // patched
-        out.push_back((char)type);
-        align4();
-        // member table: 4-byte fields first, then the bools
-        std::vector<uint16_t> offs(num_fields, 0);
-        std::string body(4, '\0'); // soffset placeholder
-        for (int pass = 0; pass < 2; ++pass)
-            for (auto& f : fields_)
-                if ((f.size == 4) == (pass == 0)) {
-                    offs[f.field] = (uint16_t)body.size();
-                    body.append(f.bytes, f.size);
-                }
-        while (body.size() & 3) body.push_back(0);
-        const size_t vt = out.size();
-        put16((uint16_t)(4 + 2 * num_fields));
-        put16((uint16_t)body.size());
-        for (auto o : offs) put16(o);
-        align4();
-        const size_t tab = out.size();
-        const uint32_t so = (uint32_t)(int32_t)(tab - vt);
-        memcpy(&body[0], &so, 4);
-        out += body;
-        const uint32_t rel = (uint32_t)(tab - value_pos), root = (uint32_t)root_tab;
-        memcpy(&out[value_pos], &rel, 4);
-        memcpy(&out[0], &root, 4);
-        return out;
+    std::string Finish(OpParamType type, int /*num_fields*/) const {
+        Down b;
+        // member table
+        uint32_t start = b.Size();
+        for (int size = 4; size >= 1; size -= 3) // 4-byte fields, then 1-byte fields
+            for (int field = 63; field >= 0; --field)
+                for (auto& f : fields_)
+                    if (f.field == field && f.size == size) b.AddElement(4 + 2 * field, f.bytes, size);
+        const uint32_t member = b.EndTable(start);
+        // OpParam { value_type: u8 (slot 4), value: offset (slot 6) }: the offset is added first
+        start = b.Size();
+        const uint32_t rel = b.ReferTo(member);
+        b.AddElement(6, &rel, 4);
+        const uint8_t tag = (uint8_t)type;
+        b.AddElement(4, &tag, 1);
+        const uint32_t root = b.EndTable(start);
+        // Finish(root): pad so that the whole buffer is a multiple of the largest alignment used, then the root offset
+        b.Pad((4 - (b.Size() + 4) % 4) % 4);
+        const uint32_t root_rel = b.ReferTo(root);
+        b.Push(&root_rel, 4);
+        return b.bytes;
     }
 
 private:
+    struct Down final { // bytes written so far, in memory order: a write prepends; offsets count from the end
+        std::string bytes;
+        std::vector<std::pair<int, uint32_t>> slots; // (vtable slot, offset) of the table being built
+        uint32_t Size() const { return (uint32_t)bytes.size(); }
+        void Pad(size_t n) { bytes.insert(0, n, '\0'); }
+        void Align(size_t n) { Pad((n - bytes.size() % n) % n); }
+        uint32_t Push(const void* v, int size) {
+            Align(size);
+            bytes.insert(0, (const char*)v, size);
+            return Size();
+        }
+        void AddElement(int slot, const void* v, int size) { slots.emplace_back(slot, Push(v, size)); }
+        uint32_t ReferTo(uint32_t off) {
+            Align(4);
+            return Size() - off + 4;
+        }
+        uint32_t EndTable(uint32_t start) {
+            const int32_t zero = 0;
+            const uint32_t table = Push(&zero, 4); // soffset, patched below
+            int max_slot = 2;
+            for (auto& s : slots) max_slot = s.first > max_slot ? s.first : max_slot;
+            std::string vt(max_slot + 2, '\0');
+            const uint16_t vt_bytes = (uint16_t)vt.size(), table_bytes = (uint16_t)(table - start);
+            memcpy(&vt[0], &vt_bytes, 2);
+            memcpy(&vt[2], &table_bytes, 2);
+            for (auto& s : slots) {
+                const uint16_t pos = (uint16_t)(table - s.second);
+                memcpy(&vt[s.first], &pos, 2);
+            }
+            bytes.insert(0, vt);
+            slots.clear();
+            const int32_t so = (int32_t)(Size() - table); // the vtable sits right in front of its table
+            memcpy(&bytes[bytes.size() - table], &so, 4);
+            return table;
+        }
+    };
     struct Field {
         int field;
         int size;
