@@ -148,6 +148,18 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* args, const pplhip_mh
                                    void* stream);
 
 /*
+ * pplhip_mhca_forward for callers that cannot allocate device memory or bring a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The split-k
+ * partial results go to an array that is part of the library's device image (16 MiB on every GPU the library runs on,
+ * held until the process ends); the call allocates nothing and frees nothing. Limits: plan->workspace_bytes must not
+ * exceed 16 MiB (PPLHIP_RC_OUT_OF_RANGE otherwise; every configuration named in this header's examples needs under
+ * 7 MiB) and plan->prefill_staging must be 0 (PPLHIP_RC_UNSUPPORTED: staging rows need a caller-owned workspace).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
+ * on it and must be serialised by the caller; calls on different GPUs are independent.
+ */
+pplhip_retcode pplhip_mhca_forward_noalloc(const pplhip_mhca_args* args, const pplhip_mhca_plan* plan, void* stream);
+
+/*
  * Quantize-on-write alone: new token t of sequence b goes to slab token cachestarts[b] + start_pos[b] + t.
  * Per (token, K|V, kv head, group of 8 channels): scale = max(fp16(absmax / 127), fp16(1e-5)),
  * q = int8(rint(fp16(x / scale))). This is the first step of the reference's fused `forward`.

@@ -120,6 +120,7 @@ PROTOTYPES = {
     "pplhip_init": (_i32, []),
     "pplhip_mhca_prepare": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan)]),
     "pplhip_mhca_forward": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan), _p, _p]),
+    "pplhip_mhca_forward_noalloc": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan), _p]),
     "pplhip_mha_forward": (_i32, [C.POINTER(MhaArgs), _p]),
     "pplhip_rope_forward": (_i32, [C.POINTER(RopeArgs), _p]),
     "pplhip_position_index": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),

@@ -18,6 +18,32 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+// Scratch of the entry point that allocates nothing (pplhip_mhca_forward_noalloc): split-k partial results and the
+// per-range first-sequence table of one call. Every GPU the library runs on holds its own copy of the array until the
+// process ends. The name below is a host-side stand-in, not a device address: host code only ever uses the per-device
+// address that hipGetSymbolAddress returned.
+constexpr uint64_t kNoAllocScratchBytes = 16ull << 20;
+static __device__ __align__(256) unsigned char g_noalloc_scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_noalloc_scratch_ptr[kMaxDevices];
+
+// the current device's copy of the scratch array (looked up once per device, with that device current)
+static pplhip_retcode noalloc_scratch_of_current_device(void** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "no current HIP device (or more than %d devices)", kMaxDevices);
+    void* ptr = g_noalloc_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_noalloc_scratch));
+        if (e != hipSuccess || !ptr)
+            PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "cannot locate the scratch array on device %d: %s", dev,
+                        hipGetErrorString(e));
+        g_noalloc_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return PPLHIP_RC_SUCCESS;
+}
+
 // Compute units the decode plan is sized for: MI355X's 256 until pplhip_init() has read the current device's count.
 static std::atomic<int> g_cu_count{256};
 static int device_cu_count() {
@@ -120,7 +146,8 @@ pplhip_retcode pplhip_init(void) {
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
         PPLHIP_FAIL(PPLHIP_RC_DEVICE_RUNTIME_ERROR, "init: no current HIP device");
     if (prop.multiProcessorCount > 0) g_cu_count.store(prop.multiProcessorCount, std::memory_order_relaxed);
-    return PPLHIP_RC_SUCCESS;
+    void* scratch = nullptr; // this device's copy of the no-allocation entry point's scratch array
+    return noalloc_scratch_of_current_device(&scratch);
 }
 
 pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* plan) {
@@ -220,6 +247,24 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
                                                  prefill_writes_new_tokens(a) ? a->decoding_batches : -1);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
     return launch_decode_and_prefill(a, plan, d_workspace, s);
+}
+
+pplhip_retcode pplhip_mhca_forward_noalloc(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* stream) {
+    if (!a || !plan) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    if (plan->workspace_bytes > kNoAllocScratchBytes)
+        PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE,
+                    "this call needs %llu bytes of scratch, the built-in array holds %llu: use pplhip_mhca_forward with "
+                    "a caller-owned workspace", (unsigned long long)plan->workspace_bytes,
+                    (unsigned long long)kNoAllocScratchBytes);
+    if (plan->prefill_staging)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "cache-prefill with fp16 staging rows needs a caller-owned workspace (clear "
+                                           "plan.prefill_staging, or use pplhip_mhca_forward)");
+    void* scratch = nullptr;
+    const pplhip_retcode rc = noalloc_scratch_of_current_device(&scratch);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    // nothing in the scratch has to start at zero: every partial result and table entry a call reads was written by
+    // that call's own decode workgroups
+    return pplhip_mhca_forward(a, plan, scratch, stream);
 }
 
 pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {
