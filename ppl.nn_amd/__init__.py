@@ -10,7 +10,9 @@ from . import cabi
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libppl_llm_kernel_hip.so")
+CONSERVATIVE_WAITS_LIB_PATH = os.path.join(_HERE, "lib", "libppl_llm_kernel_hip_conservative_waits.so")
 _LIB = None
+_CHECK_LIB = None
 
 
 class LibraryMissing(RuntimeError):
@@ -34,6 +36,19 @@ def load_library():
         _LIB = cabi.bind(ctypes.CDLL(LIB_PATH))
         _assert_single_hip_runtime()
     return _LIB
+
+
+def load_conservative_waits_library():
+    """The checking build of the kernel library (every hand-counted wait of the decode kernel replaced by a wait
+    for everything in flight). For tests that compare it bit for bit with the product build; nothing else loads it."""
+    global _CHECK_LIB
+    if _CHECK_LIB is None:
+        if not os.path.exists(CONSERVATIVE_WAITS_LIB_PATH):
+            raise LibraryMissing(f"{CONSERVATIVE_WAITS_LIB_PATH} is not built; run `python __graft_entry__.py`")
+        load_library()
+        _CHECK_LIB = cabi.bind(ctypes.CDLL(CONSERVATIVE_WAITS_LIB_PATH))
+        _assert_single_hip_runtime()
+    return _CHECK_LIB
 
 
 def _assert_single_hip_runtime():

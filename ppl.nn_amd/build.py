@@ -29,9 +29,13 @@ def _newer(target, sources):
     return any(os.path.getmtime(s) > t for s in sources)
 
 
-def build_kernels(force=False, verbose=False):
+def build_kernels(force=False, verbose=False, conservative_waits=False):
+    """The kernel library. conservative_waits: the checking build, in which every hand-counted wait of the decode
+    kernel waits for all memory operations in flight (-DPPLHIP_CONSERVATIVE_WAITS); it exists to be compared
+    bit for bit with the product build and is never what the package loads by default."""
     os.makedirs(LIBDIR, exist_ok=True)
-    out = os.path.join(LIBDIR, "libppl_llm_kernel_hip.so")
+    tag = "_conservative_waits" if conservative_waits else ""
+    out = os.path.join(LIBDIR, f"libppl_llm_kernel_hip{tag}.so")
     srcs = [os.path.join(CSRC, s) for s in KERNEL_SOURCES]
     deps = srcs + [os.path.join(CSRC, s) for s in KERNEL_INCLUDED] + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "exports.map"),
                    os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip.h")]
@@ -40,9 +44,9 @@ def build_kernels(force=False, verbose=False):
     objs = []
     procs = []
     for s in srcs:
-        o = os.path.join(LIBDIR, os.path.basename(s) + ".o")
+        o = os.path.join(LIBDIR, os.path.basename(s) + tag + ".o")
         objs.append(o)
-        cmd = [HIPCC] + HIP_FLAGS + ["-c", s, "-o", o]
+        cmd = [HIPCC] + HIP_FLAGS + (["-DPPLHIP_CONSERVATIVE_WAITS"] if conservative_waits else []) + ["-c", s, "-o", o]
         if verbose:
             print(" ".join(cmd))
         procs.append((s, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -64,6 +68,7 @@ def build_kernels(force=False, verbose=False):
 
 def build_all(force=False, verbose=False):
     build_kernels(force=force, verbose=verbose)
+    build_kernels(force=force, verbose=verbose, conservative_waits=True)
     engine_build = os.path.join(HERE, "engine", "build_engine.py")
     if os.path.exists(engine_build):
         import importlib.util

@@ -206,7 +206,14 @@ __device__ inline void lds_write_b16(uint32_t addr, uint32_t v) {
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at "no wait"), gfx9 encoding
 #define PPLHIP_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | 0x0f70)
 // the same with `extra` (0, 4 or 8: result stores of the previous segment) younger operations more left in flight; the
-// immediate has to be a constant
+// immediate has to be a constant.
+// These counts are kept by hand: `n` is the number of transfers and untracked loads issued after the data that is
+// waited for, `extra` a lower bound on the store instructions issued after those. A build with
+// -DPPLHIP_CONSERVATIVE_WAITS waits for everything in flight instead (slower, no counting to get wrong); its results
+// must be bit-identical, which is what a test of the two builds against each other checks.
+#ifdef PPLHIP_CONSERVATIVE_WAITS
+#define PPLHIP_WAIT_VMCNT_PLUS(n, extra) PPLHIP_WAIT_VMCNT(0)
+#else
 #define PPLHIP_WAIT_VMCNT_PLUS(n, extra)            \
     do {                                            \
         switch (extra) {                            \
@@ -215,6 +222,7 @@ __device__ inline void lds_write_b16(uint32_t addr, uint32_t v) {
             default: PPLHIP_WAIT_VMCNT(n); break;      \
         }                                           \
     } while (0)
+#endif
 // A 16-byte global load the compiler does not track: its waitcnt pass merges what it knows about loads in flight at
 // every loop header, and for the query registers (loaded once per sequence, read by every stage) that put a
 // vmcnt(0) in front of the first MFMA of EVERY stage and another in front of every stage's transfers -- the wave never
@@ -536,7 +544,6 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
         g.tail_rows_mem =
             (int)(((int64_t)g.seg_end - last_stage_t0) < kStageTokens ? ((int64_t)g.seg_end - last_stage_t0) : kStageTokens);
         g.tail_rows_valid = (int)(t_end - last_stage_t0);
-        const int64_t seq_len = seq_hi - seq_lo;
         g.has_new = g.n_stages > 0 && t_end == seq_hi - seq_lo;
         const int64_t row0 = (PAGED ? 0 : (cachestarts[b] + (int64_t)g.t_begin) * (int64_t)stride) + head_off;
         g.cbase = reinterpret_cast<const char*>(p.cache) + row0;

@@ -141,11 +141,12 @@ def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0, staging=None):
+def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0, staging=None, lib=None):
     """Same call through the C ABI on cuda:0. staging=0 clears plan.prefill_staging (the caller's way to keep a
-    cache-prefill call on the kernel that reads the int8 slab itself)."""
+    cache-prefill call on the kernel that reads the int8 slab itself). lib: another build of the kernel library than
+    the product one."""
     import torch
-    lib = pkg.load_library()
+    lib = lib or pkg.load_library()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     cache_h, scale_h = new_slab(b, paged, layout)
     cache, scale = to_dev(cache_h), to_dev(scale_h)
