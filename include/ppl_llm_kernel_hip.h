@@ -78,7 +78,7 @@ typedef struct pplhip_mhca_args {
     const void* d_query;
     const void* d_current_key;
     const void* d_current_value;
-    const void* d_attn_mask; /* additive fp16 mask: must be NULL (no shipped model passes one) */
+    const void* d_attn_mask; /* optional additive fp16 mask (NULL: none), see attn_mask_stride_* below */
     const int64_t* d_seqstarts;
     const int64_t* d_kvstarts;
     const int64_t* d_cachestarts;
@@ -112,6 +112,15 @@ typedef struct pplhip_mhca_args {
     void* d_scale;
     void* d_output;
     int64_t total_new_tokens; /* S = query dim 0 (the reference passes the query TensorShape) */
+    /* attn_mask (the reference passes its TensorShape, …_kernel.cc:105-110,178-179): the value added to the scaled score
+     * of query token t (of sequence b, head h) and key j of that sequence is
+     *     mask[h * attn_mask_stride_h + (seqstarts[b] + t) * attn_mask_stride_q + kvstarts[b] + j]
+     * i.e. a [S, >= kvstarts[batch]] matrix over packed query tokens x packed keys (stride_q = its last extent, which
+     * exporters pad to a multiple of 8), one per head or, with attn_mask_stride_h == 0, one for all heads. It is
+     * applied in addition to is_causal. -inf entries mask a key out; a row with every key masked yields zeros.
+     * The layout is this library's definition: the reference's CUDA kernel, which would fix it, is not in its tree. */
+    int64_t attn_mask_stride_h;
+    int64_t attn_mask_stride_q;
 } pplhip_mhca_args;
 
 /* What `heuristic_prepare` stores in the reference kernel object's `.cfg` (…_kernel.cc:218-228 reads
@@ -129,7 +138,9 @@ typedef struct pplhip_mhca_plan {
                                 attention kernel dequantises the int8 slab itself (small chunks, or staging too large).
                                 The caller may clear it before forward to stay on the second route. */
     int32_t prefill_staging_offset_256; /* where the staging rows start in the workspace, in units of 256 bytes */
-    int32_t reserved[1];
+    int32_t general_kernel; /* 1 = the call runs the general attention kernel (head_dim other than 128, more than 16
+                               query heads per kv head, or an attn_mask): write kernel + one attention launch, no
+                               workspace */
 } pplhip_mhca_plan;
 
 /* Host-only: validates `args` exactly like the reference wrapper + kernel library would
@@ -223,13 +234,14 @@ pplhip_retcode pplhip_kv_cache_forward(const pplhip_kv_cache_args* args, void* s
  * The queries of a sequence are its LAST seqlen keys: with is_causal, query i of sequence b attends to keys
  * 0 .. (kvlen_b - seqlen_b) + i; without, to all kvlen_b keys. kvlen_b >= seqlen_b >= 1 is required.
  * MultiHeadCacheAttention == MultiHeadAttention applied to the outputs of KeyValueCache.
- * Same limits as above: head_dim 128, at most 16 query heads per kv head, no attn_mask, no alibi.
+ * head_dim: a multiple of 32 up to 256 (128 with at most 16 query heads per kv head and no mask runs the tuned kernel,
+ * everything else the general one); no alibi.
  */
 typedef struct pplhip_mha_args {
     const void* d_query;
     const void* d_key;
     const void* d_value;
-    const void* d_attn_mask; /* must be NULL */
+    const void* d_attn_mask; /* optional additive fp16 mask, laid out as for pplhip_mhca_args */
     const int64_t* d_seqstarts; /* [batch+1] */
     const int64_t* d_kvstarts; /* [batch+1] */
     int32_t is_causal;
@@ -243,6 +255,8 @@ typedef struct pplhip_mha_args {
     int32_t head_dim;
     int32_t reserved;
     void* d_output;
+    int64_t attn_mask_stride_h;
+    int64_t attn_mask_stride_q;
 } pplhip_mha_args;
 
 pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* args, void* stream);

@@ -141,6 +141,13 @@ void oracle_kv_dequant_groups(const int8_t* q, const uint16_t* scale, float* out
         for (int i = 0; i < kGroup; ++i) out[g * kGroup + i] = (float)q[g * kGroup + i] * half_to_float(scale[g]);
 }
 
+// The additive attention mask (null: none): the entry for head h, packed query token `qtok` and packed key `key`.
+// Layout as the C ABI header defines it for pplhip_mhca_args.
+static inline double mask_value(const uint16_t* mask, int64_t stride_h, int64_t stride_q, int h, int64_t qtok,
+                                int64_t key) {
+    return mask ? (double)half_to_float(mask[h * stride_h + qtok * stride_q + key]) : 0.0;
+}
+
 // All pointers in the argument blocks are HOST pointers here.
 int oracle_kv_quantize_write(const pplhip_kv_write_args* a) {
     if (a->head_dim % kGroup) return PPLHIP_RC_INVALID_VALUE;
@@ -152,7 +159,8 @@ int oracle_kv_quantize_write(const pplhip_kv_write_args* a) {
 int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
     const int H = a->num_heads, KVH = a->num_kv_heads, Dh = a->head_dim;
     if (H <= 0 || KVH <= 0 || H % KVH || Dh % kGroup) return PPLHIP_RC_INVALID_VALUE;
-    if (a->d_attn_mask || a->d_alibi_slopes || (a->cache_mode != 0 && a->cache_mode != 1)) return PPLHIP_RC_UNSUPPORTED;
+    if (a->d_alibi_slopes || (a->cache_mode != 0 && a->cache_mode != 1)) return PPLHIP_RC_UNSUPPORTED;
+    if (a->d_attn_mask && (a->attn_mask_stride_q <= 0 || a->attn_mask_stride_h < 0)) return PPLHIP_RC_INVALID_VALUE;
     pplhip_kv_write_args w;
     memset(&w, 0, sizeof(w));
     w.d_current_key = a->d_current_key;
@@ -185,6 +193,7 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
     uint16_t* O = (uint16_t*)a->d_output;
     const int rep = H / KVH;
     const double sm_scale = 1.0 / sqrt((double)Dh);
+    const uint16_t* mask = (const uint16_t*)a->d_attn_mask;
 
 #pragma omp parallel for collapse(2) schedule(dynamic, 1)
     for (int64_t b = 0; b < a->batch; ++b) {
@@ -221,19 +230,20 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
                 for (int64_t j = 0; j <= last; ++j) {
                     double s = 0;
                     for (int d = 0; d < Dh; ++d) s += q[d] * K[j * Dh + d];
-                    p[j] = s * sm_scale;
+                    p[j] = s * sm_scale + mask_value(mask, a->attn_mask_stride_h, a->attn_mask_stride_q, h, s0 + t,
+                                                     a->d_kvstarts[b] + j);
                     m = std::max(m, p[j]);
                 }
                 double l = 0;
                 for (int64_t j = 0; j <= last; ++j) {
-                    p[j] = exp(p[j] - m);
+                    p[j] = m == -INFINITY ? 0.0 : exp(p[j] - m); // every key masked out: no distribution, zeros
                     l += p[j];
                 }
                 std::fill(acc.begin(), acc.end(), 0.0);
                 for (int64_t j = 0; j <= last; ++j)
                     for (int d = 0; d < Dh; ++d) acc[d] += p[j] * V[j * Dh + d];
                 for (int d = 0; d < Dh; ++d) {
-                    const double o = acc[d] / l;
+                    const double o = l > 0 ? acc[d] / l : 0.0;
                     const int64_t idx = ((s0 + t) * H + h) * Dh + d;
                     if (out_f64) out_f64[idx] = o;
                     O[idx] = float_to_half((float)o);
@@ -250,13 +260,15 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
 int oracle_mha_forward(const pplhip_mha_args* a, double* out_f64) {
     const int H = a->num_heads, KVH = a->num_kv_heads, Dh = a->head_dim;
     if (H <= 0 || KVH <= 0 || H % KVH) return PPLHIP_RC_INVALID_VALUE;
-    if (a->d_attn_mask || a->is_alibi) return PPLHIP_RC_UNSUPPORTED;
+    if (a->is_alibi) return PPLHIP_RC_UNSUPPORTED;
+    if (a->d_attn_mask && (a->attn_mask_stride_q <= 0 || a->attn_mask_stride_h < 0)) return PPLHIP_RC_INVALID_VALUE;
     const uint16_t* Q = (const uint16_t*)a->d_query;
     const uint16_t* Kp = (const uint16_t*)a->d_key;
     const uint16_t* Vp = (const uint16_t*)a->d_value;
     uint16_t* O = (uint16_t*)a->d_output;
     const int rep = H / KVH;
     const double sm_scale = 1.0 / sqrt((double)Dh);
+    const uint16_t* mask = (const uint16_t*)a->d_attn_mask;
 #pragma omp parallel for collapse(2) schedule(dynamic, 1)
     for (int64_t b = 0; b < a->batch; ++b) {
         for (int h = 0; h < H; ++h) {
@@ -274,12 +286,12 @@ int oracle_mha_forward(const pplhip_mha_args* a, double* out_f64) {
                     const uint16_t* kr = Kp + ((k0 + j) * KVH + kvh) * Dh;
                     double s = 0;
                     for (int d = 0; d < Dh; ++d) s += q[d] * (double)half_to_float(kr[d]);
-                    p[j] = s * sm_scale;
+                    p[j] = s * sm_scale + mask_value(mask, a->attn_mask_stride_h, a->attn_mask_stride_q, h, s0 + t, k0 + j);
                     m = std::max(m, p[j]);
                 }
                 double l = 0;
                 for (int64_t j = 0; j <= last; ++j) {
-                    p[j] = exp(p[j] - m);
+                    p[j] = m == -INFINITY ? 0.0 : exp(p[j] - m);
                     l += p[j];
                 }
                 std::fill(acc.begin(), acc.end(), 0.0);
@@ -288,7 +300,7 @@ int oracle_mha_forward(const pplhip_mha_args* a, double* out_f64) {
                     for (int d = 0; d < Dh; ++d) acc[d] += p[j] * (double)half_to_float(vr[d]);
                 }
                 for (int d = 0; d < Dh; ++d) {
-                    const double o = acc[d] / l;
+                    const double o = l > 0 ? acc[d] / l : 0.0;
                     const int64_t idx = ((s0 + t) * H + h) * Dh + d;
                     if (out_f64) out_f64[idx] = o;
                     O[idx] = float_to_half((float)o);

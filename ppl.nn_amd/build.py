@@ -10,7 +10,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # attention.hip is decode.hip + prefill.hip in one translation unit (it includes them: a call with decode sequences and
 # prompts runs both kinds of workgroup in one launch)
-KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "attention.hip", "pack.hip", "rope.hip", "probe.hip"]
+KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "attention.hip", "pack.hip", "rope.hip", "probe.hip", "generic.hip"]
 KERNEL_INCLUDED = ["decode.hip", "prefill.hip"]
 
 HIP_FLAGS = [

@@ -42,6 +42,7 @@ class MhcaArgs(C.Structure):
         ("specify_decoding_attn_split_k", _i32), ("specify_decoding_attn_tpb", _i32),
         ("d_cache", _p), ("d_scale", _p), ("d_output", _p),
         ("total_new_tokens", _i64),
+        ("attn_mask_stride_h", _i64), ("attn_mask_stride_q", _i64),
     ]
 
 
@@ -51,7 +52,7 @@ class MhcaPlan(C.Structure):
         ("decode_num_ranges", _i32), ("decode_heads_per_block", _i32), ("decode_waves_per_block", _i32),
         ("prefill_q_tile", _i32), ("prefill_num_q_tiles", _i32),
         ("prefill_staging", _i32), ("prefill_staging_offset_256", _i32),
-        ("reserved", _i32 * 1),
+        ("general_kernel", _i32),
     ]
 
 
@@ -85,6 +86,7 @@ class MhaArgs(C.Structure):
         ("batch", _i64), ("decoding_batches", _i64), ("max_seqlen", _i64), ("max_kvlen", _i64),
         ("num_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32), ("reserved", _i32),
         ("d_output", _p),
+        ("attn_mask_stride_h", _i64), ("attn_mask_stride_q", _i64),
     ]
 
 

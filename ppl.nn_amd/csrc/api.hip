@@ -56,8 +56,8 @@ static pplhip_retcode validate_common(int num_kv_heads, int head_dim, int num_la
     if (num_kv_heads <= 0 || num_layer <= 0 || layer_idx < 0 || layer_idx >= num_layer)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "bad num_kv_heads/num_layer/layer_idx (%d/%d/%d)", num_kv_heads,
                     num_layer, layer_idx);
-    if (head_dim != 128)
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: the gfx950 kernels are specialised for head_dim 128", head_dim);
+    if (!generic_head_dim_supported(head_dim))
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 32 between 32 and 256", head_dim);
     if (!cache) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache pointer is null");
     if (!scale)
         PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support quantized cache but scale not found");
@@ -69,6 +69,21 @@ static pplhip_retcode validate_common(int num_kv_heads, int head_dim, int num_la
                     (long long)stride_s);
     if (((uintptr_t)cache & 15) || ((uintptr_t)scale & 15))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache and scale must be 16-byte aligned");
+    return PPLHIP_RC_SUCCESS;
+}
+
+// The tuned kernels take head_dim 128 with at most 16 query heads per kv head and no mask; everything else runs the
+// general kernel.
+static bool needs_general_kernel(int head_dim, int num_heads, int num_kv_heads, const void* mask) {
+    return head_dim != 128 || num_heads / num_kv_heads > 16 || mask != nullptr;
+}
+
+static pplhip_retcode validate_mask(const void* mask, int64_t stride_h, int64_t stride_q) {
+    if (!mask) return PPLHIP_RC_SUCCESS;
+    if ((uintptr_t)mask & 1) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "attn_mask must be 2-byte aligned");
+    if (stride_q <= 0 || stride_h < 0)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "attn_mask strides: stride_q %lld must be positive, stride_h %lld not negative",
+                    (long long)stride_q, (long long)stride_h);
     return PPLHIP_RC_SUCCESS;
 }
 
@@ -137,7 +152,7 @@ const char* pplhip_last_error(void) {
 }
 
 int32_t pplhip_version(void) {
-    return 200; // 0.2.0
+    return 300; // 0.3.0
 }
 
 pplhip_retcode pplhip_init(void) {
@@ -154,16 +169,15 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     if (!a || !plan) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
     memset(plan, 0, sizeof(*plan));
     if (a->d_alibi_slopes) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support is_alibi == false");
-    if (a->d_attn_mask) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "attn_mask is not supported");
     {
         pplhip_retcode rcm = validate_cache_mode(a->cache_mode, a->page_size, a->cachestart_stride_b);
+        if (rcm != PPLHIP_RC_SUCCESS) return rcm;
+        rcm = validate_mask(a->d_attn_mask, a->attn_mask_stride_h, a->attn_mask_stride_q);
         if (rcm != PPLHIP_RC_SUCCESS) return rcm;
     }
     if (a->num_heads <= 0 || a->num_kv_heads <= 0 || a->num_heads % a->num_kv_heads)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d is not a multiple of num_kv_heads %d", a->num_heads,
                     a->num_kv_heads);
-    if (a->num_heads / a->num_kv_heads > 16)
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "more than 16 query heads per kv head");
     pplhip_retcode rc = validate_common(a->num_kv_heads, a->head_dim, a->num_layer, a->layer_idx, a->cache_stride_s,
                                         a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->d_cache, a->d_scale);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
@@ -185,6 +199,12 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_split_k must be 0, 1 or 2");
     if (a->specify_decoding_attn_tpb != 0 && a->specify_decoding_attn_tpb != 256 && a->specify_decoding_attn_tpb != 512)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_tpb must be 0, 256 or 512");
+
+    if (needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask)) {
+        // write kernel + one launch of the general attention kernel; nothing to plan and no workspace
+        plan->general_kernel = 1;
+        return PPLHIP_RC_SUCCESS;
+    }
 
     // ---- decode: the kernel cuts the decode sequences' cached tokens, laid end to end, into S equal ranges on the
     // device; the host only picks S from the chip size. One workgroup (4 waves) per range and group of <= 4 kv heads,
@@ -235,11 +255,19 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     if (plan->workspace_bytes > 0 && (!d_workspace || ((uintptr_t)d_workspace & 255)))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "workspace of %llu bytes (256-byte aligned) required",
                     (unsigned long long)plan->workspace_bytes);
-    if (a->decoding_batches > 0 && plan->decode_num_ranges <= 0)
+    const bool general = needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask);
+    if ((plan->general_kernel != 0) != general || (!general && a->decoding_batches > 0 && plan->decode_num_ranges <= 0))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
     hipStream_t s = (hipStream_t)stream;
     pplhip_kv_write_args w;
     write_args_from_mhca(a, &w);
+    if (general) {
+        // every new token goes into the slab first; decode sequences (and, in a cache-prefill call, the prompts) then
+        // attend over the slab
+        pplhip_retcode rcw = launch_kv_quantize_write(&w, s);
+        if (rcw != PPLHIP_RC_SUCCESS) return rcw;
+        return launch_generic_mhca(a, s);
+    }
     // the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens) into the
     // slab itself, and the prompt tokens are left to the prefill launch unless it reads them back from the slab
     // (cache-prefill): on the default path this launches nothing
@@ -270,13 +298,15 @@ pplhip_retcode pplhip_mhca_forward_noalloc(const pplhip_mhca_args* a, const pplh
 pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {
     if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
     if (a->is_alibi) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support is_alibi == false");
-    if (a->d_attn_mask) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "attn_mask is not supported");
-    if (a->head_dim != 128) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: only 128 is supported", a->head_dim);
+    if (!generic_head_dim_supported(a->head_dim))
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 32 between 32 and 256", a->head_dim);
+    {
+        const pplhip_retcode rcm = validate_mask(a->d_attn_mask, a->attn_mask_stride_h, a->attn_mask_stride_q);
+        if (rcm != PPLHIP_RC_SUCCESS) return rcm;
+    }
     if (a->num_heads <= 0 || a->num_kv_heads <= 0 || a->num_heads % a->num_kv_heads != 0)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d must be a positive multiple of num_kv_heads %d",
                     a->num_heads, a->num_kv_heads);
-    if (a->num_heads / a->num_kv_heads > 16)
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "more than 16 query heads per kv head");
     if (a->batch < 0 || a->max_seqlen < 0 || a->max_kvlen < a->max_seqlen)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "inconsistent batch %lld / max_seqlen %lld / max_kvlen %lld",
                     (long long)a->batch, (long long)a->max_seqlen, (long long)a->max_kvlen);
@@ -286,6 +316,8 @@ pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {
     if (((uintptr_t)a->d_query & 15) || ((uintptr_t)a->d_key & 15) || ((uintptr_t)a->d_value & 15) ||
         ((uintptr_t)a->d_output & 15))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "query/key/value/output must be 16-byte aligned");
+    if (needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask))
+        return launch_generic_mha(a, (hipStream_t)stream);
     return launch_mha(a, (hipStream_t)stream);
 }
 

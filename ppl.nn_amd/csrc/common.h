@@ -143,6 +143,11 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
 pplhip_retcode launch_decode_and_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws,
                                          hipStream_t stream);
 pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream);
+// the general attention kernel: any head_dim that is a multiple of 32 up to 256, any number of query heads per kv
+// head, optional attn_mask. The MHCA form reads the slab, which must already hold the call's new tokens.
+bool generic_head_dim_supported(int head_dim);
+pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, hipStream_t stream);
+pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream);
 pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream);
 pplhip_retcode launch_position_index(const int64_t* d_seqstarts, const int64_t* d_start_pos, int64_t batch,
                                      int64_t total_tokens, int64_t* d_out, hipStream_t stream);

@@ -21,6 +21,8 @@ struct QuantWriteParams {
     int32_t batch;
     int32_t kv_heads;
     int32_t per_tok; // 4-group units per token: 2 * kv_heads * (head_dim / 32)
+    int32_t units_per_head; // head_dim / 32
+    uint32_t inv_units_per_head; // ceil(65536 / units_per_head): r / units_per_head == (r * inv) >> 16 for r < 8192
     int32_t blocks_per_tok, tok_per_block; // one of the two is 1
     uint32_t inv_per_tok; // ceil(65536 / per_tok)
     int64_t first_token, end_token; // packed tokens [first_token, end_token) are written
@@ -28,7 +30,7 @@ struct QuantWriteParams {
 
 // One thread owns four consecutive groups (64 B of fp16 in, 32 B of int8 + 8 B of scales out) so that enough bytes
 // are in flight per CU to cover the memory latency. Thread -> (token, K or V, head, quarter of the head) without
-// integer division: a token has per_tok = 2 * kv_heads * 4 such units (head_dim is 128); a block covers 256 / per_tok
+// integer division: a token has per_tok = 2 * kv_heads * (head_dim / 32) such units; a block covers 256 / per_tok
 // whole tokens, one token, or a 256-unit slice of one.
 __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWriteParams p) {
     int64_t t; // packed new-token index
@@ -45,12 +47,13 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
         r = (int)threadIdx.x - lt * p.per_tok;
     }
     if (t >= p.end_token) return;
-    const int hi = r >> 2; // 0 .. 2 * kv_heads - 1: K heads, then V heads
-    const int grp = (r & 3) * 4; // first of the unit's four groups
+    const int hi = (int)(((uint32_t)r * p.inv_units_per_head) >> 16); // 0 .. 2 * kv_heads - 1: K heads, then V heads
+    const int grp = (r - hi * p.units_per_head) * 4; // first of the unit's four groups
     const int kv = hi >= p.kv_heads;
     const int head = hi - kv * p.kv_heads;
     // the values do not depend on which sequence the token belongs to: their loads go out before the look-up
-    const uint4* src = reinterpret_cast<const uint4*>((kv ? p.value : p.key) + ((t * p.kv_heads + head) * 16 + grp) * 8);
+    const uint4* src = reinterpret_cast<const uint4*>((kv ? p.value : p.key) +
+                                                      ((t * p.kv_heads + head) * (4 * p.units_per_head) + grp) * 8);
     uint4 raw[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) raw[i] = src[i];
@@ -100,8 +103,12 @@ pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream
     p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
     p.batch = (int32_t)a->batch;
     p.kv_heads = a->num_kv_heads;
-    if (a->head_dim != 128) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: head_dim must be 128");
-    p.per_tok = 2 * a->num_kv_heads * (a->head_dim / (4 * kQuantGroup));
+    if (a->head_dim <= 0 || a->head_dim % (4 * kQuantGroup) || a->head_dim > 256)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: head_dim must be a multiple of 32, at most 256");
+    p.units_per_head = a->head_dim / (4 * kQuantGroup);
+    p.inv_units_per_head = (65536u + (uint32_t)p.units_per_head - 1) / (uint32_t)p.units_per_head;
+    p.per_tok = 2 * a->num_kv_heads * p.units_per_head;
+    if (p.per_tok >= 8192) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: too many kv heads (%d)", a->num_kv_heads);
     p.blocks_per_tok = p.per_tok >= 256 ? (p.per_tok + 255) / 256 : 1;
     p.tok_per_block = p.per_tok >= 256 ? 1 : 256 / p.per_tok;
     p.inv_per_tok = (65536u + (uint32_t)p.per_tok - 1) / (uint32_t)p.per_tok;

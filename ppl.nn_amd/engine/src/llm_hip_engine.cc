@@ -37,6 +37,25 @@ struct EngineConfig final { // src/ppl/nn/engines/llm_cuda/engine_config.h:25-36
     int32_t rope_pair_layout = PPLHIP_ROPE_PAIRS_INTERLEAVED;
 };
 
+// The strides of an attn_mask tensor in the C ABI's terms: shape [S, K] (one mask for all heads) or [H, S, K] (one per
+// head), K >= kvstarts[batch] (exporters pad the last extent to a multiple of 8).
+static RetCode MaskStrides(const TensorImpl* mask, int num_heads, int64_t* stride_h, int64_t* stride_q) {
+    const TensorShape* sh = mask->GetShape();
+    const uint32_t n = sh->GetDimCount();
+    if (n == 2) {
+        *stride_h = 0;
+        *stride_q = sh->GetDim(1);
+        return RC_SUCCESS;
+    }
+    if (n == 3 && (sh->GetDim(0) == num_heads || sh->GetDim(0) == 1)) {
+        *stride_h = sh->GetDim(0) == 1 ? 0 : sh->GetDim(1) * sh->GetDim(2);
+        *stride_q = sh->GetDim(2);
+        return RC_SUCCESS;
+    }
+    LOG(ERROR) << "attn_mask must be [tokens, keys] or [num_heads, tokens, keys]";
+    return RC_INVALID_VALUE;
+}
+
 // ---------------------------------------------------------------- device
 class LlmHipDevice final : public Device {
 public:
@@ -364,6 +383,10 @@ protected:
         a.d_current_key = current_key->GetBufferPtr();
         a.d_current_value = current_value->GetBufferPtr();
         a.d_attn_mask = attn_mask_data;
+        if (attn_mask_data) {
+            const RetCode mrc = MaskStrides(attn_mask, param_->num_heads, &a.attn_mask_stride_h, &a.attn_mask_stride_q);
+            if (mrc != RC_SUCCESS) return mrc;
+        }
         a.d_seqstarts = seqstarts->GetBufferPtr<int64_t>();
         a.d_kvstarts = kvstarts->GetBufferPtr<int64_t>();
         a.d_cachestarts = cachestarts->GetBufferPtr<int64_t>();
@@ -578,6 +601,10 @@ protected:
         a.d_key = key->GetBufferPtr();
         a.d_value = value->GetBufferPtr();
         a.d_attn_mask = attn_mask_data;
+        if (attn_mask_data) {
+            const RetCode mrc = MaskStrides(attn_mask, param_->num_heads, &a.attn_mask_stride_h, &a.attn_mask_stride_q);
+            if (mrc != RC_SUCCESS) return mrc;
+        }
         a.d_seqstarts = seqstarts->GetBufferPtr<int64_t>();
         a.d_kvstarts = kvstarts->GetBufferPtr<int64_t>();
         a.is_causal = param_->is_causal;

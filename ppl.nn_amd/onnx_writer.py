@@ -83,18 +83,23 @@ MHCA_INPUTS = ["query", "current_key", "current_value", "seqstarts", "kvstarts",
 
 
 def mhca_model(num_heads, num_kv_heads, head_dim, num_layer, layer_idx, extra_attrs=(), drop_attrs=(), with_scale=True,
-               domain="opmx.dynamic_batching", opsets=None):
+               domain="opmx.dynamic_batching", opsets=None, mask_rank=0):
+    """mask_rank 2 or 3 appends the optional 13th input `attn_mask` ([tokens, keys] or [heads, tokens, keys])."""
     attrs = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, num_layer=num_layer,
                  layer_idx=layer_idx, quant_bit=8, quant_group=8)
     attrs.update(dict(extra_attrs))
     for k in drop_attrs:
         attrs.pop(k)
     names = list(MHCA_INPUTS) if with_scale else MHCA_INPUTS[:-1]
+    if mask_rank:
+        names.append("attn_mask")
     n = node("MultiHeadCacheAttention", names, ["attn_output"], name="attn", domain=domain,
              attrs=[attr_int(k, v) for k, v in attrs.items()])
-    types = {"query": FLOAT16, "current_key": FLOAT16, "current_value": FLOAT16, "cache": INT8, "scale": FLOAT16}
+    types = {"query": FLOAT16, "current_key": FLOAT16, "current_value": FLOAT16, "cache": INT8, "scale": FLOAT16,
+             "attn_mask": FLOAT16}
     ranks = {"query": 3, "current_key": 3, "current_value": 3, "seqstarts": 1, "kvstarts": 1, "cachestarts": 1,
-             "start_pos": 1, "decoding_batches": 0, "max_seqlen": 0, "max_kvlen": 0, "cache": 5, "scale": 5}
+             "start_pos": 1, "decoding_batches": 0, "max_seqlen": 0, "max_kvlen": 0, "cache": 5, "scale": 5,
+             "attn_mask": mask_rank}
     ins = [value_info(x, types.get(x, INT64), ["d%d" % i for i in range(ranks[x])]) for x in names]
     outs = [value_info("attn_output", FLOAT16, ["s", "h", "d"])]
     return model([n], ins, outs, opsets if opsets is not None else [("", 11), (domain, 1)])

@@ -83,11 +83,21 @@ def fill_write_args(w, b, key, value, seqstarts, start_pos, cachestarts, cache, 
     return w
 
 
+def _set_mask(a, mask, ptr):
+    """mask: None, or an fp16 array / device tensor [tokens, keys] (all heads) or [heads, tokens, keys]."""
+    if mask is None:
+        a.d_attn_mask, a.attn_mask_stride_h, a.attn_mask_stride_q = None, 0, 0
+        return
+    a.d_attn_mask = ptr(mask)
+    a.attn_mask_stride_q = int(mask.shape[-1])
+    a.attn_mask_stride_h = int(mask.shape[-2]) * int(mask.shape[-1]) if len(mask.shape) == 3 else 0
+
+
 def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out, ptr=_ptr,
-                   cache_prefill=0, split_k=1, paged=None, layout=0):
+                   cache_prefill=0, split_k=1, paged=None, layout=0, mask=None):
     st = _strides(b, paged, layout)
     a.d_query, a.d_current_key, a.d_current_value = ptr(q), ptr(k), ptr(v)
-    a.d_attn_mask = None
+    _set_mask(a, mask, ptr)
     a.d_alibi_slopes = None
     a.d_seqstarts, a.d_kvstarts = ptr(seqstarts), ptr(kvstarts)
     a.d_cachestarts, a.d_start_pos = ptr(cachestarts), ptr(start_pos)
@@ -105,11 +115,11 @@ def fill_mhca_args(a, b, q, k, v, seqstarts, kvstarts, cachestarts, start_pos, c
     a.specify_decoding_attn_tpb = 0
     a.d_cache, a.d_scale, a.d_output = ptr(cache), ptr(scale), ptr(out)
     a.total_new_tokens = b.total_new_tokens
-    a._refs = [q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out]
+    a._refs = [q, k, v, seqstarts, kvstarts, cachestarts, start_pos, cache, scale, out, mask]
     return a
 
 
-def run_oracle(b, t, cache_prefill=0, want_f64=True, paged=None, layout=0):
+def run_oracle(b, t, cache_prefill=0, want_f64=True, paged=None, layout=0, mask=None):
     """History write + MHCA on the CPU oracle. Returns cache (int8), scale (fp16), output (fp16), output_f64."""
     import oracle
     L = oracle.lib()
@@ -124,7 +134,7 @@ def run_oracle(b, t, cache_prefill=0, want_f64=True, paged=None, layout=0):
     out64 = np.zeros(out.shape, np.float64) if want_f64 else None
     seqstarts, kvstarts, sp = b.seqstarts, b.kvstarts, b.start_pos.copy()
     a = fill_mhca_args(cabi.MhcaArgs(), b, t["query"], t["current_key"], t["current_value"], seqstarts, kvstarts,
-                       cs, sp, cache, scale, out, cache_prefill=cache_prefill, paged=paged, layout=layout)
+                       cs, sp, cache, scale, out, cache_prefill=cache_prefill, paged=paged, layout=layout, mask=mask)
     rc = L.oracle_mhca_forward(C.byref(a), _ptr(out64))
     assert rc == 0, rc
     return dict(cache=cache, scale=scale, output=out, output_f64=out64)
@@ -141,7 +151,8 @@ def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0, staging=None, lib=None):
+def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0, staging=None, lib=None,
+               mask=None):
     """Same call through the C ABI on cuda:0. staging=0 clears plan.prefill_staging (the caller's way to keep a
     cache-prefill call on the kernel that reads the int8 slab itself). lib: another build of the kernel library than
     the product one."""
@@ -162,7 +173,8 @@ def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layo
     out = torch.zeros((b.total_new_tokens, b.num_heads, b.head_dim), dtype=torch.float16, device="cuda")
     a = fill_mhca_args(cabi.MhcaArgs(), b, d["query"], d["current_key"], d["current_value"], dt["seqstarts"],
                        dt["kvstarts"], dt["cachestarts"], dt["start_pos"], cache, scale, out, ptr=dev_ptr,
-                       cache_prefill=cache_prefill, split_k=split_k, paged=paged, layout=layout)
+                       cache_prefill=cache_prefill, split_k=split_k, paged=paged, layout=layout,
+                       mask=None if mask is None else to_dev(mask))
     plan = cabi.MhcaPlan()
     pkg.check(lib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)), "mhca_prepare")
     ws = torch.empty(max(int(plan.workspace_bytes), 256), dtype=torch.uint8, device="cuda")
@@ -189,36 +201,37 @@ def mha_inputs(b, t):
     return cat(keys), cat(values)
 
 
-def fill_mha_args(a, b, q, key, value, seqstarts, kvstarts, out, ptr=_ptr):
-    a.d_query, a.d_key, a.d_value, a.d_attn_mask = ptr(q), ptr(key), ptr(value), None
+def fill_mha_args(a, b, q, key, value, seqstarts, kvstarts, out, ptr=_ptr, mask=None):
+    a.d_query, a.d_key, a.d_value = ptr(q), ptr(key), ptr(value)
+    _set_mask(a, mask, ptr)
     a.d_seqstarts, a.d_kvstarts = ptr(seqstarts), ptr(kvstarts)
     a.is_causal, a.is_alibi = b.is_causal, 0
     a.batch, a.decoding_batches = b.batch, b.decoding_batches
     a.max_seqlen, a.max_kvlen = b.max_seqlen, b.max_kvlen
     a.num_heads, a.num_kv_heads, a.head_dim = b.num_heads, b.num_kv_heads, b.head_dim
     a.d_output = ptr(out)
-    a._refs = [q, key, value, seqstarts, kvstarts, out]
+    a._refs = [q, key, value, seqstarts, kvstarts, out, mask]
     return a
 
 
-def run_oracle_mha(b, q, key, value):
+def run_oracle_mha(b, q, key, value, mask=None):
     import oracle
     out = np.zeros((b.total_new_tokens, b.num_heads, b.head_dim), np.float16)
     out64 = np.zeros(out.shape, np.float64)
-    a = fill_mha_args(cabi.MhaArgs(), b, q, key, value, b.seqstarts, b.kvstarts, out)
+    a = fill_mha_args(cabi.MhaArgs(), b, q, key, value, b.seqstarts, b.kvstarts, out, mask=mask)
     rc = oracle.lib().oracle_mha_forward(C.byref(a), _ptr(out64))
     assert rc == 0, rc
     return dict(output=out, output_f64=out64)
 
 
-def run_device_mha(b, q, key, value):
+def run_device_mha(b, q, key, value, mask=None):
     import torch
     lib = pkg.load_library()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     dq, dk, dv = to_dev(q), to_dev(key), to_dev(value)
     ss, ks = to_dev(b.seqstarts), to_dev(b.kvstarts)
     out = torch.zeros((b.total_new_tokens, b.num_heads, b.head_dim), dtype=torch.float16, device="cuda")
-    a = fill_mha_args(cabi.MhaArgs(), b, dq, dk, dv, ss, ks, out, ptr=dev_ptr)
+    a = fill_mha_args(cabi.MhaArgs(), b, dq, dk, dv, ss, ks, out, ptr=dev_ptr, mask=None if mask is None else to_dev(mask))
     pkg.check(lib.pplhip_mha_forward(C.byref(a), stream), "mha_forward")
     torch.cuda.synchronize()
     return dict(output=out.cpu().view(torch.int16).numpy().view(np.float16))
@@ -257,11 +270,13 @@ def assert_attn_close(got_f16, ref_f64, abs_tol=ABS_TOL, rel_tol=REL_TOL, what="
     return float(err.max())
 
 
-def textbook_attention(q, k, v, causal_offset=None):
+def textbook_attention(q, k, v, causal_offset=None, mask=None):
     """float64 softmax(q k^T / sqrt(d) + mask) v for one head. q [Lq, d], k/v [Lk, d].
-    causal_offset: query row i sees keys j <= causal_offset + i (None = no mask)."""
+    causal_offset: query row i sees keys j <= causal_offset + i (None = no causal mask); mask: additive [Lq, Lk]."""
     q, k, v = (x.astype(np.float64) for x in (q, k, v))
     s = q @ k.T / np.sqrt(q.shape[-1])
+    if mask is not None:
+        s = s + mask.astype(np.float64)
     if causal_offset is not None:
         i = np.arange(q.shape[0])[:, None]
         j = np.arange(k.shape[0])[None, :]

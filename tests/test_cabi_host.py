@@ -71,14 +71,18 @@ def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
 @pytest.mark.parametrize("mutate,rc", [
     (lambda a: setattr(a, "d_alibi_slopes", 0x10), cabi.RC_UNSUPPORTED),  # …_kernel.cc:95-98
     (lambda a: setattr(a, "d_scale", None), cabi.RC_UNSUPPORTED),  # …_kernel.cc:100-103
-    (lambda a: setattr(a, "d_attn_mask", 0x10), cabi.RC_UNSUPPORTED),
+    (lambda a: setattr(a, "d_attn_mask", 0x10), cabi.RC_INVALID_VALUE),  # a mask without its row stride
+    (lambda a: (setattr(a, "d_attn_mask", 0x11), setattr(a, "attn_mask_stride_q", 64)), cabi.RC_INVALID_VALUE),
+    (lambda a: (setattr(a, "d_attn_mask", 0x10), setattr(a, "attn_mask_stride_q", 64),
+                setattr(a, "attn_mask_stride_h", -1)), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "cache_mode", 1), cabi.RC_INVALID_VALUE),  # no 2-d page table: …_kernel.cc:162-166
     (lambda a: setattr(a, "cache_mode", 2), cabi.RC_UNSUPPORTED),
     (lambda a: (setattr(a, "cache_mode", 1), setattr(a, "cachestart_stride_b", 4), setattr(a, "page_size", 96)),
      cabi.RC_UNSUPPORTED),
     (lambda a: (setattr(a, "cache_mode", 1), setattr(a, "cachestart_stride_b", 4), setattr(a, "page_size", 32)),
      cabi.RC_UNSUPPORTED),
-    (lambda a: setattr(a, "head_dim", 64), cabi.RC_UNSUPPORTED),
+    (lambda a: setattr(a, "head_dim", 80), cabi.RC_UNSUPPORTED),  # multiples of 32 up to 256
+    (lambda a: setattr(a, "head_dim", 288), cabi.RC_UNSUPPORTED),
     (lambda a: setattr(a, "num_kv_heads", 3), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "layer_idx", 5), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "decoding_batches", 3), cabi.RC_INVALID_VALUE),
@@ -94,6 +98,22 @@ def test_prepare_rejects(hiplib, mutate, rc):
     mutate(a)
     assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == rc
     assert len(hiplib.pplhip_last_error()) > 0
+
+
+@pytest.mark.parametrize("mutate", [
+    lambda a: setattr(a, "head_dim", 64),
+    lambda a: setattr(a, "head_dim", 256),
+    lambda a: (setattr(a, "num_heads", 34), setattr(a, "num_kv_heads", 2)),  # 17 query heads per kv head
+    lambda a: (setattr(a, "d_attn_mask", 0x10), setattr(a, "attn_mask_stride_q", 64)),
+])
+def test_prepare_routes_other_shapes_to_the_general_kernel(hiplib, mutate):
+    """head_dim other than 128, more than 16 query heads per kv head, or an attn_mask: the plan says so, needs no
+    workspace and plans no split-k ranges."""
+    a, plan = _valid_args(), cabi.MhcaPlan()
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS and plan.general_kernel == 0
+    mutate(a)
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS, hiplib.pplhip_last_error()
+    assert plan.general_kernel == 1 and plan.workspace_bytes == 0 and plan.decode_num_ranges == 0
 
 
 @pytest.mark.parametrize("kvh", [1, 2, 3, 4, 5, 8, 12, 16, 32, 40, 64])
@@ -182,8 +202,10 @@ def test_mha_rejects_like_the_reference_wrapper(hiplib):
     # multi_head_attention_kernel.cc:71-74
     assert hiplib.pplhip_mha_forward(C.byref(args(is_alibi=1)), None) == cabi.RC_UNSUPPORTED
     assert b"is_alibi" in hiplib.pplhip_last_error()
-    assert hiplib.pplhip_mha_forward(C.byref(args(d_attn_mask=0x1000)), None) == cabi.RC_UNSUPPORTED
-    assert hiplib.pplhip_mha_forward(C.byref(args(head_dim=64)), None) == cabi.RC_UNSUPPORTED
+    assert hiplib.pplhip_mha_forward(C.byref(args(d_attn_mask=0x1000)), None) == cabi.RC_INVALID_VALUE  # no stride
+    assert hiplib.pplhip_mha_forward(C.byref(args(d_attn_mask=0x1000, attn_mask_stride_q=8)), None) == cabi.RC_SUCCESS
+    assert hiplib.pplhip_mha_forward(C.byref(args(head_dim=64)), None) == cabi.RC_SUCCESS
+    assert hiplib.pplhip_mha_forward(C.byref(args(head_dim=72)), None) == cabi.RC_UNSUPPORTED
     assert hiplib.pplhip_mha_forward(C.byref(args(num_kv_heads=3)), None) == cabi.RC_INVALID_VALUE
     assert hiplib.pplhip_mha_forward(C.byref(args(batch=1, max_seqlen=4, max_kvlen=2)), None) == cabi.RC_INVALID_VALUE
     assert hiplib.pplhip_mha_forward(C.byref(args(batch=1, max_seqlen=1, max_kvlen=2, d_key=0)), None) == \

@@ -122,6 +122,40 @@ def test_mhca_graph_through_the_engine(hiplib, cache_prefill):
     s.close()
 
 
+@pytest.mark.parametrize("head_dim,mask_rank", [(64, 0), (64, 3), (128, 2), (256, 0)])
+def test_mhca_graph_other_head_dims_and_attn_mask(hiplib, head_dim, mask_rank):
+    """The same graph with a head_dim other than 128 and / or the optional 13th input attn_mask: the engine reads the
+    mask's strides off its shape and the call runs the general kernel."""
+    import torch
+    from test_oracle_attention import _mask_for
+    eng = harness.pkg.load_engine_library()
+    b = workloads.Batch(8, 2, head_dim, [1, 1, 70, 130], [500, 3, 0, 0], 2, num_layer=2, layer_idx=1, name="engine_general")
+    t = workloads.make_tensors(b, seed=78)
+    mask = _mask_for(b, np.random.default_rng(1), per_head=mask_rank == 3) if mask_rank else None
+    ref = harness.run_oracle(b, t, mask=mask)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    s = Session(eng, ow.mhca_model(8, 2, head_dim, 2, 1, mask_rank=mask_rank))
+    assert eng.pplnn_hip_runtime_input_count(s.rt) == 12 + (1 if mask_rank else 0)
+    for i, name in enumerate(("query", "current_key", "current_value")):
+        s.set_device_tensor(i, harness.to_dev(t[name]))
+    for i, tab in enumerate((b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)):
+        s.set_table(3 + i, tab)
+    for i, v in enumerate((b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+        s.set_host_scalar(7 + i, v)
+    s.set_device_tensor(10, cache)
+    s.set_device_tensor(11, scale)
+    if mask_rank:
+        s.set_device_tensor(12, harness.to_dev(mask))
+    print(f"case {b.name} head_dim={head_dim} mask_rank={mask_rank}", flush=True)
+    assert eng.pplnn_hip_runtime_run(s.rt) == 0, eng.pplnn_hip_last_error()
+    out = s.output(0, np.float16)
+    assert out.shape == (b.total_new_tokens, 8, head_dim)
+    harness.assert_attn_close(out, ref["output_f64"])
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), ref["cache"])
+    s.close()
+
+
 def test_engine_error_paths_on_device(hiplib):
     eng = harness.pkg.load_engine_library()
     eng.pplnn_hip_set_log_level(4)

@@ -1,0 +1,140 @@
+"""The general attention kernel through the C ABI: head_dim other than 128, more than 16 query heads per kv head and
+the additive attn_mask, for MultiHeadCacheAttention (decode sequences, prompts, cache-prefill, paged slab, layer
+strides) and MultiHeadAttention. Same bar as the tuned kernels: slab bytes and scales bit-exact against the oracle,
+outputs within 2e-3 abs + 1e-2 rel of its float64 result."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness
+from harness import cabi, workloads
+from test_oracle_attention import _mask_for
+
+pytestmark = pytest.mark.gpu
+
+
+def check(b, t, what, **kw):
+    print(f"case {what}: H={b.num_heads} KVH={b.num_kv_heads} Dh={b.head_dim} B={b.batch} nd={b.decoding_batches} "
+          f"S={b.total_new_tokens} hist={b.total_hist_tokens} {sorted(k for k in kw)}", flush=True)
+    plans = []
+    ref = harness.run_oracle(b, t, **kw)
+    got = harness.run_device(b, t, plan_out=plans, **kw)
+    assert plans[0].general_kernel == 1 and plans[0].workspace_bytes == 0
+    assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
+    assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
+    harness.assert_attn_close(got["output"], ref["output_f64"], what=what)
+    return ref, got
+
+
+@pytest.mark.parametrize("Dh", [32, 64, 96, 160, 192, 224, 256])
+@pytest.mark.parametrize("H,KVH", [(8, 2), (5, 5), (6, 1)])
+def test_head_dims_mixed_batch(Dh, H, KVH):
+    # decode sequences of 1 .. several tiles of history, prompts that straddle the 64-row and 64-token tile edges
+    b = workloads.Batch(H, KVH, Dh, [1, 1, 1, 1, 7, 65, 130], [300, 1, 63, 64, 0, 0, 0], 4, num_layer=2, layer_idx=1,
+                        name="general_mixed")
+    check(b, workloads.make_tensors(b, seed=Dh + H), f"head_dim {Dh}")
+
+
+@pytest.mark.parametrize("H,KVH", [(34, 2), (20, 1), (48, 2)])
+def test_more_than_16_query_heads_per_kv_head(H, KVH):
+    b = workloads.Batch(H, KVH, 128, [1, 1, 40, 3], [500, 17, 0, 0], 2, name="general_rep")
+    check(b, workloads.make_tensors(b, seed=H), f"{H // KVH} query heads per kv head")
+
+
+@pytest.mark.parametrize("Dh", [64, 128])
+@pytest.mark.parametrize("per_head", [False, True])
+@pytest.mark.parametrize("causal", [1, 0])
+def test_attn_mask(Dh, per_head, causal):
+    b = workloads.Batch(8, 2, Dh, [1, 1, 1, 9, 70, 129], [200, 3, 64, 0, 0, 0], 3, is_causal=causal, name="general_mask")
+    t = workloads.make_tensors(b, seed=7 + Dh)
+    mask = _mask_for(b, np.random.default_rng(Dh + per_head), per_head)
+    ref, got = check(b, t, f"attn_mask per_head={per_head} causal={causal}", mask=mask)
+    plain = harness.run_oracle(b, t)
+    assert np.abs(plain["output_f64"] - ref["output_f64"]).max() > 1e-3  # the mask matters
+
+
+def test_attn_mask_with_a_fully_masked_row():
+    b = workloads.Batch(4, 2, 64, [1, 5], [70, 0], 1, name="general_mask_row")
+    t = workloads.make_tensors(b, seed=3)
+    mask = _mask_for(b, np.random.default_rng(9), per_head=False)
+    mask[0, :] = -np.inf  # the decode sequence sees nothing
+    mask[3, :] = -np.inf  # so does one prompt token
+    ref, got = check(b, t, "fully masked rows", mask=mask)
+    assert (got["output"][0] == 0).all() and (got["output"][3] == 0).all()
+
+
+def test_cache_prefill_paged_and_layout_3():
+    b = workloads.Batch(8, 2, 64, [1, 1, 70, 300], [130, 1000, 64, 0], 2, num_layer=2, layer_idx=1, name="general_cp")
+    t = workloads.make_tensors(b, seed=52)
+    ref, flat = check(b, t, "cache-prefill", cache_prefill=1)
+    paged = harness.PagedLayout(b, page_size=64, seed=5)
+    _, got = check(b, t, "cache-prefill, paged slab", cache_prefill=1, paged=paged)
+    assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
+    _, got3 = check(b, t, "cache-prefill, cache_layout 3", cache_prefill=1, layout=3)
+    assert np.array_equal(got3["output"].view(np.uint16), flat["output"].view(np.uint16))
+
+
+@pytest.mark.parametrize("Dh,mask_on", [(64, False), (96, True), (256, False), (128, True)])
+def test_multi_head_attention_general(Dh, mask_on):
+    b = workloads.Batch(8, 2, Dh, [1, 1, 7, 130, 64], [300, 0, 0, 70, 64], 2, name="general_mha")
+    t = workloads.make_tensors(b, seed=31)
+    key, value = harness.mha_inputs(b, t)
+    mask = _mask_for(b, np.random.default_rng(2), per_head=True) if mask_on else None
+    print(f"case {b.name} Dh={Dh} mask={mask_on}", flush=True)
+    ref = harness.run_oracle_mha(b, t["query"], key, value, mask=mask)
+    got = harness.run_device_mha(b, t["query"], key, value, mask=mask)
+    harness.assert_attn_close(got["output"], ref["output_f64"], what="MultiHeadAttention (general kernel)")
+
+
+def test_general_kernel_agrees_with_the_tuned_kernels():
+    """At head_dim 128 an all-zero mask sends the same call through the general kernel: both paths must agree with
+    the oracle, and with each other within twice the tolerance."""
+    b = workloads.Batch(32, 8, 128, [1] * 6 + [100, 257], [900, 64, 1, 2047, 333, 65, 0, 0], 6, name="general_vs_tuned")
+    t = workloads.make_tensors(b, seed=4)
+    zero = np.zeros((b.total_new_tokens, (int(b.kvstarts[-1]) + 7) // 8 * 8), np.float16)
+    ref, gen = check(b, t, "zero mask", mask=zero)
+    tuned = harness.run_device(b, t)
+    harness.assert_attn_close(tuned["output"], ref["output_f64"])
+    assert np.array_equal(tuned["cache"], gen["cache"])
+    d = np.abs(tuned["output"].astype(np.float64) - gen["output"].astype(np.float64))
+    assert d.max() <= 2 * (2e-3 + 1e-2 * np.abs(ref["output_f64"]).max())
+
+
+def test_key_value_cache_op_other_head_dim(hiplib, olib):
+    """KeyValueCache (quantise-write + gather) at head_dim 96: slab and gathered rows bit-exact."""
+    import torch
+    b = workloads.Batch(3, 3, 96, [1, 6, 40], [9, 0, 3], 0, num_layer=2, layer_idx=1, slack_tokens=2)
+    t = workloads.make_tensors(b, seed=9)
+    zeros = np.zeros(b.batch, np.int64)
+    total_kv = int(b.kvstarts[-1])
+
+    def run(lib_write, lib_fwd, ptr, conv, stream_args):
+        cache, scale = harness.new_slab(b)
+        cache, scale = conv(cache), conv(scale)
+        tt = {k: conv(v) for k, v in t.items()}
+        tabs = {k: conv(v) for k, v in dict(hs=b.histstarts, z=zeros, cs=b.cachestarts, ss=b.seqstarts,
+                                            ks=b.kvstarts, sp=b.start_pos).items()}
+        w = harness.fill_write_args(cabi.KvWriteArgs(), b, tt["hist_key"], tt["hist_value"], tabs["hs"], tabs["z"],
+                                    tabs["cs"], cache, scale, ptr=ptr)
+        assert lib_write(C.byref(w), *stream_args) == 0
+        a = cabi.KvCacheArgs()
+        harness.fill_write_args(a.write, b, tt["current_key"], tt["current_value"], tabs["ss"], tabs["sp"], tabs["cs"],
+                                cache, scale, ptr=ptr)
+        a.d_kvstarts = ptr(tabs["ks"])
+        a.total_kv_tokens, a.max_kvlen = total_kv, b.max_kvlen
+        a.num_repeat, a.cache_mode, a.cache_layout = 1, 0, 0
+        ko = conv(np.zeros((total_kv, 3, 96), np.float16))
+        vo = conv(np.zeros((total_kv, 3, 96), np.float16))
+        a.d_key_out, a.d_value_out = ptr(ko), ptr(vo)
+        assert lib_fwd(C.byref(a), *stream_args) == 0
+        return cache, scale, ko, vo
+
+    co, so, ko, vo = run(lambda w: olib.oracle_kv_quantize_write(w), lambda a: olib.oracle_kv_cache_forward(a),
+                         harness._ptr, lambda x: np.ascontiguousarray(x).copy(), ())
+    cd, sd, kd, vd = run(hiplib.pplhip_kv_quantize_write, hiplib.pplhip_kv_cache_forward, harness.dev_ptr,
+                         harness.to_dev, (None,))
+    torch.cuda.synchronize()
+    f16 = lambda x: x.cpu().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(cd.cpu().numpy(), co) and np.array_equal(f16(sd), so.view(np.uint16))
+    assert np.array_equal(f16(kd), ko.view(np.uint16)) and np.array_equal(f16(vd), vo.view(np.uint16))

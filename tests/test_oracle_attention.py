@@ -246,3 +246,93 @@ def test_cache_layout_3_equals_layout_0():
     assert np.array_equal(l0["output_f64"], l3["output_f64"])
     assert np.array_equal(l0["cache"].transpose(1, 2, 3, 0, 4), l3["cache"])
     assert np.array_equal(l0["scale"].view(np.uint16).transpose(1, 2, 3, 0, 4), l3["scale"].view(np.uint16))
+
+
+def _random_mask(rng, shape, kstart_pad=0, frac_inf=0.15):
+    """fp16 additive mask with some keys masked out completely (-inf), never a whole row."""
+    m = (rng.standard_normal(shape) * 2).astype(np.float16)
+    drop = rng.random(shape) < frac_inf
+    drop[..., 0] = False  # key 0 of the packed axis is not what rows see; rows are fixed up by the callers
+    m[drop] = -np.inf
+    return m
+
+
+def _mask_for(b, rng, per_head):
+    """A mask over packed query tokens x packed keys, last extent padded to a multiple of 8 (as exporters do); every
+    row keeps its sequence's first key so that no row is masked out entirely."""
+    S, K = b.total_new_tokens, int(b.kvstarts[-1])
+    kpad = (K + 7) // 8 * 8
+    shape = (b.num_heads, S, kpad) if per_head else (S, kpad)
+    m = _random_mask(rng, shape)
+    for i in range(b.batch):
+        m[..., b.seqstarts[i]:b.seqstarts[i + 1], b.kvstarts[i]] = np.float16(0.25)
+    return m
+
+
+@pytest.mark.parametrize("per_head", [False, True])
+@pytest.mark.parametrize("causal", [1, 0])
+def test_attn_mask_vs_textbook(per_head, causal):
+    """The additive mask: entry [h?, seqstarts[b] + t, kvstarts[b] + j] is added to the scaled score of query t and key
+    j of sequence b, on top of the causal rule. Checked per head against the float64 textbook routine."""
+    b = workloads.Batch(6, 2, 64, [1, 1, 9, 33], [40, 3, 0, 0], 2, is_causal=causal)
+    t = workloads.make_tensors(b, seed=77)
+    mask = _mask_for(b, np.random.default_rng(5), per_head)
+    res = harness.run_oracle(b, t, mask=mask)
+    deq = dequant_slab(res["cache"], res["scale"])
+    rep = b.num_heads // b.num_kv_heads
+    for i in range(b.batch):
+        s0, L, sp, kv, k0 = b.seqstarts[i], b.seqlens[i], b.start_pos[i], b.kvlens[i], b.kvstarts[i]
+        for h in range(b.num_heads):
+            if i < b.decoding_batches:
+                rows = slice(b.cachestarts[i], b.cachestarts[i] + kv)
+                k, v = deq[rows, 0, 0, h // rep], deq[rows, 0, 1, h // rep]
+            else:
+                k, v = t["current_key"][s0:s0 + L, h // rep], t["current_value"][s0:s0 + L, h // rep]
+            mm = (mask[h] if per_head else mask)[s0:s0 + L, k0:k0 + kv]
+            want = harness.textbook_attention(t["query"][s0:s0 + L, h], k, v, causal_offset=sp if causal else None,
+                                              mask=mm)
+            assert np.abs(res["output_f64"][s0:s0 + L, h] - want).max() < 1e-12, (i, h)
+    # the mask matters: without it the result differs
+    plain = harness.run_oracle(b, t)
+    assert np.abs(plain["output_f64"] - res["output_f64"]).max() > 1e-3
+
+
+def test_attn_mask_special_cases():
+    b = workloads.Batch(4, 2, 32, [1, 5], [6, 0], 1)
+    t = workloads.make_tensors(b, seed=78)
+    S, K = b.total_new_tokens, int(b.kvstarts[-1])
+    # an all-zero mask changes nothing
+    zero = np.zeros((S, K), np.float16)
+    plain = harness.run_oracle(b, t)
+    assert np.array_equal(harness.run_oracle(b, t, mask=zero)["output_f64"], plain["output_f64"])
+    # a constant added to a whole row cancels in the softmax
+    const = np.full((S, K), 3.0, np.float16)
+    assert np.abs(harness.run_oracle(b, t, mask=const)["output_f64"] - plain["output_f64"]).max() < 1e-12
+    # -inf on every key but one: the output is that key's value row
+    only = np.full((S, K), -np.inf, np.float16)
+    only[0, b.kvstarts[0] + 2] = 0
+    for tq in range(5):
+        only[1 + tq, b.kvstarts[1] + 0] = 0
+    res = harness.run_oracle(b, t, mask=only)
+    deq = dequant_slab(res["cache"], res["scale"])
+    assert np.abs(res["output_f64"][0, 3] - deq[b.cachestarts[0] + 2, 0, 1, 1]).max() < 1e-12
+    assert np.abs(res["output_f64"][3, 0] - t["current_value"][b.seqstarts[1], 0].astype(np.float64)).max() < 1e-12
+    # every key of a row masked out: zeros, not NaN
+    none = only.copy()
+    none[0, :] = -np.inf
+    res = harness.run_oracle(b, t, mask=none)
+    assert (res["output_f64"][0] == 0).all() and np.isfinite(res["output_f64"]).all()
+
+
+def test_mha_attn_mask_vs_textbook():
+    b = workloads.Batch(4, 1, 96, [1, 7, 20], [30, 0, 12], 1)
+    t = workloads.make_tensors(b, seed=79)
+    key, value = harness.mha_inputs(b, t)
+    mask = _mask_for(b, np.random.default_rng(6), per_head=True)
+    res = harness.run_oracle_mha(b, t["query"], key, value, mask=mask)
+    for i in range(b.batch):
+        s0, L, kv, k0 = b.seqstarts[i], b.seqlens[i], b.kvlens[i], b.kvstarts[i]
+        for h in range(b.num_heads):
+            want = harness.textbook_attention(t["query"][s0:s0 + L, h], key[k0:k0 + kv, 0], value[k0:k0 + kv, 0],
+                                              causal_offset=kv - L, mask=mask[h, s0:s0 + L, k0:k0 + kv])
+            assert np.abs(res["output_f64"][s0:s0 + L, h] - want).max() < 1e-12
