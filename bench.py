@@ -229,6 +229,26 @@ def mfma_sustained(lib, pkg):
     return out
 
 
+def hbm_sustained(lib, pkg):
+    """GB/s of a plain streaming read of 2 GiB (eight times the memory-side cache) by 512 / 2048 / 8192 workgroups:
+    the practical ceiling of this box beside the published HBM peak."""
+    import torch
+    n = 2 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for wgs in (512, 2048, 8192):
+        dst = torch.empty(wgs * 256, dtype=torch.int32, device="cuda")
+        got = C.c_uint64()
+        call = lambda i: pkg.check(lib.pplhip_probe_hbm_read(C.c_void_p(src.data_ptr()), n, C.c_void_p(dst.data_ptr()),
+                                                              wgs, C.byref(got), stream), "hbm probe")
+        _, med_ms, _ = timed_robust(call, min_warmup=3, min_iters=20, min_ms=100.0, batches=5)
+        out["%d_workgroups" % wgs] = got.value / (med_ms * 1e-3) / 1e9
+    del src
+    torch.cuda.empty_cache()
+    return out
+
+
 PROFILE_TRAFFIC = os.path.join(ROOT, "profiles", "decode_int8kv_cfg2_hbm_traffic.txt")
 
 
@@ -414,6 +434,11 @@ def main():
                      "median_ms_per_launch_long_run": dec_med_ms, "long_run_calls": dec_n,
                      "traffic_source": "recorded rocprofv3 --pmc summary under profiles/ (not re-measured in this run)"},
     }
+    stream_gbs = hbm_sustained(lib, pkg)
+    result["hbm_read_sustained_GBs"] = dict(
+        stream_gbs, note="plain streaming read of 2 GiB measured in this run; the published peak is %.0f" % HBM_PEAK_GBS)
+    result["roofline"]["frac_of_sustained_hbm_read"] = gbs / max(stream_gbs.values())
+
     def frac(tflops):
         return tflops / MFMA_FP16_PEAK_TFLOPS
 

@@ -374,6 +374,16 @@ pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot
 pplhip_retcode pplhip_probe_mfma_f16(const void* d_operands, void* d_out, int32_t workgroups, int32_t iterations,
                                      double* flops, void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): `workgroups` workgroups each stream their own contiguous share
+ * of the `bytes` at `d_src` (device, 16-byte aligned) with plain 16-byte loads, eight in flight per lane, and write one
+ * word per lane to `d_out` (workgroups x 256 words). `*bytes_read` (host, may be NULL) receives what the launch read
+ * (shares are rounded down to whole rounds of 32 KiB). Timed over a buffer much larger than the memory-side cache it
+ * gives the streaming-read rate the chip sustains, the practical ceiling beside the published 8 TB/s.
+ */
+pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_out, int32_t workgroups,
+                                     uint64_t* bytes_read, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,5 @@
-// Calibration probe for the fp16 matrix-core roofline: a bare loop of independent v_mfma_f32_32x32x16_f16 over operands
+// Calibration probes for the two rooflines.
+// fp16 matrix cores: a bare loop of independent v_mfma_f32_32x32x16_f16 over operands
 // the caller supplies. The rate this chip SUSTAINS depends on the operand data (power management lowers the clock when
 // the operands toggle many bits): the benchmark reports the prefill kernel next to the published peak and next to
 // this measured figure for random fp16 operands.
@@ -36,9 +37,46 @@ __global__ __launch_bounds__(256) void probe_mfma_f16_kernel(const half8_t* __re
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// HBM: every workgroup streams its own contiguous share of a buffer with 16-byte loads, eight in flight per lane, and
+// folds what it read into one word per lane (so that no load can be dropped). The benchmark runs it over a buffer far
+// larger than the 256 MB memory-side cache and reports the decode kernel next to the published 8 TB/s and next to
+// this measured streaming rate.
+constexpr int kProbeLoadsInFlight = 8;
+
+typedef uint32_t u32x4_probe_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void probe_hbm_read_kernel(const u32x4_probe_t* __restrict__ src, uint64_t chunk16,
+                                                             uint32_t* __restrict__ out) {
+    const u32x4_probe_t* p = src + (uint64_t)blockIdx.x * chunk16;
+    uint32_t acc = 0;
+    for (uint64_t i = threadIdx.x; i + (kProbeLoadsInFlight - 1) * 256 < chunk16; i += kProbeLoadsInFlight * 256) {
+        u32x4_probe_t v[kProbeLoadsInFlight];
+#pragma unroll
+        for (int j = 0; j < kProbeLoadsInFlight; ++j) v[j] = __builtin_nontemporal_load(p + i + j * 256);
+#pragma unroll
+        for (int j = 0; j < kProbeLoadsInFlight; ++j) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    }
+    out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+
 } // namespace pplhip
 
 using namespace pplhip;
+
+extern "C" pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_out, int32_t workgroups,
+                                                uint64_t* bytes_read, void* stream) {
+    if (!d_src || !d_out || workgroups <= 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "probe: null buffer or no workgroups");
+    if (((uintptr_t)d_src & 15)) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "probe: source must be 16-byte aligned");
+    // whole rounds of 256 lanes x 8 loads x 16 bytes per workgroup
+    const uint64_t round16 = 256ull * kProbeLoadsInFlight;
+    const uint64_t chunk16 = bytes / 16 / (uint64_t)workgroups / round16 * round16;
+    if (chunk16 == 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "probe: buffer too small for %d workgroups", workgroups);
+    hipLaunchKernelGGL(probe_hbm_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4_probe_t*)d_src, chunk16, (uint32_t*)d_out);
+    PPLHIP_CHECK_LAUNCH("probe_hbm_read");
+    if (bytes_read) *bytes_read = chunk16 * 16 * (uint64_t)workgroups;
+    return PPLHIP_RC_SUCCESS;
+}
 
 extern "C" pplhip_retcode pplhip_probe_mfma_f16(const void* d_operands, void* d_out, int32_t workgroups,
                                                 int32_t iterations, double* flops, void* stream) {
