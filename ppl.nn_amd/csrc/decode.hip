@@ -853,10 +853,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave, 2) void decode_int8kv_kernel(c
 
 // One workgroup per (decode sequence, query head): kMergeGroups groups of 32 lanes stride over the partial slots of the
 // sequence (one per range it touches), each lane owning 4 channels; the groups' running (max, sum, acc) are combined
-// through LDS. Eight groups where sequences span dozens of ranges (each step of a group is a memory round trip), four
-// where they span a few (half the waves to launch: 5.8 -> 4.8 us on 120 sequences over 256 ranges). out[d] = sum_s w_s acc_s[d] / sum_s w_s l_s with w_s = exp2(m_s - max_s m_s). Sequences that lie inside a
-// single range were already written by the decode kernel.
-template <int kMergeGroups>
+// through LDS. Every step of a group is a memory round trip for four slots, so the group count follows the slots per
+// sequence: sixteen where sequences span dozens of ranges (63 slots: one round trip), four where they span a few (half
+// the waves to launch: 5.8 -> 4.8 us on 120 sequences over 256 ranges).
+// out[d] = sum_s w_s acc_s[d] / sum_s w_s l_s with w_s = exp2(m_s - max_s m_s). Sequences that lie inside a single
+// range were already written by the decode kernel.
+template <int kMergeGroups, int kSlotsPerStep>
 __global__ __launch_bounds__(32 * kMergeGroups) void decode_merge_kernel(const DecodeParams p) {
     __shared__ float red[kMergeGroups][kDh + 2];
     const int head = blockIdx.x;
@@ -881,37 +883,32 @@ __global__ __launch_bounds__(32 * kMergeGroups) void decode_merge_kernel(const D
     if (s_lo == s_hi) return;
     float mx = -INFINITY, l = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    // four slots per step, their loads issued together: a long sequence has dozens of slots per lane group, and one
-    // memory latency per slot would add up; what is left after the full steps goes one slot at a time
-    int64_t s = s_lo + g;
-    for (; s + 3 * kMergeGroups <= s_hi; s += 4 * kMergeGroups) {
-        float mc[4], lc[4];
-        float4_t a[4];
+    // kSlotsPerStep slots per step, their loads issued together: a long sequence has dozens of slots per lane group,
+    // and one memory latency per slot would add up. A step that runs past the sequence's last slot re-reads that slot
+    // and gives it no weight, so that every step is the same loads (a remainder walked one slot at a time cost some
+    // lane groups three more round trips on sequences of 63 slots). Where sequences have a handful of slots a lane
+    // group gets one or two of them and takes them one at a time.
+    for (int64_t s = s_lo + g; s <= s_hi; s += kSlotsPerStep * kMergeGroups) {
+        float mc[kSlotsPerStep], lc[kSlotsPerStep];
+        float4_t a[kSlotsPerStep];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t prow = (s + u * kMergeGroups + b) * p.num_heads + head;
+        for (int u = 0; u < kSlotsPerStep; ++u) {
+            const int64_t su = s + u * kMergeGroups;
+            const int64_t prow = ((su <= s_hi ? su : s_hi) + b) * p.num_heads + head;
             mc[u] = p.part_ml[prow * 2];
             lc[u] = p.part_ml[prow * 2 + 1];
             a[u] = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
+            if (su > s_hi) mc[u] = -INFINITY;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kSlotsPerStep; ++u) {
             const float m_new = fmaxf(mx, mc[u]);
+            // (the first slot of a lane group is always a real one, so m_new is finite from there on)
             const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc[u] - m_new);
             acc = acc * w_old + a[u] * w_new;
             l = l * w_old + lc[u] * w_new;
             mx = m_new;
         }
-    }
-    for (; s <= s_hi; s += kMergeGroups) {
-        const int64_t prow = (s + b) * p.num_heads + head;
-        const float mc = p.part_ml[prow * 2], lc = p.part_ml[prow * 2 + 1];
-        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * kDh + d4);
-        const float m_new = fmaxf(mx, mc);
-        const float w_old = __builtin_amdgcn_exp2f(mx - m_new), w_new = __builtin_amdgcn_exp2f(mc - m_new);
-        acc = acc * w_old + a * w_new;
-        l = l * w_old + lc * w_new;
-        mx = m_new;
     }
     red[g][d4 + 0] = acc[0];
     red[g][d4 + 1] = acc[1];
@@ -1012,10 +1009,14 @@ static pplhip_retcode decode_setup(const pplhip_mhca_args* a, const pplhip_mhca_
 // many sequences there are (2048 short sequences launched 65k workgroups that all left at once: 35 us)
 static pplhip_retcode launch_decode_merge(const DecodeParams& p, hipStream_t stream) {
     const dim3 grid(p.num_heads, p.merge_by_boundary ? p.num_ranges - 1 : p.nd);
-    if (p.num_ranges >= 16 * p.nd)
-        hipLaunchKernelGGL(decode_merge_kernel<8>, grid, dim3(256), 0, stream, p);
+    // lane groups per workgroup by the slots a sequence has on average (ranges / sequences + 1): with dozens of slots
+    // every group takes four per memory round trip, with a handful one
+    if (p.num_ranges >= 32 * p.nd)
+        hipLaunchKernelGGL((decode_merge_kernel<16, 4>), grid, dim3(512), 0, stream, p);
+    else if (p.num_ranges >= 16 * p.nd)
+        hipLaunchKernelGGL((decode_merge_kernel<8, 4>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL(decode_merge_kernel<4>, grid, dim3(128), 0, stream, p);
+        hipLaunchKernelGGL((decode_merge_kernel<4, 1>), grid, dim3(128), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("decode_merge");
     return PPLHIP_RC_SUCCESS;
 }
