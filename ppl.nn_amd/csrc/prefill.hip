@@ -351,7 +351,8 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const Prefill
     // m_ref: reference maximum of the RAW scores (before the exp2 scaling) that the probabilities are taken against
     float m_ref = -INFINITY, l_part = 0.f;
 
-    const int64_t wave_last_vis = p.is_causal ? sp + q0 + 32 * wave + 31 : kvlen; // last key any row of this wave sees
+    // last key any row of this wave sees (none when all its rows lie past the end of the sequence)
+    const int64_t wave_last_vis = q0 + 32 * wave >= L ? -1 : (p.is_causal ? sp + q0 + 32 * wave + 31 : kvlen);
     const int64_t wave_first_vis = p.is_causal ? sp + q0 + 32 * wave : kvlen; // keys <= this are seen by all its rows
     const int64_t vis = p.is_causal ? sp + row : kvlen; // last visible key of this lane's row
     const int64_t last_key = vis < kvlen - 1 ? vis : kvlen - 1; // last key this lane's row may attend to
@@ -827,6 +828,10 @@ __device__ __forceinline__ void prefill_workgroup(const PrefillParams& p, uint32
     // tiles this wave computes: those with a key some row of the wave sees (a prefix of the workgroup's tiles)
     int n_act = (int)(wave_last_vis / kBN) + 1;
     if (n_act > nkv) n_act = nkv;
+    // a wave whose 32 rows all lie past the end of the sequence (the last query tile of a sequence is rarely full)
+    // computes nothing: it only takes part in the transfers and the barriers, and leaves the matrix cores to the
+    // workgroup it shares the CU with
+    if (q0 + 32 * wave >= L) n_act = 0;
 
     // ---- per-lane LDS read offsets (relative to the slot)
     // K operand of step (blk, kk): row 32*blk + n, chunk 2*kk + hb, stored at position chunk ^ (n & 15), which is
