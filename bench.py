@@ -377,6 +377,58 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
             "decode_GBps_if_step_were_decode_only": dec_bytes / (ms * steps * 1e-3) / 1e9}
 
 
+def rope_cache_write(pkg, lib, b):
+    """RotaryPositionEmbedding followed by the quantize-on-write of the same new tokens (two launches) against the
+    one launch that does both, on the packed new tokens of batch `b` (decode tokens and prompts); HBM-bound streaming:
+    the algorithmic bytes are Q, K read + written, V read, and the int8 + scale bytes written."""
+    import torch
+    from ppl_nn_amd import cabi
+    S, H, KVH, Dh = b.total_new_tokens, b.num_heads, b.num_kv_heads, b.head_dim
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    q = torch.randn((S, H, Dh), generator=g, **f16)
+    k = torch.randn((S, KVH, Dh), generator=g, **f16)
+    v = torch.randn((S, KVH, Dh), generator=g, **f16)
+    qo, ko = torch.empty_like(q), torch.empty_like(k)
+    i64 = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).cuda()
+    ss, sp, cs = i64(b.seqstarts), i64(b.start_pos), i64(b.cachestarts)
+    cache = torch.zeros((b.max_tokens, 1, 2, KVH, Dh), dtype=torch.int8, device="cuda")
+    scale = torch.zeros((b.max_tokens, 1, 2, KVH, Dh // 8), **f16)
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    r = cabi.RopeArgs()
+    r.d_query, r.d_key, r.d_start_pos, r.d_seqstarts = ptr(q), ptr(k), ptr(sp), ptr(ss)
+    r.theta, r.bypass_key, r.rotary_dim, r.pair_layout = 500000.0, 0, 0, 0
+    r.batch, r.total_tokens, r.num_heads, r.num_key_heads, r.head_dim = b.batch, S, H, KVH, Dh
+    r.max_position_embeddings, r.max_seqlen, r.scaling_type, r.scaling_factor = 8192, b.max_seqlen, 0, 1.0
+    r.d_rotated_query, r.d_rotated_key = ptr(qo), ptr(ko)
+    w = cabi.KvWriteArgs()
+    w.d_current_key, w.d_current_value = ptr(ko), ptr(v)
+    w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(ss), ptr(cs), ptr(sp)
+    w.batch, w.total_new_tokens, w.layer_idx, w.num_layer, w.num_kv_heads, w.head_dim = b.batch, S, 0, 1, KVH, Dh
+    for kk, vv in cabi.cache_strides_layout0(1, KVH, Dh).items():
+        setattr(w, kk, vv)
+    w.d_cache, w.d_scale = ptr(cache), ptr(scale)
+
+    def two(i):
+        rc = lib.pplhip_rope_forward(C.byref(r), stream) or lib.pplhip_kv_quantize_write(C.byref(w), stream)
+        if rc:
+            pkg.check(rc, "rope + write")
+
+    def one(i):
+        rc = lib.pplhip_rope_kv_write_forward(C.byref(r), C.byref(w), stream)
+        if rc:
+            pkg.check(rc, "rope_kv_write")
+
+    _, two_ms, _ = timed_robust(two, min_ms=50.0)
+    _, one_ms, n = timed_robust(one, min_ms=50.0)
+    byts = S * (2 * (H + KVH) * Dh * 2 + KVH * Dh * 2 + 2 * KVH * (Dh + Dh // 4))
+    return {"workload": "new tokens of the mixed batch: %d tokens, H%d/KVH%d/Dh%d" % (S, H, KVH, Dh),
+            "two_launches_us": two_ms * 1e3, "one_launch_us": one_ms * 1e3, "calls_timed": n,
+            "algorithmic_bytes": byts, "one_launch_GBs": byts / (one_ms * 1e-3) / 1e9}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -468,6 +520,7 @@ def main():
         result["fused_mixed_call_ms"] = mix_med
         result["fused_mixed_call_ms_mean"] = mix_mean
         del mixed
+        result["rope_cache_write"] = rope_cache_write(pkg, lib, full)
     if args.workload == "cfg2" and not args.no_churn:
         del dec.slabs[1:], dec.args[1:]
         torch.cuda.empty_cache()

@@ -323,6 +323,20 @@ typedef struct pplhip_rope_args {
 pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* args, void* stream);
 
 /*
+ * RotaryPositionEmbedding and the quantize-on-write of the same new tokens in ONE launch: what pplhip_rope_forward
+ * followed by pplhip_kv_quantize_write (with `write->d_current_key` = `rope->d_rotated_key`) leaves behind, bit for
+ * bit -- rotated_query, rotated_key, and the int8 bytes + fp16 scales of the rotated keys and of
+ * `write->d_current_value` at the new tokens' slab positions. The reference runs the two steps as separate operators
+ * (rotary_position_embedding_kernel.cc:110-132, then the cache write inside multi_head_cache_attention_kernel.cc:230);
+ * here the 8 channels a lane rotates are one quantisation group, so the key rows are quantised from the registers
+ * they are stored from and K and V are read once. `write->d_current_key` is not read. Both argument blocks must
+ * describe the same tokens: same batch, token count, key heads, head_dim and the same seqstarts / start_pos pointers
+ * (PPLHIP_RC_INVALID_VALUE otherwise). A MultiHeadCacheAttention call that follows may write the same tokens again
+ * (its kernels quantise the new tokens themselves): the bytes are the same.
+ */
+pplhip_retcode pplhip_rope_kv_write_forward(const pplhip_rope_args* rope, const pplhip_kv_write_args* write, void* stream);
+
+/*
  * opmx.dynamic_batching::PositionIndex (`dynamic_batching_position_index` as called from
  * src/ppl/nn/engines/llm_cuda/kernels/opmx/dynamic_batching/position_index_kernel.cc:60-67):
  * position_idx[t] = start_pos[b] + (t - seqstarts[b]) for every packed token t of sequence b; i64 [total_tokens].

@@ -125,6 +125,7 @@ PROTOTYPES = {
     "pplhip_mhca_forward_noalloc": (_i32, [C.POINTER(MhcaArgs), C.POINTER(MhcaPlan), _p]),
     "pplhip_mha_forward": (_i32, [C.POINTER(MhaArgs), _p]),
     "pplhip_rope_forward": (_i32, [C.POINTER(RopeArgs), _p]),
+    "pplhip_rope_kv_write_forward": (_i32, [C.POINTER(RopeArgs), C.POINTER(KvWriteArgs), _p]),
     "pplhip_position_index": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
     "pplhip_kv_quantize_write": (_i32, [C.POINTER(KvWriteArgs), _p]),
     "pplhip_kv_cache_forward": (_i32, [C.POINTER(KvCacheArgs), _p]),

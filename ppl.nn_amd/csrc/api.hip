@@ -321,7 +321,9 @@ pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {
     return launch_mha(a, (hipStream_t)stream);
 }
 
-pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* a, void* stream) {
+// *empty: nothing to do (no sequences or no tokens)
+static pplhip_retcode validate_rope(const pplhip_rope_args* a, bool* empty) {
+    *empty = false;
     if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
     if (a->scaling_type != PPLHIP_ROPE_SCALING_NONE && a->scaling_type != PPLHIP_ROPE_SCALING_LINEAR &&
         a->scaling_type != PPLHIP_ROPE_SCALING_DYNAMIC)
@@ -348,13 +350,48 @@ pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* a, void* stream) {
     if (a->scaling_type == PPLHIP_ROPE_SCALING_DYNAMIC && (a->max_position_embeddings <= 0 || rotary_dim <= 2))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "dynamic scaling needs max_position_embeddings > 0 and rotary_dim > 2");
     if (a->batch < 0 || a->total_tokens < 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "negative batch or token count");
-    if (a->batch == 0 || a->total_tokens == 0) return PPLHIP_RC_SUCCESS;
+    if (a->batch == 0 || a->total_tokens == 0) {
+        *empty = true;
+        return PPLHIP_RC_SUCCESS;
+    }
     if (!a->d_query || !a->d_key || !a->d_seqstarts || !a->d_start_pos || !a->d_rotated_query || !a->d_rotated_key)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null tensor pointer");
     if (((uintptr_t)a->d_query & 15) || ((uintptr_t)a->d_key & 15) || ((uintptr_t)a->d_rotated_query & 15) ||
         ((uintptr_t)a->d_rotated_key & 15))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "query/key tensors must be 16-byte aligned");
-    return launch_rope(a, (hipStream_t)stream);
+    return PPLHIP_RC_SUCCESS;
+}
+
+pplhip_retcode pplhip_rope_forward(const pplhip_rope_args* a, void* stream) {
+    bool empty;
+    const pplhip_retcode rc = validate_rope(a, &empty);
+    if (rc != PPLHIP_RC_SUCCESS || empty) return rc;
+    return launch_rope(a, nullptr, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_rope_kv_write_forward(const pplhip_rope_args* a, const pplhip_kv_write_args* w, void* stream) {
+    bool empty;
+    pplhip_retcode rc = validate_rope(a, &empty);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    if (!w) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
+    {
+        pplhip_kv_write_args checked = *w; // (the keys that are quantised are the rotated ones: current_key is not read)
+        checked.d_current_key = a->d_rotated_key;
+        rc = validate_write(&checked);
+        if (rc != PPLHIP_RC_SUCCESS) return rc;
+    }
+    // one pass over the new tokens serves both operators: they must describe the same tokens
+    if (w->batch != a->batch || w->total_new_tokens != a->total_tokens || w->num_kv_heads != a->num_key_heads ||
+        w->head_dim != a->head_dim)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE,
+                    "rotary embedding + cache write: batch %lld/%lld, tokens %lld/%lld, key heads %d/%d, head_dim %d/%d differ",
+                    (long long)a->batch, (long long)w->batch, (long long)a->total_tokens, (long long)w->total_new_tokens,
+                    a->num_key_heads, w->num_kv_heads, a->head_dim, w->head_dim);
+    if (empty) return PPLHIP_RC_SUCCESS;
+    if (w->d_seqstarts != a->d_seqstarts || w->d_start_pos != a->d_start_pos)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "rotary embedding + cache write: both must use the same seqstarts / start_pos");
+    if (a->head_dim > 256) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "rotary embedding + cache write: head_dim at most 256");
+    return launch_rope(a, w, (hipStream_t)stream);
 }
 
 pplhip_retcode pplhip_position_index(const int64_t* d_start_pos, const int64_t* d_seqstarts, int64_t batch,

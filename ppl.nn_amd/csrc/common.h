@@ -148,7 +148,8 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream);
 bool generic_head_dim_supported(int head_dim);
 pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, hipStream_t stream);
 pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream);
-pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream);
+// w != null: the launch also quantises the rotated keys and the values of the new tokens into the slab
+pplhip_retcode launch_rope(const pplhip_rope_args* a, const pplhip_kv_write_args* w, hipStream_t stream);
 pplhip_retcode launch_position_index(const int64_t* d_seqstarts, const int64_t* d_start_pos, int64_t batch,
                                      int64_t total_tokens, int64_t* d_out, hipStream_t stream);
 pplhip_retcode launch_pack_tables(const pplhip_pack_args* a, hipStream_t stream);

@@ -6,6 +6,12 @@
 // reduced mod 2*pi before it is narrowed), because a float32 product loses the low bits of a 100k-token position.
 // Pair i rotates by position * theta^(-2i / rotary_dim); its two channels are (2i, 2i + 1) or (i, i + rotary_dim / 2),
 // the caller's pair_layout; channels >= rotary_dim pass through.
+//
+// The same kernel can quantise the new tokens into the KV slab on the way (rope_kernel<true>): the 8 channels a lane
+// rotates are exactly one quantisation group, so the rotated key group is quantised from the registers it is written
+// to rotated_key from (the fp16-rounded values, i.e. the bytes are those of quantising rotated_key afterwards), and the
+// value rows ride along as rows that are only quantised. One launch then replaces the rotary launch and the
+// quantize-on-write launch, and the key and value rows are read once instead of twice.
 #include "common.h"
 
 namespace pplhip {
@@ -26,10 +32,17 @@ struct RopeParams {
     int32_t max_position_embeddings;
     double log2_theta;
     double scaling_factor;
+    // rope_kernel<true> only: where the new tokens' K (rotated) and V go in the slab
+    const half_t* v; // current_value [S, num_key_heads, head_dim]
+    int8_t* cache;
+    half_t* scale;
+    PageMap pages;
+    CacheAddr addr;
 };
 
 constexpr double kTwoPi = 6.283185307179586476925286766559;
 
+template <bool WRITE_KV>
 __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     const int64_t t = blockIdx.x; // packed token
     const int cpr = p.head_dim / 8; // 16-byte chunks per head row
@@ -38,7 +51,9 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     const int chunk = threadIdx.x - slot * cpr;
     if (slot >= rows_per_pass) return;
 
-    const int b = find_sequence(p.seqstarts, p.batch, t);
+    // (every lane of the workgroup looks for the same token: one table read per lane and a count, one memory round
+    // trip instead of a binary search's chain of them)
+    const int b = find_sequence_wave(p.seqstarts, p.batch, t);
     const int64_t s0 = p.seqstarts[b];
     const int64_t sp = p.start_pos[b];
     double pos = (double)(sp + (t - s0));
@@ -73,15 +88,18 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
             }
         }
     }
-    const int rows = p.num_heads + p.num_key_heads;
+    // rows of a token: query heads, key heads and, when the launch also fills the slab, value heads
+    const int rows = p.num_heads + p.num_key_heads * (WRITE_KV ? 2 : 1);
+    const int64_t slab_tok = WRITE_KV ? p.pages.token(b, sp + (t - s0)) : 0;
     for (int r = slot; r < rows; r += rows_per_pass) {
-        const bool is_key = r >= p.num_heads;
-        const int head = is_key ? r - p.num_heads : r;
-        const int64_t off = ((t * (is_key ? p.num_key_heads : p.num_heads) + head) * (int64_t)p.head_dim) + 8 * chunk;
-        const half_t* src = is_key ? p.k : p.q;
+        const bool is_value = WRITE_KV && r >= p.num_heads + p.num_key_heads;
+        const bool is_key = r >= p.num_heads && !is_value;
+        const int head = is_value ? r - p.num_heads - p.num_key_heads : (is_key ? r - p.num_heads : r);
+        const int64_t off = ((t * (is_key || is_value ? p.num_key_heads : p.num_heads) + head) * (int64_t)p.head_dim) + 8 * chunk;
+        const half_t* src = is_value ? p.v : (is_key ? p.k : p.q);
         const uint4 raw = *reinterpret_cast<const uint4*>(src + off);
         uint4 res = raw;
-        if (rotate && !(is_key && p.bypass_key)) {
+        if (rotate && !is_value && !(is_key && p.bypass_key)) {
             half_t x[8], y[8];
             __builtin_memcpy(x, &raw, 16);
             if (p.half_split) {
@@ -104,7 +122,15 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
             }
             __builtin_memcpy(&res, y, 16);
         }
-        *reinterpret_cast<uint4*>((is_key ? p.k_out : p.q_out) + off) = res;
+        if (!is_value) *reinterpret_cast<uint4*>((is_key ? p.k_out : p.q_out) + off) = res;
+        if (WRITE_KV && (is_key || is_value)) {
+            uint2 q;
+            half_t sc;
+            quantize_group8(res, &q, &sc);
+            const int64_t row = p.addr.row(slab_tok, is_value ? 1 : 0, head);
+            *reinterpret_cast<uint2*>(p.cache + row + 8 * chunk) = q;
+            p.scale[row / kQuantGroup + chunk] = sc;
+        }
     }
 }
 
@@ -117,7 +143,9 @@ __global__ __launch_bounds__(256) void position_index_kernel(const int64_t* __re
     out[t] = start_pos[b] + (t - seqstarts[b]);
 }
 
-pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream) {
+// w: null, or where the launch also quantises the new tokens to (same tables, key heads and head_dim as `a`: checked
+// by the entry point)
+pplhip_retcode launch_rope(const pplhip_rope_args* a, const pplhip_kv_write_args* w, hipStream_t stream) {
     if (a->total_tokens == 0 || a->batch == 0) return PPLHIP_RC_SUCCESS;
     RopeParams p;
     p.q = (const half_t*)a->d_query;
@@ -138,7 +166,21 @@ pplhip_retcode launch_rope(const pplhip_rope_args* a, hipStream_t stream) {
     p.log2_theta = log2((double)a->theta);
     p.scaling_factor = (double)a->scaling_factor;
     if (a->total_tokens > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "rotary embedding: too many tokens");
-    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a->total_tokens), dim3(256), 0, stream, p);
+    p.v = nullptr;
+    p.cache = nullptr;
+    p.scale = nullptr;
+    p.pages = PageMap{nullptr, 0, 0};
+    p.addr = CacheAddr{0, 0, 0, 0, 0};
+    if (w) {
+        p.v = (const half_t*)w->d_current_value;
+        p.cache = (int8_t*)w->d_cache;
+        p.scale = (half_t*)w->d_scale;
+        p.pages = PageMap{w->d_cachestarts, w->cachestart_stride_b, page_shift_of(w->cache_mode, w->page_size)};
+        p.addr = CacheAddr{w->cache_stride_s, w->cache_stride_l, w->cache_stride_h, w->cache_stride_kv, w->layer_idx};
+        hipLaunchKernelGGL(rope_kernel<true>, dim3((unsigned)a->total_tokens), dim3(256), 0, stream, p);
+    } else {
+        hipLaunchKernelGGL(rope_kernel<false>, dim3((unsigned)a->total_tokens), dim3(256), 0, stream, p);
+    }
     PPLHIP_CHECK_LAUNCH("rotary_position_embedding");
     return PPLHIP_RC_SUCCESS;
 }

@@ -124,3 +124,81 @@ def test_position_index_bit_exact(hiplib, olib):
                                                        int(seqlens.max()), out.data_ptr(), None), "position_index")
         torch.cuda.synchronize()
         assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("H,KVH,Dh,rd,layout,paged,cache_layout", [
+    (32, 8, 128, 0, cabi.ROPE_PAIRS_INTERLEAVED, False, 0),
+    (32, 8, 128, 64, cabi.ROPE_PAIRS_HALF_SPLIT, True, 0),
+    (6, 2, 64, 0, cabi.ROPE_PAIRS_HALF_SPLIT, False, 3),
+    (4, 4, 256, 0, cabi.ROPE_PAIRS_INTERLEAVED, True, 0),
+])
+def test_rope_with_cache_write_equals_the_two_steps(hiplib, olib, H, KVH, Dh, rd, layout, paged, cache_layout):
+    """pplhip_rope_kv_write_forward against pplhip_rope_forward followed by pplhip_kv_quantize_write over the rotated
+    keys: rotated outputs, int8 bytes and fp16 scales bit for bit (byte work: no tolerance), and the slab bytes also
+    against the CPU oracle's quantisation of the rotated keys the GPU produced."""
+    import torch
+    from ppl_nn_amd import workloads
+    rng = np.random.default_rng(31)
+    seqlens = np.array([1, 1, 37, 1, 130, 5])
+    start = np.array([700, 0, 0, 4095, 900, 31])
+    b = workloads.Batch(H, KVH, Dh, seqlens, start, 0, num_layer=2, layer_idx=1, slack_tokens=3)
+    pl = harness.PagedLayout(b, page_size=64, seed=5) if paged else None
+    T = int(seqlens.sum())
+    print(f"case rope+write H={H} KVH={KVH} Dh={Dh} rotary_dim={rd} layout={layout} paged={paged} cache_layout={cache_layout}",
+          flush=True)
+    q = rng.standard_normal((T, H, Dh)).astype(np.float16)
+    k = rng.standard_normal((T, KVH, Dh)).astype(np.float16)
+    v = rng.standard_normal((T, KVH, Dh)).astype(np.float16)
+    ss = b.seqstarts
+    cs = pl.table if paged else b.cachestarts
+    dq, dk, dv = harness.to_dev(q), harness.to_dev(k), harness.to_dev(v)
+    tabs = (harness.to_dev(ss), harness.to_dev(start.astype(np.int64)))
+    dcs = harness.to_dev(cs)
+    f16 = lambda x: x.cpu().view(torch.int16).numpy()
+    results = []
+    for fused in (False, True):
+        cache, scale = harness.new_slab(b, paged=pl, layout=cache_layout)
+        dc, dsc = harness.to_dev(cache), harness.to_dev(scale)
+        dqo, dko = torch.zeros_like(dq), torch.zeros_like(dk)
+        ra = harness.fill_rope_args(cabi.RopeArgs(), dq, dk, seqlens, start, dqo, dko, ptr=harness.dev_ptr, tables=tabs,
+                                    theta=500000.0, rotary_dim=rd, pair_layout=layout)
+        w = harness.fill_write_args(cabi.KvWriteArgs(), b, dko, dv, tabs[0], tabs[1], dcs, dc, dsc, ptr=harness.dev_ptr,
+                                    paged=pl, layout=cache_layout)
+        if fused:
+            w.d_current_key = None  # not read
+            harness.pkg.check(hiplib.pplhip_rope_kv_write_forward(C.byref(ra), C.byref(w), None), "rope_kv_write")
+        else:
+            harness.pkg.check(hiplib.pplhip_rope_forward(C.byref(ra), None), "rope_forward")
+            harness.pkg.check(hiplib.pplhip_kv_quantize_write(C.byref(w), None), "kv_quantize_write")
+        torch.cuda.synchronize()
+        results.append((f16(dqo), f16(dko), dc.cpu().numpy(), f16(dsc)))
+    for name, x, y in zip(("rotated_query", "rotated_key", "cache", "scale"), results[0], results[1]):
+        assert np.array_equal(x, y), f"{name}: the fused launch differs from the two steps"
+    assert (results[1][2] != harness.CACHE_FILL).any()
+    # the oracle's quantisation of those rotated keys (and of the values)
+    ko = results[1][1].view(np.float16)
+    cache, scale = harness.new_slab(b, paged=pl, layout=cache_layout)
+    wo = harness.fill_write_args(cabi.KvWriteArgs(), b, ko, v, ss, start.astype(np.int64), np.ascontiguousarray(cs), cache,
+                                 scale, paged=pl, layout=cache_layout)
+    assert olib.oracle_kv_quantize_write(C.byref(wo)) == 0
+    assert np.array_equal(cache, results[1][2]) and np.array_equal(scale.view(np.int16), results[1][3])
+
+
+def test_rope_with_cache_write_checks_that_both_blocks_agree(hiplib):
+    q = np.zeros((4, 2, 128), np.float16)
+    ptr = lambda t: C.c_void_p(0x1000)
+    a = harness.fill_rope_args(cabi.RopeArgs(), q, q, [4], [0], q, q, ptr=ptr)
+    w = cabi.KvWriteArgs()
+    w.d_current_value, w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(0), a.d_seqstarts, ptr(0), a.d_start_pos
+    w.d_cache, w.d_scale = ptr(0), ptr(0)
+    w.batch, w.total_new_tokens, w.num_layer, w.num_kv_heads, w.head_dim = 1, 4, 1, 2, 128
+    for kk, x in cabi.cache_strides_layout0(1, 2, 128).items():
+        setattr(w, kk, x)
+    w.total_new_tokens = 5
+    assert hiplib.pplhip_rope_kv_write_forward(C.byref(a), C.byref(w), None) == cabi.RC_INVALID_VALUE
+    w.total_new_tokens, w.num_kv_heads = 4, 1
+    assert hiplib.pplhip_rope_kv_write_forward(C.byref(a), C.byref(w), None) == cabi.RC_INVALID_VALUE
+    w.num_kv_heads = 2
+    w.d_start_pos = C.c_void_p(0x2000)
+    assert hiplib.pplhip_rope_kv_write_forward(C.byref(a), C.byref(w), None) == cabi.RC_INVALID_VALUE
+    assert hiplib.pplhip_rope_kv_write_forward(C.byref(a), None, None) == cabi.RC_INVALID_VALUE
