@@ -91,9 +91,16 @@ struct DecodeParams {
 // ranges give a range with many boundaries fewer tokens.
 constexpr int kBoundaryTokens = 32;
 
+// a / b for non-negative a and positive b: positions are nearly always below 2^32, and a 32-bit division is a fraction
+// of the 64-bit one's instructions (neither has hardware behind it)
+__device__ inline int64_t div_positions(int64_t a, int64_t b) {
+    if (((uint64_t)a | (uint64_t)b) >> 32) return a / b;
+    return (int64_t)((uint32_t)a / (uint32_t)b);
+}
+
 // Positions per range: the total is only known on the device. At least 128 so that tiny batches are not shredded.
 __device__ inline int64_t range_tokens(int64_t total, int num_ranges) {
-    int64_t r = (total + num_ranges - 1) / num_ranges;
+    int64_t r = div_positions(total + num_ranges - 1, num_ranges);
     r = (r + 31) & ~(int64_t)31;
     return r < 128 ? 128 : r;
 }
@@ -470,9 +477,9 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
     const int groups = p.kv_heads / p.hpb;
     const int xcd = block & 7;
-    const int64_t j = block >> 3;
-    const int hg = (int)(j % groups);
-    const int64_t s_idx = (j / groups) * 8 + xcd; // range index
+    const uint32_t j = block >> 3;
+    const int hg = (int)(j % (uint32_t)groups);
+    const int64_t s_idx = (int64_t)(j / (uint32_t)groups) * 8 + xcd; // range index
     // (virtual positions: see kBoundaryTokens)
     const const_tab_t kvstarts = (const_tab_t)p.kvstarts, seqstarts = (const_tab_t)p.seqstarts,
                       cachestarts = (const_tab_t)p.cachestarts;
@@ -547,7 +554,8 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
         g.whole_sequence = seg_begin == 0 && g.seg_end == seq_hi - seq_lo;
         g.page_row = PAGED ? cachestarts + (int64_t)b * p.cs_stride_b : nullptr;
         g.qrow = (int32_t)seqstarts[b];
-        int64_t sub = (g.seg_end - seg_begin + tsplits - 1) / tsplits;
+        // (tsplits is 1, 2 or 4; a segment's length fits 32 bits)
+        int64_t sub = (int64_t)((uint32_t)(g.seg_end - seg_begin + tsplits - 1) / (uint32_t)tsplits);
         sub = (sub + kStageTokens - 1) / kStageTokens * kStageTokens;
         g.t_begin = (int32_t)(seg_begin + (int64_t)ts * sub);
         const int64_t t_end = (g.t_begin + sub < g.seg_end) ? g.t_begin + sub : (int64_t)g.seg_end; // may be <= t_begin: none
@@ -874,12 +882,12 @@ __global__ __launch_bounds__(32 * kMergeGroups) void decode_merge_kernel(const D
         if (edge >= total) return;
         b = p.range_first[blockIdx.y + 1]; // the sequence that holds position `edge` (found by the decode kernel)
         const int64_t vb = p.kvstarts[b] + (int64_t)b * kBoundaryTokens;
-        if (vb >= edge || vb / R != blockIdx.y) return; // starts there, or crossed a boundary before this one
+        if (vb >= edge || div_positions(vb, R) != blockIdx.y) return; // starts there, or crossed a boundary before this one
     } else {
         b = blockIdx.y;
     }
     const int64_t vlo = p.kvstarts[b] + (int64_t)b * kBoundaryTokens;
-    const int64_t s_lo = vlo / R, s_hi = (vlo + (p.kvstarts[b + 1] - p.kvstarts[b]) - 1) / R;
+    const int64_t s_lo = div_positions(vlo, R), s_hi = div_positions(vlo + (p.kvstarts[b + 1] - p.kvstarts[b]) - 1, R);
     if (s_lo == s_hi) return;
     float mx = -INFINITY, l = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
