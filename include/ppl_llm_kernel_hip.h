@@ -139,8 +139,11 @@ typedef struct pplhip_mhca_plan {
                                 The caller may clear it before forward to stay on the second route. */
     int32_t prefill_staging_offset_256; /* where the staging rows start in the workspace, in units of 256 bytes */
     int32_t general_kernel; /* 1 = the call runs the general attention kernel (head_dim other than 128, more than 16
-                               query heads per kv head, or an attn_mask): write kernel + one attention launch, no
-                               workspace */
+                               query heads per kv head, or an attn_mask): write kernel + one attention launch */
+    int32_t general_decode_splits; /* general kernel only: pieces the longest decode sequence's keys (max_kvlen) are
+                                      cut into, shorter sequences into as many pieces of that length as they fill
+                                      (partial results go through the workspace and a merge launch); 0 or 1 = none.
+                                      The caller may lower it before forward. */
 } pplhip_mhca_plan;
 
 /* Host-only: validates `args` exactly like the reference wrapper + kernel library would

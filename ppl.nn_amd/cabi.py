@@ -52,7 +52,7 @@ class MhcaPlan(C.Structure):
         ("decode_num_ranges", _i32), ("decode_heads_per_block", _i32), ("decode_waves_per_block", _i32),
         ("prefill_q_tile", _i32), ("prefill_num_q_tiles", _i32),
         ("prefill_staging", _i32), ("prefill_staging_offset_256", _i32),
-        ("general_kernel", _i32),
+        ("general_kernel", _i32), ("general_decode_splits", _i32),
     ]
 
 

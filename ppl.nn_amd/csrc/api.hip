@@ -201,8 +201,10 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "specify_decoding_attn_tpb must be 0, 256 or 512");
 
     if (needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask)) {
-        // write kernel + one launch of the general attention kernel; nothing to plan and no workspace
+        // write kernel + one launch of the general attention kernel (+ the merge of the decode sequences' pieces)
         plan->general_kernel = 1;
+        plan->general_decode_splits = generic_decode_splits(a, device_cu_count());
+        plan->workspace_bytes = (generic_workspace_bytes(a, plan->general_decode_splits) + 255) / 256 * 256;
         return PPLHIP_RC_SUCCESS;
     }
 
@@ -266,7 +268,10 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
         // attend over the slab
         pplhip_retcode rcw = launch_kv_quantize_write(&w, s);
         if (rcw != PPLHIP_RC_SUCCESS) return rcw;
-        return launch_generic_mhca(a, s);
+        if (plan->general_decode_splits < 0 || plan->general_decode_splits > 64 ||
+            generic_workspace_bytes(a, plan->general_decode_splits) > plan->workspace_bytes)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
+        return launch_generic_mhca(a, plan->general_decode_splits, d_workspace, s);
     }
     // the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens) into the
     // slab itself, and the prompt tokens are left to the prefill launch unless it reads them back from the slab

@@ -88,6 +88,39 @@ __device__ inline void quantize_group8(const uint4 raw, uint2* q_out, half_t* s_
     *s_out = s;
 }
 
+// ---- the way back: int8 -> fp16 without a trip through fp32
+__device__ inline half2_t as_half2(uint32_t u) {
+    half2_t h;
+    __builtin_memcpy(&h, &u, 4);
+    return h;
+}
+__device__ inline uint32_t as_u32(half2_t h) {
+    uint32_t u;
+    __builtin_memcpy(&u, &h, 4);
+    return u;
+}
+
+// bytes 0,1 (lo) or 2,3 (hi) of x, each widened to an fp16 bit pattern 0x64bb = 1024 + b
+__device__ inline uint32_t widen_lo(uint32_t x) {
+    return __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
+}
+__device__ inline uint32_t widen_hi(uint32_t x) {
+    return __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
+}
+// (1024 + (q + 128)) - 1152 = q exactly; times the group scale, rounded to fp16
+__device__ inline half2_t dequant2(uint32_t widened, half2_t s2) {
+    const half2_t bias = {(half_t)1152.0f, (half_t)1152.0f};
+    return (as_half2(widened) - bias) * s2;
+}
+// 8 int8 channels (one quantisation group) -> 8 fp16 values times the group scale
+__device__ inline half8_t dequant8(uint32_t w0, uint32_t w1, half_t scale) {
+    const half2_t s2 = {scale, scale};
+    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+    const half2_t a = dequant2(widen_lo(x0), s2), b = dequant2(widen_hi(x0), s2);
+    const half2_t c = dequant2(widen_lo(x1), s2), d = dequant2(widen_hi(x1), s2);
+    return half8_t{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
+}
+
 // first index b in [0, n) with starts[b+1] > x  (starts is a non-decreasing prefix-sum table with n+1 entries)
 __device__ inline int find_sequence(const int64_t* __restrict__ starts, int n, int64_t x) {
     int lo = 0, hi = n;
@@ -146,7 +179,10 @@ pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream);
 // the general attention kernel: any head_dim that is a multiple of 32 up to 256, any number of query heads per kv
 // head, optional attn_mask. The MHCA form reads the slab, which must already hold the call's new tokens.
 bool generic_head_dim_supported(int head_dim);
-pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, hipStream_t stream);
+// nsplit pieces per decode sequence (generic_decode_splits), their partial results in `ws` (generic_workspace_bytes)
+int generic_decode_splits(const pplhip_mhca_args* a, int cu_count);
+uint64_t generic_workspace_bytes(const pplhip_mhca_args* a, int nsplit);
+pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* ws, hipStream_t stream);
 pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream);
 // w != null: the launch also quantises the rotated keys and the values of the new tokens into the slab
 pplhip_retcode launch_rope(const pplhip_rope_args* a, const pplhip_kv_write_args* w, hipStream_t stream);

@@ -113,38 +113,6 @@ typedef const int64_t __attribute__((address_space(4)))* const_tab_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
-__device__ inline half2_t as_half2(uint32_t u) {
-    half2_t h;
-    __builtin_memcpy(&h, &u, 4);
-    return h;
-}
-__device__ inline uint32_t as_u32(half2_t h) {
-    uint32_t u;
-    __builtin_memcpy(&u, &h, 4);
-    return u;
-}
-
-// bytes 0,1 (lo) or 2,3 (hi) of x, each widened to an fp16 bit pattern 0x64bb = 1024 + b
-__device__ inline uint32_t widen_lo(uint32_t x) {
-    return __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
-}
-__device__ inline uint32_t widen_hi(uint32_t x) {
-    return __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
-}
-// (1024 + (q + 128)) - 1152 = q exactly; times the group scale, rounded to fp16
-__device__ inline half2_t dequant2(uint32_t widened, half2_t s2) {
-    const half2_t bias = {(half_t)1152.0f, (half_t)1152.0f};
-    return (as_half2(widened) - bias) * s2;
-}
-// 8 int8 channels (one quantisation group) -> 8 fp16 values times the group scale
-__device__ inline half8_t dequant8(uint32_t w0, uint32_t w1, half_t scale) {
-    const half2_t s2 = {scale, scale};
-    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
-    const half2_t a = dequant2(widen_lo(x0), s2), b = dequant2(widen_hi(x0), s2);
-    const half2_t c = dequant2(widen_lo(x1), s2), d = dequant2(widen_hi(x1), s2);
-    return half8_t{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
-}
-
 // Reductions over the four 16-lane rows of the wave (lanes l, l^16, l^32, l^48) in the vector ALU: the swap
 // instructions hand every lane of a row pair both rows' values, where a shuffle would be a round trip through the LDS
 // pipeline. v_permlane16_swap(x, y) exchanges the odd rows of x with the even rows of y; v_permlane32_swap(x, y) the

@@ -14,6 +14,8 @@
 // path is for coverage, the tuned kernels for speed.
 #include "common.h"
 
+#include <type_traits>
+
 namespace pplhip {
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
@@ -37,25 +39,58 @@ struct GenericParams {
     int32_t is_causal;
     int32_t tiles_max; // row tiles of the longest sequence
     float scale_log2; // log2(e) / sqrt(DH)
+    // Decode sequences (the first `split_seqs`) are cut into pieces of `piece_tokens` keys (whole tiles; at most
+    // `nsplit` of them for the longest sequence), one workgroup each, whose un-normalised results (accumulator,
+    // maximum, sum) go to the workspace and are combined by generic_merge_kernel: one workgroup per (sequence, kv
+    // head) would walk a 4 096-token sequence's 64 tiles one after the other while the short sequences' workgroups are
+    // long gone. A piece that starts past its sequence's end has no workgroup work and no partial result. nsplit 1: no
+    // pieces, no workspace.
+    int32_t nsplit, split_seqs, piece_tokens;
+    // generic_attention_kernel covers sequences [first_seq, batch): the decode sequences before them are
+    // generic_decode_kernel's when it can take them (see there)
+    int32_t first_seq;
+    float* part_o; // [split_seqs * num_heads, nsplit, DH]
+    float* part_ml; // [split_seqs * num_heads, nsplit, 2]
 };
 
 constexpr int kGenRows = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <int DH>
-__global__ __launch_bounds__(256) void generic_attention_kernel(const GenericParams p) {
+__global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : DH <= 192 ? 2 : 1) void generic_attention_kernel(const GenericParams p) {
     constexpr int BN = DH <= 128 ? 64 : 32; // kv tokens per tile
     constexpr int LDK = DH + 8; // halves per LDS row (padding spreads the rows over the banks)
     constexpr int KC = DH / 16;
     constexpr int TB = BN / 16;
-    __shared__ __attribute__((aligned(16))) half_t Ks[BN * LDK];
-    __shared__ __attribute__((aligned(16))) half_t Vs[BN * LDK];
+    __shared__ __attribute__((aligned(16))) half_t lds[2 * BN * LDK];
+    half_t* const Ks = lds;
+    half_t* const Vs = lds + BN * LDK;
 
-    const int64_t blk = blockIdx.x;
-    const int tile = (int)(blk % p.tiles_max);
-    const int64_t rest = blk / p.tiles_max;
-    const int kvh = (int)(rest % p.kv_heads);
-    const int b = (int)(rest / p.kv_heads);
+    // Workgroups go to the chip's 8 XCDs in turn (workgroup i to XCD i % 8). The kv heads of one (sequence, row tile,
+    // piece) sit next to each other in the slab (a token's row of head_dim 64 is half a cache line), so they run on
+    // the same XCD, one after the other in its share of the grid; the (sequence, tile, piece) groups themselves go
+    // round the XCDs in the order: every sequence's row tiles, then the second pieces of the decode sequences, the
+    // third, ... so that each XCD gets its share of every piece index (pieces with a high index exist for long
+    // sequences only).
+    const int64_t wi = blockIdx.x >> 3;
+    const int kvh = (int)(wi % p.kv_heads);
+    const int64_t group = (wi / p.kv_heads) * 8 + (blockIdx.x & 7);
+    const int64_t whole = (int64_t)(p.batch - p.first_seq) * p.tiles_max;
+    int split = 0, b, tile;
+    if (group < whole) {
+        b = (int)(group / p.tiles_max);
+        tile = (int)(group - (int64_t)b * p.tiles_max);
+        b += p.first_seq;
+    } else {
+        const int64_t extra = group - whole;
+        if (extra >= (int64_t)p.split_seqs * (p.nsplit - 1)) return; // (the grid is rounded up to 8 groups)
+        split = 1 + (int)(extra / p.split_seqs);
+        b = (int)(extra - (int64_t)(split - 1) * p.split_seqs);
+        tile = 0;
+    }
+    // this sequence's keys are shared out among up to nsplit workgroups (a decode sequence: packed token b, its only
+    // one, whose rep <= 64 rows are one tile)
+    const bool pieces = b < p.split_seqs;
     const int64_t s0 = p.seqstarts[b];
     const int64_t L = p.seqstarts[b + 1] - s0;
     const int64_t kv_first = p.kvstarts[b];
@@ -79,7 +114,13 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
     const int64_t all = kvlen - 1;
     const int64_t row_limit = !valid ? -1 : (p.is_causal ? (sp + tok < all ? sp + tok : all) : all);
     const int64_t last_row = (row0 + kGenRows - 1 < rows - 1) ? row0 + kGenRows - 1 : rows - 1;
-    const int64_t kv_end = p.is_causal ? ((sp + last_row / p.rep + 1 < kvlen) ? sp + last_row / p.rep + 1 : kvlen) : kvlen;
+    int64_t kv_end = p.is_causal ? ((sp + last_row / p.rep + 1 < kvlen) ? sp + last_row / p.rep + 1 : kvlen) : kvlen;
+    int64_t kv_begin = 0;
+    if (pieces) { // (a decode sequence: one token, which sees every key)
+        kv_begin = (int64_t)split * p.piece_tokens;
+        if (kv_begin >= kvlen) return; // the merge knows from kvlen that this piece does not exist
+        kv_end = kv_begin + p.piece_tokens < kvlen ? kv_begin + p.piece_tokens : kvlen;
+    }
 
     // Q^T as the B operand of the score product: channels 16 * kc + 4 * g .. + 3 of the lane's row
     half4_t qf[KC];
@@ -166,19 +207,15 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
     // a wave none of whose 16 rows exists (a decode sequence fills rep rows of the tile's 64) only helps to stage the
     // tiles: its arithmetic would be thrown away, and it would take the matrix cores from the waves that have rows
     const bool wave_has_rows = row0 + wave * 16 < rows;
-    fetch(0);
-    for (int64_t kv0 = 0; kv0 < kv_end; kv0 += BN) {
-        __syncthreads(); // everybody has finished reading the previous tile
-        stash();
-        if (kv0 + BN < kv_end) fetch(kv0 + BN);
-        __syncthreads();
-        if (!wave_has_rows) continue;
-
+    // one K/V tile for the lane's row: NTB blocks of 16 tokens from block tb0 on
+    auto tile_step = [&](auto ntb, const int tb0, const int64_t kv0) {
+        constexpr int NTB = decltype(ntb)::value;
         // ---- scores of the lane's row against tokens kv0 + 16 * tb + 4 * g + i, in the exp2 domain
-        float s[TB][4];
+        float s[NTB][4];
         float mx = -INFINITY;
 #pragma unroll
-        for (int tb = 0; tb < TB; ++tb) {
+        for (int t = 0; t < NTB; ++t) {
+            const int tb = tb0 + t;
             float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kc = 0; kc < KC; ++kc) {
@@ -194,7 +231,7 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
                 } else {
                     v = -INFINITY;
                 }
-                s[tb][i] = v;
+                s[t][i] = v;
                 mx = fmaxf(mx, v);
             }
         }
@@ -203,15 +240,15 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
         const float m_new = fmaxf(m_run, mx);
         // a row that has seen nothing but masked keys so far keeps max -inf: its probabilities are zero, not NaN
         const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
-        half4_t pf[TB];
+        half4_t pf[NTB];
         float psum = 0.f;
 #pragma unroll
-        for (int tb = 0; tb < TB; ++tb) {
+        for (int t = 0; t < NTB; ++t) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[tb][i] - m_new);
+                const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[t][i] - m_new);
                 const half_t h = (half_t)e;
-                pf[tb][i] = h;
+                pf[t][i] = h;
                 psum += (float)h; // the sum of what the second product multiplies
             }
         }
@@ -221,7 +258,8 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
         for (int db = 0; db < KC; ++db) {
             o[db] *= alpha;
 #pragma unroll
-            for (int tb = 0; tb < TB; ++tb) {
+            for (int t = 0; t < NTB; ++t) {
+                const int tb = tb0 + t;
                 // V^T operand: lane (block g, j) receives channel 16 * db + j of tokens 16 * tb + 4 * g .. + 3 when
                 // lane 4 * i + c of the block addresses token 16 * tb + 4 * g + i, channels 16 * db + 4 * c .. + 3
                 const half_t* src = &Vs[(16 * tb + 4 * g + (r_lane >> 2)) * LDK + 16 * db + 4 * (r_lane & 3)];
@@ -229,14 +267,34 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
                     __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)src);
                 half4_t a;
                 __builtin_memcpy(&a, &raw, 8);
-                o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf[tb], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf[t], o[db], 0, 0, 0);
             }
         }
+    };
+    fetch(kv_begin);
+    for (int64_t kv0 = kv_begin; kv0 < kv_end; kv0 += BN) {
+        __syncthreads(); // everybody has finished reading the previous tile
+        stash();
+        if (kv0 + BN < kv_end) fetch(kv0 + BN);
+        __syncthreads();
+        if (!wave_has_rows) continue;
+        tile_step(std::integral_constant<int, TB>{}, 0, kv0);
     }
     float l = l_part;
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     if (!valid) return;
+    if (pieces) {
+        const int64_t prow = ((int64_t)b * p.num_heads + head) * p.nsplit + split;
+        float* dst = p.part_o + prow * DH + 4 * g;
+#pragma unroll
+        for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[db];
+        if (g == 0) {
+            p.part_ml[prow * 2] = m_run; // -inf for a piece without (unmasked) keys: weight 0 in the merge
+            p.part_ml[prow * 2 + 1] = l;
+        }
+        return;
+    }
     // a row whose keys were all masked out has no distribution: zeros
     const float inv_l = l > 0.f ? 1.0f / l : 0.f;
     half_t* dst = p.out + ((s0 + tok) * p.num_heads + head) * DH + 4 * g;
@@ -248,9 +306,291 @@ __global__ __launch_bounds__(256) void generic_attention_kernel(const GenericPar
     }
 }
 
+// ---- decode sequences with no more than 16 query heads per kv head: a wave per (sequence, kv head, piece of keys)
+//
+// The tile kernel above would give such a sequence one wave of arithmetic and three that only stage tiles and wait at
+// its two barriers per tile. Here every wave works alone, with no barrier at all: it walks its piece 16 tokens at a
+// time, the int8 rows and scales of the next kBlocksAhead blocks already requested (straight into registers, in program
+// order, so that waiting for the oldest block leaves the younger ones in flight).
+//   S^T = K Q^T   A = K[token m][channels]: lane (m = lane & 15, g = lane >> 4) loads the g-th quarter of the token's
+//                 row and takes 4 of its int8 per 16-channel step of the product; which channels a step multiplies
+//                 does not matter as long as the query operand is loaded in the same order, so K never passes through
+//                 LDS;
+//   O^T += V^T P^T  needs 4 tokens of one channel per lane: the wave's own LDS region takes the dequantised block
+//                 [16 tokens][DH] and gives it back transposed (ds_read_b64_tr_b16), as in the tile kernel.
+// Whole sequences (nsplit 1) are normalised and written; pieces leave (accumulator, maximum, sum) for the merge.
+// Paged slabs: a block of 16 tokens lies within one page (pages are powers of two of at least 64 tokens, checked at
+// the entry points), so the page's start is one wave-uniform look-up through the constant address space: a scalar
+// load, which does not queue behind the vector loads in flight.
+typedef const int64_t __attribute__((address_space(4)))* gen_const_tab_t;
+
 template <int DH>
-static void launch_one(const GenericParams& p, int64_t blocks, hipStream_t stream) {
-    hipLaunchKernelGGL(generic_attention_kernel<DH>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+struct GenDecodeShape {
+    static constexpr int kBlocksAhead = DH <= 64 ? 4 : DH <= 128 ? 3 : 2;
+    // waves per SIMD the register allocator is to leave room for (one fewer with a mask, whose values travel with
+    // the blocks)
+    static constexpr int kMinWaves = DH <= 64 ? 4 : DH <= 128 ? 3 : 2;
+};
+
+template <int DH, bool MASK>
+__global__ __launch_bounds__(256, GenDecodeShape<DH>::kMinWaves - (MASK && GenDecodeShape<DH>::kMinWaves > 1 ? 1 : 0))
+void generic_decode_kernel(const GenericParams p) {
+    constexpr int KC = DH / 16; // 16-channel steps of a product
+    // A token's row goes to its four lanes by quarters: lane g holds channels g * DH / 4 .. + DH / 4 - 1, as NCK
+    // chunks of 8 int8 (one quantisation group, one 8-byte load each). The first of these loads touches every cache
+    // line of the block's rows; handing the chunks round the four lanes instead (each load covering consecutive bytes
+    // of a row, the lines of a block requested over several loads) measured up to twice slower, and 16-byte chunks
+    // no faster.
+    constexpr int CB = 8;
+    constexpr int NCK = DH / (4 * CB); // chunks per lane
+    typedef uint2 chunk_t;
+    constexpr int LDV = DH + 8; // halves per LDS row
+    constexpr int NB = GenDecodeShape<DH>::kBlocksAhead;
+    __shared__ __attribute__((aligned(16))) half_t lds[4 * 16 * LDV];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r_lane = lane & 15, g = lane >> 4;
+    half_t* const Vs = lds + wave * 16 * LDV;
+
+    // unit -> (piece, sequence, kv head): the kv heads of a (sequence, piece) are neighbours in the slab and in the
+    // grid (waves of one workgroup); first pieces first, so that the pieces only long sequences have come last
+    const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
+    const int kvh = (int)(unit % p.kv_heads);
+    const int64_t item = unit / p.kv_heads;
+    const int piece = (int)(item / p.split_seqs);
+    const int b = (int)(item - (int64_t)piece * p.split_seqs);
+    if (piece >= p.nsplit) return; // (the grid is rounded up to whole workgroups)
+    const gen_const_tab_t seqstarts = (gen_const_tab_t)p.seqstarts, kvstarts = (gen_const_tab_t)p.kvstarts,
+                          cachestarts = (gen_const_tab_t)p.pages.cachestarts;
+    const int64_t s0 = seqstarts[b]; // the sequence's one new token
+    const int64_t kv_first = kvstarts[b];
+    const int64_t kvlen = kvstarts[b + 1] - kv_first;
+    const int64_t kv_begin = (int64_t)piece * p.piece_tokens;
+    if (kv_begin >= kvlen) return; // the merge knows from kvlen that this piece does not exist
+    const int64_t kv_end = kv_begin + p.piece_tokens < kvlen ? kv_begin + p.piece_tokens : kvlen;
+
+    const bool valid = r_lane < p.rep;
+    const int head = kvh * p.rep + (valid ? r_lane : p.rep - 1);
+    half4_t qf[KC];
+    {
+        // step kc of the score product: channels g * DH / 4 + 4 * kc .. + 3
+        const half_t* qp = p.q + (s0 * p.num_heads + head) * DH;
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc)
+            qf[kc] = *reinterpret_cast<const half4_t*>(qp + g * (DH / 4) + 4 * kc);
+    }
+    const half_t* mrow = MASK ? p.mask + (int64_t)head * p.mask_stride_h + s0 * p.mask_stride_q + kv_first : nullptr;
+
+    // a block of 16 tokens as it comes from memory: the lane's quarter of token (block start + r_lane)'s K and V row
+    struct RawBlock {
+        chunk_t k[NCK], v[NCK];
+        uint32_t ks[NCK], vs[NCK]; // the chunks' scales: fp16 bits
+        uint32_t m0, m1, m2, m3; // MASK: the mask values (fp16 bits) of the lane's row for tokens block start + 4 * g .. + 3
+    };
+    RawBlock raw[NB];
+    const int64_t seq_tok0 = p.pages.page_shift == 0 ? cachestarts[b] : 0;
+    const gen_const_tab_t page_row = cachestarts + (int64_t)b * p.pages.stride_b;
+    const int64_t head_off = p.addr.row(0, 0, kvh) + g * (DH / 4); // + token * stride_s (+ stride_kv for V)
+    auto fetch = [&](RawBlock& r, int64_t kv0) {
+        // past the piece's end: its last token again (finite values under a probability of zero)
+        if (kv0 > kv_end - 1) kv0 = (kv_end - 1) & ~int64_t(15);
+        int64_t j = kv0 + r_lane;
+        if (j > kv_end - 1) j = kv_end - 1;
+        int64_t t_slab;
+        if (p.pages.page_shift == 0) {
+            t_slab = seq_tok0 + j;
+        } else {
+            const int64_t page0 = page_row[kv0 >> p.pages.page_shift]; // (kv0: wave-uniform)
+            t_slab = page0 + (j & ((int64_t(1) << p.pages.page_shift) - 1));
+        }
+        const int64_t rk = t_slab * p.addr.stride_s + head_off, rv = rk + p.addr.stride_kv;
+        const uint16_t* sk = reinterpret_cast<const uint16_t*>(p.scale) + rk / kQuantGroup;
+        const uint16_t* sv = reinterpret_cast<const uint16_t*>(p.scale) + rv / kQuantGroup;
+#pragma unroll
+        for (int i = 0; i < NCK; ++i) {
+            r.k[i] = *reinterpret_cast<const chunk_t*>(p.cache + rk + CB * i);
+            r.v[i] = *reinterpret_cast<const chunk_t*>(p.cache + rv + CB * i);
+            r.ks[i] = sk[i];
+            r.vs[i] = sv[i];
+        }
+        if (MASK) {
+            const uint16_t* mp = reinterpret_cast<const uint16_t*>(mrow);
+            const int64_t last = kvlen - 1, j0 = kv0 + 4 * g;
+            r.m0 = mp[j0 < last ? j0 : last];
+            r.m1 = mp[j0 + 1 < last ? j0 + 1 : last];
+            r.m2 = mp[j0 + 2 < last ? j0 + 2 : last];
+            r.m3 = mp[j0 + 3 < last ? j0 + 3 : last];
+        }
+    };
+    auto as_half = [](uint32_t bits16) {
+        const uint16_t bits = (uint16_t)bits16;
+        half_t h;
+        __builtin_memcpy(&h, &bits, 2);
+        return h;
+    };
+
+    float m_run = -INFINITY, l_part = 0.f;
+    float4_t o[KC];
+#pragma unroll
+    for (int i = 0; i < KC; ++i) o[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // A block is taken out of its registers first (V into the wave's LDS rows as fp16, K through the score product:
+    // nothing of it is needed afterwards but the 4 scores and the mask values), so that the same registers can be sent
+    // for a later block before the rest of the arithmetic.
+    float4_t acc;
+    float mask4[4];
+    auto unpack = [&](const RawBlock& r) {
+        acc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NCK; ++i) {
+            *reinterpret_cast<half8_t*>(&Vs[r_lane * LDV + g * (DH / 4) + CB * i]) =
+                dequant8(r.v[i].x, r.v[i].y, as_half(r.vs[i]));
+            const half8_t k8 = dequant8(r.k[i].x, r.k[i].y, as_half(r.ks[i]));
+            const half4_t lo = {k8[0], k8[1], k8[2], k8[3]}, hi = {k8[4], k8[5], k8[6], k8[7]};
+            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(lo, qf[2 * i], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(hi, qf[2 * i + 1], acc, 0, 0, 0);
+        }
+        if (MASK) {
+            mask4[0] = (float)as_half(r.m0) * kLog2e;
+            mask4[1] = (float)as_half(r.m1) * kLog2e;
+            mask4[2] = (float)as_half(r.m2) * kLog2e;
+            mask4[3] = (float)as_half(r.m3) * kLog2e;
+        }
+    };
+    auto block_step = [&](const int64_t kv0) {
+        // ---- scores of the lane's row against tokens kv0 + 4 * g + i, in the exp2 domain
+        float sc[4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t j = kv0 + 4 * g + i;
+            float v = acc[i] * p.scale_log2;
+            if (j < kv_end) {
+                if (MASK) v += mask4[i];
+            } else {
+                v = -INFINITY;
+            }
+            sc[i] = v;
+            mx = fmaxf(mx, v);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        // a row that has seen nothing but masked keys so far keeps max -inf: its probabilities are zero, not NaN
+        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+        half4_t pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[i] - m_new);
+            const half_t h = (half_t)e;
+            pf[i] = h;
+            psum += (float)h; // the sum of what the second product multiplies
+        }
+        l_part = l_part * alpha + psum;
+        m_run = m_new;
+        // the block's V rows, written by the wave's other lanes: LDS operations of one wave complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int db = 0; db < KC; ++db) {
+            o[db] *= alpha;
+            // V^T operand: lane (block g, j) receives channel 16 * db + j of tokens 4 * g .. + 3 when lane 4 * i + c of
+            // the block addresses token 4 * g + i, channels 16 * db + 4 * c .. + 3
+            const half_t* src = &Vs[(4 * g + (r_lane >> 2)) * LDV + 16 * db + 4 * (r_lane & 3)];
+            const short4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)src);
+            half4_t a;
+            __builtin_memcpy(&a, &t, 8);
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf, o[db], 0, 0, 0);
+        }
+        // (the next block's V rows are written after these reads: same wave, in order)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+#pragma unroll
+    for (int u = 0; u < NB; ++u) fetch(raw[u], kv_begin + 16 * u);
+    for (int64_t kv0 = kv_begin; kv0 < kv_end; kv0 += 16 * NB) {
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int64_t kvu = kv0 + 16 * u;
+            if (kvu >= kv_end) break; // wave-uniform
+            unpack(raw[u]);
+            fetch(raw[u], kvu + 16 * NB);
+            block_step(kvu);
+        }
+    }
+
+    float l = l_part;
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    if (!valid) return;
+    if (p.nsplit > 1) {
+        const int64_t prow = ((int64_t)b * p.num_heads + head) * p.nsplit + piece;
+        float* dst = p.part_o + prow * DH + 4 * g;
+#pragma unroll
+        for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[db];
+        if (g == 0) {
+            p.part_ml[prow * 2] = m_run;
+            p.part_ml[prow * 2 + 1] = l;
+        }
+        return;
+    }
+    const float inv_l = l > 0.f ? 1.0f / l : 0.f; // a row whose keys were all masked out: zeros
+    half_t* dst = p.out + (s0 * p.num_heads + head) * DH + 4 * g;
+#pragma unroll
+    for (int db = 0; db < KC; ++db) {
+        const half4_t r = {(half_t)(o[db][0] * inv_l), (half_t)(o[db][1] * inv_l), (half_t)(o[db][2] * inv_l),
+                           (half_t)(o[db][3] * inv_l)};
+        *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
+    }
+}
+
+// Combines the pieces of a decode sequence's row: out = sum_s w_s o_s / sum_s w_s l_s, w_s = exp2(m_s - max m). One
+// wave per row (query head of a decode token), a lane per four channels.
+template <int DH>
+__global__ __launch_bounds__(64) void generic_merge_kernel(const GenericParams p) {
+    const int64_t row = blockIdx.x; // token * num_heads + head over the decode tokens
+    const int d4 = threadIdx.x * 4;
+    if (d4 >= DH) return;
+    const int64_t b = row / p.num_heads;
+    const int64_t kvlen = p.kvstarts[b + 1] - p.kvstarts[b];
+    int n = (int)((kvlen + p.piece_tokens - 1) / p.piece_tokens); // the pieces that exist
+    if (n > p.nsplit) n = p.nsplit;
+    float M = -INFINITY;
+    for (int s = 0; s < n; ++s) M = fmaxf(M, p.part_ml[(row * p.nsplit + s) * 2]);
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;
+    if (M != -INFINITY) { // (all pieces without unmasked keys: the row has no distribution -> zeros)
+        for (int s = 0; s < n; ++s) {
+            const int64_t pr = row * p.nsplit + s;
+            const float w = __builtin_amdgcn_exp2f(p.part_ml[pr * 2] - M);
+            acc += *reinterpret_cast<const float4_t*>(p.part_o + pr * DH + d4) * w;
+            L += p.part_ml[pr * 2 + 1] * w;
+        }
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    const half4_t r = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv), (half_t)(acc[2] * inv), (half_t)(acc[3] * inv)};
+    *reinterpret_cast<half4_t*>(p.out + row * DH + d4) = r;
+}
+
+template <int DH>
+static void launch_one(const GenericParams& p, int64_t blocks, int64_t decode_blocks, hipStream_t stream) {
+    if (decode_blocks > 0) { // the decode sequences, a wave per (sequence, kv head, piece)
+        if (p.mask)
+            hipLaunchKernelGGL((generic_decode_kernel<DH, true>), dim3((unsigned)decode_blocks), dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((generic_decode_kernel<DH, false>), dim3((unsigned)decode_blocks), dim3(256), 0, stream, p);
+    }
+    if (blocks > 0) {
+        GenericParams t = p;
+        if (decode_blocks > 0) t.first_seq = p.split_seqs, t.split_seqs = 0, t.nsplit = 1;
+        hipLaunchKernelGGL(generic_attention_kernel<DH>, dim3((unsigned)blocks), dim3(256), 0, stream, t);
+    }
+    if (p.nsplit > 1 && p.split_seqs > 0)
+        hipLaunchKernelGGL(generic_merge_kernel<DH>, dim3((unsigned)(p.split_seqs * p.num_heads)), dim3(64), 0, stream, p);
 }
 
 bool generic_head_dim_supported(int head_dim) {
@@ -263,26 +603,74 @@ static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max
     p.scale_log2 = kLog2e / sqrtf((float)head_dim);
     const int64_t tiles = (max_seqlen * p.rep + kGenRows - 1) / kGenRows;
     if (tiles <= 0 || p.batch <= 0) return PPLHIP_RC_SUCCESS;
-    const int64_t blocks = tiles * p.kv_heads * (int64_t)p.batch;
-    if (tiles > 0x7fffffffLL || blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many row tiles");
+    // p.split_seqs: the decode sequences (the first of the batch, one new token each, all of whose keys are in the slab)
+    if (p.nsplit < 1) p.nsplit = 1;
+    p.first_seq = 0;
+    int64_t blocks, decode_blocks = 0;
+    if (p.split_seqs > 0 && p.rep <= 16 && (p.pages.page_shift == 0 || p.pages.page_shift >= 4)) {
+        // generic_decode_kernel takes them; the tile kernel the rest of the batch
+        if (p.nsplit == 1) p.piece_tokens = 0x7fffffc0; // the whole sequence
+        decode_blocks = ((int64_t)p.split_seqs * p.nsplit * p.kv_heads + 3) / 4;
+        const int64_t groups = tiles * (int64_t)(p.batch - p.split_seqs);
+        blocks = (groups + 7) / 8 * 8 * p.kv_heads;
+    } else {
+        // the tile kernel takes everything: pieces for decode tokens of one row tile, else whole sequences
+        if (p.nsplit == 1 || p.rep > kGenRows) p.nsplit = 1, p.split_seqs = 0;
+        const int64_t groups = tiles * (int64_t)p.batch + (int64_t)p.split_seqs * (p.nsplit - 1);
+        blocks = (groups + 7) / 8 * 8 * p.kv_heads;
+    }
+    if (tiles > 0x7fffffffLL || blocks > 0x7fffffffLL || decode_blocks > 0x7fffffffLL)
+        PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many row tiles");
     p.tiles_max = (int32_t)tiles;
     switch (head_dim) {
-        case 32: launch_one<32>(p, blocks, stream); break;
-        case 64: launch_one<64>(p, blocks, stream); break;
-        case 96: launch_one<96>(p, blocks, stream); break;
-        case 128: launch_one<128>(p, blocks, stream); break;
-        case 160: launch_one<160>(p, blocks, stream); break;
-        case 192: launch_one<192>(p, blocks, stream); break;
-        case 224: launch_one<224>(p, blocks, stream); break;
-        default: launch_one<256>(p, blocks, stream); break;
+        case 32: launch_one<32>(p, blocks, decode_blocks, stream); break;
+        case 64: launch_one<64>(p, blocks, decode_blocks, stream); break;
+        case 96: launch_one<96>(p, blocks, decode_blocks, stream); break;
+        case 128: launch_one<128>(p, blocks, decode_blocks, stream); break;
+        case 160: launch_one<160>(p, blocks, decode_blocks, stream); break;
+        case 192: launch_one<192>(p, blocks, decode_blocks, stream); break;
+        case 224: launch_one<224>(p, blocks, decode_blocks, stream); break;
+        default: launch_one<256>(p, blocks, decode_blocks, stream); break;
     }
     PPLHIP_CHECK_LAUNCH("generic_attention");
     return PPLHIP_RC_SUCCESS;
 }
 
+// How many pieces the longest decode sequence of a call is cut into (1: no pieces). A piece is one to sixteen tiles of
+// keys: sixteen when even whole sequences would fill the chip many times over (fewer partial results and starts),
+// fewer when the batch is small; more than 64 pieces are not made (the pieces of a very long sequence grow instead). Host-only, a
+// function of the argument block and the CU count.
+constexpr int kGenMaxPieces = 64;
+int generic_decode_splits(const pplhip_mhca_args* a, int cu_count) {
+    // (more than 64 query heads per kv head: a decode token has more than one row tile; left whole)
+    if (a->decoding_batches <= 0 || a->max_kvlen < 2 * 64 || a->num_heads / a->num_kv_heads > kGenRows) return 1;
+    const int64_t tiles = (a->max_kvlen + 63) / 64; // of the longest sequence
+    const int64_t wgs = a->decoding_batches * a->num_kv_heads;
+    int64_t per = wgs * tiles / ((int64_t)cu_count * 32); // tiles a piece: about 32 pieces per CU at the least
+    per = per < 1 ? 1 : per > 16 ? 16 : per;
+    if (per * kGenMaxPieces < tiles) per = (tiles + kGenMaxPieces - 1) / kGenMaxPieces;
+    const int64_t n = (tiles + per - 1) / per;
+    return n < 2 ? 1 : (int)n;
+}
+// keys per piece when the longest sequence (max_kvlen keys) is cut into nsplit pieces: whole tiles
+static int generic_piece_tokens(int64_t max_kvlen, int nsplit) {
+    return (int)(((max_kvlen + nsplit - 1) / nsplit + 63) / 64 * 64);
+}
+uint64_t generic_workspace_bytes(const pplhip_mhca_args* a, int nsplit) {
+    if (nsplit <= 1) return 0;
+    return (uint64_t)a->decoding_batches * a->num_heads * nsplit * (a->head_dim + 2) * sizeof(float);
+}
+
 // MultiHeadCacheAttention through the general kernel; the new tokens are already in the slab.
-pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, hipStream_t stream) {
+pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* ws, hipStream_t stream) {
     GenericParams p;
+    p.nsplit = nsplit < 1 ? 1 : nsplit;
+    p.split_seqs = (int32_t)a->decoding_batches;
+    p.piece_tokens = generic_piece_tokens(a->max_kvlen, p.nsplit);
+    p.part_o = (float*)ws;
+    p.part_ml = p.nsplit > 1 ? (float*)ws + (size_t)a->decoding_batches * a->num_heads * p.nsplit * a->head_dim : nullptr;
+    if (p.nsplit > 1 && ws == nullptr)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "attention: needs the workspace reported by pplhip_mhca_prepare");
     p.q = (const half_t*)a->d_query;
     p.k16 = (const half_t*)a->d_current_key;
     p.v16 = (const half_t*)a->d_current_value;
@@ -311,6 +699,10 @@ pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, hipStream_t stream
 
 pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream) {
     GenericParams p;
+    p.nsplit = 1;
+    p.split_seqs = 0;
+    p.piece_tokens = 0;
+    p.part_o = p.part_ml = nullptr;
     p.q = (const half_t*)a->d_query;
     p.k16 = (const half_t*)a->d_key;
     p.v16 = (const half_t*)a->d_value;

@@ -107,13 +107,24 @@ def test_prepare_rejects(hiplib, mutate, rc):
     lambda a: (setattr(a, "d_attn_mask", 0x10), setattr(a, "attn_mask_stride_q", 64)),
 ])
 def test_prepare_routes_other_shapes_to_the_general_kernel(hiplib, mutate):
-    """head_dim other than 128, more than 16 query heads per kv head, or an attn_mask: the plan says so, needs no
-    workspace and plans no split-k ranges."""
+    """head_dim other than 128, more than 16 query heads per kv head, or an attn_mask: the plan says so and plans no
+    split-k ranges; short decode sequences are not cut into pieces and need no workspace, long ones are and do."""
     a, plan = _valid_args(), cabi.MhcaPlan()
     assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS and plan.general_kernel == 0
     mutate(a)
     assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS, hiplib.pplhip_last_error()
     assert plan.general_kernel == 1 and plan.workspace_bytes == 0 and plan.decode_num_ranges == 0
+    assert plan.general_decode_splits <= 1
+    a.max_kvlen = 4096  # 1 decode sequence: 64 pieces of one tile
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS, hiplib.pplhip_last_error()
+    assert plan.general_kernel == 1 and plan.general_decode_splits == 64 and plan.decode_num_ranges == 0
+    assert plan.workspace_bytes >= 1 * a.num_heads * 64 * (a.head_dim + 2) * 4 and plan.workspace_bytes % 256 == 0
+    a.max_kvlen = 1 << 20  # no more than 64 pieces: they grow instead
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS, hiplib.pplhip_last_error()
+    assert plan.general_decode_splits == 64
+    a.decoding_batches = 0  # no decode sequence, nothing to cut
+    assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS, hiplib.pplhip_last_error()
+    assert plan.general_decode_splits <= 1 and plan.workspace_bytes == 0
 
 
 @pytest.mark.parametrize("kvh", [1, 2, 3, 4, 5, 8, 12, 16, 32, 40, 64])

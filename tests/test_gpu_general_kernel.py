@@ -14,13 +14,16 @@ from test_oracle_attention import _mask_for
 pytestmark = pytest.mark.gpu
 
 
-def check(b, t, what, **kw):
+def check(b, t, what, pieces=None, **kw):
     print(f"case {what}: H={b.num_heads} KVH={b.num_kv_heads} Dh={b.head_dim} B={b.batch} nd={b.decoding_batches} "
           f"S={b.total_new_tokens} hist={b.total_hist_tokens} {sorted(k for k in kw)}", flush=True)
     plans = []
     ref = harness.run_oracle(b, t, **kw)
     got = harness.run_device(b, t, plan_out=plans, **kw)
-    assert plans[0].general_kernel == 1 and plans[0].workspace_bytes == 0
+    assert plans[0].general_kernel == 1
+    assert (plans[0].workspace_bytes == 0) == (plans[0].general_decode_splits <= 1)
+    if pieces is not None:
+        assert plans[0].general_decode_splits == pieces
     assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
     assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
     harness.assert_attn_close(got["output"], ref["output_f64"], what=what)
@@ -52,6 +55,32 @@ def test_attn_mask(Dh, per_head, causal):
     ref, got = check(b, t, f"attn_mask per_head={per_head} causal={causal}", mask=mask)
     plain = harness.run_oracle(b, t)
     assert np.abs(plain["output_f64"] - ref["output_f64"]).max() > 1e-3  # the mask matters
+
+
+@pytest.mark.parametrize("H,KVH,Dh", [(8, 2, 64), (6, 6, 96), (34, 2, 128), (4, 1, 256)])
+def test_long_decode_sequences_are_cut_into_pieces(H, KVH, Dh):
+    """Decode sequences long enough for the plan to share their keys out among several workgroups: pieces that end
+    inside a tile, pieces past a short sequence's end (empty), one sequence of exactly one piece; with a paged slab
+    the same bits."""
+    b = workloads.Batch(H, KVH, Dh, [1] * 6 + [70, 5], [2000, 5, 700, 319, 1300, 255, 0, 0], 6, num_layer=2,
+                        layer_idx=1, name="general_pieces")
+    t = workloads.make_tensors(b, seed=H + Dh)
+    _, flat = check(b, t, f"pieces {H}/{KVH}/{Dh}", pieces=32)  # 2001 keys, a tile each
+    paged = harness.PagedLayout(b, page_size=64, seed=11)
+    _, got = check(b, t, f"pieces, paged slab {H}/{KVH}/{Dh}", pieces=32, paged=paged)
+    assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
+
+
+def test_pieces_with_attn_mask_and_a_fully_masked_piece():
+    b = workloads.Batch(8, 2, 64, [1, 1, 1, 9], [1500, 600, 40, 0], 3, name="general_pieces_mask")
+    t = workloads.make_tensors(b, seed=77)
+    mask = _mask_for(b, np.random.default_rng(5), per_head=True).copy()
+    mask[:, 0, 64:192] = -np.inf  # every key of the first sequence's second and third piece (24 pieces of 64 keys)
+    mask[:, 1, :] = -np.inf  # the second decode sequence sees nothing at all
+    ref, got = check(b, t, "pieces + mask", pieces=24, mask=mask)
+    assert (got["output"][1] == 0).all()
+    plain = harness.run_oracle(b, t)
+    assert np.abs(plain["output_f64"] - ref["output_f64"]).max() > 1e-3
 
 
 def test_attn_mask_with_a_fully_masked_row():
