@@ -71,6 +71,36 @@ def test_long_decode_sequences_are_cut_into_pieces(H, KVH, Dh):
     assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes(seed):
+    """Seeded random head shapes and ragged batches through the general path: decode sequences of 1 .. 1500 cached
+    tokens (pieces or none, sequence ends inside and on block and piece edges), prompts, any number of kv heads (so
+    that a decode workgroup's four waves belong to different sequences and pieces), contiguous / paged / layout 3."""
+    rng = np.random.default_rng(1000 + seed)
+    Dh = int(rng.choice([32, 64, 96, 160, 192, 224, 256]))
+    KVH = int(rng.integers(1, 7))
+    rep = int(rng.choice([1, 2, 3, 4, 7, 8, 16, 17, 33]))
+    nd = int(rng.integers(1, 9))
+    npf = int(rng.integers(0, 3))
+    edges = [1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 319, 320, 321]
+    hist = [int(rng.choice(edges)) - 1 if rng.random() < 0.5 else int(rng.integers(0, 1500)) for _ in range(nd)]
+    seqlens = [1] * nd + [int(rng.integers(1, 150)) for _ in range(npf)]
+    start = hist + [0] * npf
+    causal = int(rng.random() < 0.8)
+    b = workloads.Batch(KVH * rep, KVH, Dh, seqlens, start, nd, num_layer=2, layer_idx=int(rng.integers(0, 2)),
+                        is_causal=causal, slack_tokens=int(rng.integers(0, 3)), name="general_random")
+    t = workloads.make_tensors(b, seed=seed)
+    kw = {}
+    how = int(rng.integers(0, 4))
+    if how == 1:
+        kw["paged"] = harness.PagedLayout(b, page_size=int(rng.choice([64, 128])), seed=seed)
+    elif how == 2:
+        kw["layout"] = 3
+    if rng.random() < 0.3:
+        kw["mask"] = _mask_for(b, rng, per_head=bool(rng.random() < 0.5))
+    check(b, t, f"random shapes, seed {seed}", **kw)
+
+
 def test_pieces_with_attn_mask_and_a_fully_masked_piece():
     b = workloads.Batch(8, 2, 64, [1, 1, 1, 9], [1500, 600, 40, 0], 3, name="general_pieces_mask")
     t = workloads.make_tensors(b, seed=77)
