@@ -324,28 +324,41 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : D
 // load, which does not queue behind the vector loads in flight.
 typedef const int64_t __attribute__((address_space(4)))* gen_const_tab_t;
 
-template <int DH>
+// HP: kv heads per wave. At head_dim 32 and 64 a head's row is a quarter or half of a 128-byte line and its scales an
+// eighth of one, and a wave asking for its head's part alone makes the memory system move every line as often as there
+// are heads in it (measured on the bare loads of 120 sequences: 150 us a head per wave, 103 us two heads per wave at
+// head_dim 64; 123 and 66 us at head_dim 32). With HP = 2 (kv heads next to each other in the slab, their number even)
+// the wave loads both heads' rows as one row of 2 * DH bytes, lane g its quarter: lanes g = 0, 1 hold the halves of
+// the first head, g = 2, 3 those of the second. Each head's score product runs over all four lanes' K operands with
+// that head's query operand set to zero in the other head's lanes.
+template <int DH, int HP>
 struct GenDecodeShape {
-    static constexpr int kBlocksAhead = DH <= 64 ? 4 : DH <= 128 ? 3 : 2;
+    static constexpr int kRowBytes = DH * HP;
+    static constexpr int kBlocksAhead = kRowBytes <= 64 ? 4 : kRowBytes <= 128 ? 3 : 2;
     // waves per SIMD the register allocator is to leave room for (one fewer with a mask, whose values travel with
-    // the blocks)
+    // the blocks; two with two heads' state)
     static constexpr int kMinWaves = DH <= 64 ? 4 : DH <= 128 ? 3 : 2;
 };
 
-template <int DH, bool MASK>
-__global__ __launch_bounds__(256, GenDecodeShape<DH>::kMinWaves - (MASK && GenDecodeShape<DH>::kMinWaves > 1 ? 1 : 0))
+template <int DH, bool MASK, int HP>
+__global__ __launch_bounds__(256, (HP > 1 ? 2 : (GenDecodeShape<DH, HP>::kMinWaves) -
+                                                     (MASK && (GenDecodeShape<DH, HP>::kMinWaves) > 1 ? 1 : 0)))
 void generic_decode_kernel(const GenericParams p) {
-    constexpr int KC = DH / 16; // 16-channel steps of a product
-    // A token's row goes to its four lanes by quarters: lane g holds channels g * DH / 4 .. + DH / 4 - 1, as NCK
-    // chunks of 8 int8 (one quantisation group, one 8-byte load each). The first of these loads touches every cache
-    // line of the block's rows; handing the chunks round the four lanes instead (each load covering consecutive bytes
-    // of a row, the lines of a block requested over several loads) measured up to twice slower, and 16-byte chunks
-    // no faster.
+    constexpr int KC = DH / 16; // 16-channel blocks of a head's output
+    // A token's row (of the wave's HP heads) goes to its four lanes by quarters: lane g holds bytes g * CPL .. + CPL - 1,
+    // as NCK chunks of 8 int8 (one quantisation group, one 8-byte load each). The first of these loads touches every
+    // cache line of the block's rows; handing the chunks round the four lanes instead (each load covering consecutive
+    // bytes of a row, the lines of a block requested over several loads) measured up to twice slower, and 16-byte
+    // chunks no faster.
     constexpr int CB = 8;
-    constexpr int NCK = DH / (4 * CB); // chunks per lane
+    constexpr int CPL = DH * HP / 4; // channels per lane
+    constexpr int NCK = CPL / CB; // chunks per lane
+    constexpr int KS = CPL / 4; // 4-channel steps of a score product per lane
+    constexpr int LPH = 4 / HP; // lanes (of the four) per head
     typedef uint2 chunk_t;
-    constexpr int LDV = DH + 8; // halves per LDS row
-    constexpr int NB = GenDecodeShape<DH>::kBlocksAhead;
+    constexpr int LDV = DH * HP + 8; // halves per LDS row
+    constexpr int NB = GenDecodeShape<DH, HP>::kBlocksAhead;
+    static_assert(HP == 1 || (HP == 2 && DH <= 96), "two heads per wave: their state has to fit the registers");
     __shared__ __attribute__((aligned(16))) half_t lds[4 * 16 * LDV];
 
     const int lane = threadIdx.x & 63;
@@ -353,11 +366,12 @@ void generic_decode_kernel(const GenericParams p) {
     const int r_lane = lane & 15, g = lane >> 4;
     half_t* const Vs = lds + wave * 16 * LDV;
 
-    // unit -> (piece, sequence, kv head): the kv heads of a (sequence, piece) are neighbours in the slab and in the
+    // unit -> (piece, sequence, kv heads): the kv heads of a (sequence, piece) are neighbours in the slab and in the
     // grid (waves of one workgroup); first pieces first, so that the pieces only long sequences have come last
     const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
-    const int kvh = (int)(unit % p.kv_heads);
-    const int64_t item = unit / p.kv_heads;
+    const int head_groups = p.kv_heads / HP;
+    const int kvh = (int)(unit % head_groups) * HP; // the wave's first kv head
+    const int64_t item = unit / head_groups;
     const int piece = (int)(item / p.split_seqs);
     const int b = (int)(item - (int64_t)piece * p.split_seqs);
     if (piece >= p.nsplit) return; // (the grid is rounded up to whole workgroups)
@@ -371,27 +385,34 @@ void generic_decode_kernel(const GenericParams p) {
     const int64_t kv_end = kv_begin + p.piece_tokens < kvlen ? kv_begin + p.piece_tokens : kvlen;
 
     const bool valid = r_lane < p.rep;
-    const int head = kvh * p.rep + (valid ? r_lane : p.rep - 1);
-    half4_t qf[KC];
-    {
-        // step kc of the score product: channels g * DH / 4 + 4 * kc .. + 3
-        const half_t* qp = p.q + (s0 * p.num_heads + head) * DH;
+    int head[HP]; // the lane's query head (row r_lane) of each kv head
+    half4_t qf[HP][KS];
+    const half_t* mrow[HP];
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc)
-            qf[kc] = *reinterpret_cast<const half4_t*>(qp + g * (DH / 4) + 4 * kc);
+    for (int h = 0; h < HP; ++h) {
+        head[h] = (kvh + h) * p.rep + (valid ? r_lane : p.rep - 1);
+        // step kc of head h's score product: the lane's channels 4 * kc .. + 3, which are head g / LPH's channels
+        // (g % LPH) * CPL + 4 * kc .. + 3; zero where the lane holds the other head
+        const half_t* qp = p.q + (s0 * p.num_heads + head[h]) * DH + (g % LPH) * CPL;
+        const bool mine = g / LPH == h;
+#pragma unroll
+        for (int kc = 0; kc < KS; ++kc) {
+            const half4_t x = *reinterpret_cast<const half4_t*>(qp + 4 * kc);
+            qf[h][kc] = mine ? x : half4_t{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        }
+        mrow[h] = MASK ? p.mask + (int64_t)head[h] * p.mask_stride_h + s0 * p.mask_stride_q + kv_first : nullptr;
     }
-    const half_t* mrow = MASK ? p.mask + (int64_t)head * p.mask_stride_h + s0 * p.mask_stride_q + kv_first : nullptr;
 
     // a block of 16 tokens as it comes from memory: the lane's quarter of token (block start + r_lane)'s K and V row
     struct RawBlock {
         chunk_t k[NCK], v[NCK];
         uint32_t ks[NCK], vs[NCK]; // the chunks' scales: fp16 bits
-        uint32_t m0, m1, m2, m3; // MASK: the mask values (fp16 bits) of the lane's row for tokens block start + 4 * g .. + 3
+        uint32_t m[HP][4]; // MASK: the mask values (fp16 bits) of the lane's rows for tokens block start + 4 * g .. + 3
     };
     RawBlock raw[NB];
     const int64_t seq_tok0 = p.pages.page_shift == 0 ? cachestarts[b] : 0;
     const gen_const_tab_t page_row = cachestarts + (int64_t)b * p.pages.stride_b;
-    const int64_t head_off = p.addr.row(0, 0, kvh) + g * (DH / 4); // + token * stride_s (+ stride_kv for V)
+    const int64_t head_off = p.addr.row(0, 0, kvh) + g * CPL; // + token * stride_s (+ stride_kv for V)
     auto fetch = [&](RawBlock& r, int64_t kv0) {
         // past the piece's end: its last token again (finite values under a probability of zero)
         if (kv0 > kv_end - 1) kv0 = (kv_end - 1) & ~int64_t(15);
@@ -415,12 +436,13 @@ void generic_decode_kernel(const GenericParams p) {
             r.vs[i] = sv[i];
         }
         if (MASK) {
-            const uint16_t* mp = reinterpret_cast<const uint16_t*>(mrow);
             const int64_t last = kvlen - 1, j0 = kv0 + 4 * g;
-            r.m0 = mp[j0 < last ? j0 : last];
-            r.m1 = mp[j0 + 1 < last ? j0 + 1 : last];
-            r.m2 = mp[j0 + 2 < last ? j0 + 2 : last];
-            r.m3 = mp[j0 + 3 < last ? j0 + 3 : last];
+#pragma unroll
+            for (int h = 0; h < HP; ++h) {
+                const uint16_t* mp = reinterpret_cast<const uint16_t*>(mrow[h]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) r.m[h][i] = mp[j0 + i < last ? j0 + i : last];
+            }
         }
     };
     auto as_half = [](uint32_t bits16) {
@@ -430,80 +452,96 @@ void generic_decode_kernel(const GenericParams p) {
         return h;
     };
 
-    float m_run = -INFINITY, l_part = 0.f;
-    float4_t o[KC];
+    float m_run[HP], l_part[HP];
+    float4_t o[HP][KC];
 #pragma unroll
-    for (int i = 0; i < KC; ++i) o[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < HP; ++h) {
+        m_run[h] = -INFINITY, l_part[h] = 0.f;
+#pragma unroll
+        for (int i = 0; i < KC; ++i) o[h][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
-    // A block is taken out of its registers first (V into the wave's LDS rows as fp16, K through the score product:
-    // nothing of it is needed afterwards but the 4 scores and the mask values), so that the same registers can be sent
-    // for a later block before the rest of the arithmetic.
-    float4_t acc;
-    float mask4[4];
+    // A block is taken out of its registers first (V into the wave's LDS rows as fp16, K through the score products:
+    // nothing of it is needed afterwards but the 4 scores a head and the mask values), so that the same registers can
+    // be sent for a later block before the rest of the arithmetic.
+    float4_t acc[HP];
+    float mask4[HP][4];
     auto unpack = [&](const RawBlock& r) {
-        acc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int h = 0; h < HP; ++h) acc[h] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
-            *reinterpret_cast<half8_t*>(&Vs[r_lane * LDV + g * (DH / 4) + CB * i]) =
+            *reinterpret_cast<half8_t*>(&Vs[r_lane * LDV + g * CPL + CB * i]) =
                 dequant8(r.v[i].x, r.v[i].y, as_half(r.vs[i]));
             const half8_t k8 = dequant8(r.k[i].x, r.k[i].y, as_half(r.ks[i]));
             const half4_t lo = {k8[0], k8[1], k8[2], k8[3]}, hi = {k8[4], k8[5], k8[6], k8[7]};
-            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(lo, qf[2 * i], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(hi, qf[2 * i + 1], acc, 0, 0, 0);
+#pragma unroll
+            for (int h = 0; h < HP; ++h) {
+                acc[h] = __builtin_amdgcn_mfma_f32_16x16x16f16(lo, qf[h][2 * i], acc[h], 0, 0, 0);
+                acc[h] = __builtin_amdgcn_mfma_f32_16x16x16f16(hi, qf[h][2 * i + 1], acc[h], 0, 0, 0);
+            }
         }
         if (MASK) {
-            mask4[0] = (float)as_half(r.m0) * kLog2e;
-            mask4[1] = (float)as_half(r.m1) * kLog2e;
-            mask4[2] = (float)as_half(r.m2) * kLog2e;
-            mask4[3] = (float)as_half(r.m3) * kLog2e;
+#pragma unroll
+            for (int h = 0; h < HP; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mask4[h][i] = (float)as_half(r.m[h][i]) * kLog2e;
         }
     };
     auto block_step = [&](const int64_t kv0) {
-        // ---- scores of the lane's row against tokens kv0 + 4 * g + i, in the exp2 domain
-        float sc[4];
-        float mx = -INFINITY;
+        half4_t pf[HP];
+        float alpha[HP];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t j = kv0 + 4 * g + i;
-            float v = acc[i] * p.scale_log2;
-            if (j < kv_end) {
-                if (MASK) v += mask4[i];
-            } else {
-                v = -INFINITY;
+        for (int h = 0; h < HP; ++h) {
+            // ---- scores of the lane's row against tokens kv0 + 4 * g + i, in the exp2 domain
+            float sc[4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t j = kv0 + 4 * g + i;
+                float v = acc[h][i] * p.scale_log2;
+                if (j < kv_end) {
+                    if (MASK) v += mask4[h][i];
+                } else {
+                    v = -INFINITY;
+                }
+                sc[i] = v;
+                mx = fmaxf(mx, v);
             }
-            sc[i] = v;
-            mx = fmaxf(mx, v);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // a row that has seen nothing but masked keys so far keeps max -inf: its probabilities are zero, not NaN
-        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
-        half4_t pf;
-        float psum = 0.f;
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run[h], mx);
+            // a row that has seen nothing but masked keys so far keeps max -inf: its probabilities are zero, not NaN
+            alpha[h] = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run[h] - m_new);
+            float psum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[i] - m_new);
-            const half_t h = (half_t)e;
-            pf[i] = h;
-            psum += (float)h; // the sum of what the second product multiplies
+            for (int i = 0; i < 4; ++i) {
+                const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[i] - m_new);
+                const half_t x = (half_t)e;
+                pf[h][i] = x;
+                psum += (float)x; // the sum of what the second product multiplies
+            }
+            l_part[h] = l_part[h] * alpha[h] + psum;
+            m_run[h] = m_new;
         }
-        l_part = l_part * alpha + psum;
-        m_run = m_new;
         // the block's V rows, written by the wave's other lanes: LDS operations of one wave complete in order
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int db = 0; db < KC; ++db) {
-            o[db] *= alpha;
-            // V^T operand: lane (block g, j) receives channel 16 * db + j of tokens 4 * g .. + 3 when lane 4 * i + c of
-            // the block addresses token 4 * g + i, channels 16 * db + 4 * c .. + 3
-            const half_t* src = &Vs[(4 * g + (r_lane >> 2)) * LDV + 16 * db + 4 * (r_lane & 3)];
-            const short4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)src);
-            half4_t a;
-            __builtin_memcpy(&a, &t, 8);
-            o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf, o[db], 0, 0, 0);
+        for (int h = 0; h < HP; ++h) {
+#pragma unroll
+            for (int db = 0; db < KC; ++db) {
+                o[h][db] *= alpha[h];
+                // V^T operand: lane (block g, j) receives channel 16 * db + j of tokens 4 * g .. + 3 when lane
+                // 4 * i + c of the block addresses token 4 * g + i, channels 16 * db + 4 * c .. + 3
+                const half_t* src = &Vs[(4 * g + (r_lane >> 2)) * LDV + h * DH + 16 * db + 4 * (r_lane & 3)];
+                const short4_t t =
+                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)src);
+                half4_t a;
+                __builtin_memcpy(&a, &t, 8);
+                o[h][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf[h], o[h][db], 0, 0, 0);
+            }
         }
         // (the next block's V rows are written after these reads: same wave, in order)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -523,28 +561,31 @@ void generic_decode_kernel(const GenericParams p) {
         }
     }
 
-    float l = l_part;
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
-    if (!valid) return;
-    if (p.nsplit > 1) {
-        const int64_t prow = ((int64_t)b * p.num_heads + head) * p.nsplit + piece;
-        float* dst = p.part_o + prow * DH + 4 * g;
 #pragma unroll
-        for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[db];
-        if (g == 0) {
-            p.part_ml[prow * 2] = m_run;
-            p.part_ml[prow * 2 + 1] = l;
+    for (int h = 0; h < HP; ++h) {
+        float l = l_part[h];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        if (!valid) continue;
+        if (p.nsplit > 1) {
+            const int64_t prow = ((int64_t)b * p.num_heads + head[h]) * p.nsplit + piece;
+            float* dst = p.part_o + prow * DH + 4 * g;
+#pragma unroll
+            for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[h][db];
+            if (g == 0) {
+                p.part_ml[prow * 2] = m_run[h];
+                p.part_ml[prow * 2 + 1] = l;
+            }
+            continue;
         }
-        return;
-    }
-    const float inv_l = l > 0.f ? 1.0f / l : 0.f; // a row whose keys were all masked out: zeros
-    half_t* dst = p.out + (s0 * p.num_heads + head) * DH + 4 * g;
+        const float inv_l = l > 0.f ? 1.0f / l : 0.f; // a row whose keys were all masked out: zeros
+        half_t* dst = p.out + (s0 * p.num_heads + head[h]) * DH + 4 * g;
 #pragma unroll
-    for (int db = 0; db < KC; ++db) {
-        const half4_t r = {(half_t)(o[db][0] * inv_l), (half_t)(o[db][1] * inv_l), (half_t)(o[db][2] * inv_l),
-                           (half_t)(o[db][3] * inv_l)};
-        *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
+        for (int db = 0; db < KC; ++db) {
+            const half4_t r = {(half_t)(o[h][db][0] * inv_l), (half_t)(o[h][db][1] * inv_l),
+                               (half_t)(o[h][db][2] * inv_l), (half_t)(o[h][db][3] * inv_l)};
+            *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
+        }
     }
 }
 
@@ -576,14 +617,30 @@ __global__ __launch_bounds__(64) void generic_merge_kernel(const GenericParams p
     *reinterpret_cast<half4_t*>(p.out + row * DH + d4) = r;
 }
 
+// two kv heads per wave of the decode kernel: head_dim up to 96 (registers), heads next to each other in the slab
+static int generic_decode_heads_per_wave(const GenericParams& p, int head_dim) {
+    return head_dim <= 96 && p.kv_heads % 2 == 0 && p.addr.stride_h == head_dim ? 2 : 1;
+}
+
 template <int DH>
 static void launch_one(const GenericParams& p, int64_t blocks, int64_t decode_blocks, hipStream_t stream) {
-    if (decode_blocks > 0) { // the decode sequences, a wave per (sequence, kv head, piece)
+    if (decode_blocks > 0) { // the decode sequences, a wave per (sequence, kv head or pair of them, piece)
+        const dim3 grid((unsigned)decode_blocks), block(256);
+        if constexpr (DH <= 96) {
+            if (generic_decode_heads_per_wave(p, DH) == 2) {
+                if (p.mask)
+                    hipLaunchKernelGGL((generic_decode_kernel<DH, true, 2>), grid, block, 0, stream, p);
+                else
+                    hipLaunchKernelGGL((generic_decode_kernel<DH, false, 2>), grid, block, 0, stream, p);
+                goto decode_launched;
+            }
+        }
         if (p.mask)
-            hipLaunchKernelGGL((generic_decode_kernel<DH, true>), dim3((unsigned)decode_blocks), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((generic_decode_kernel<DH, true, 1>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((generic_decode_kernel<DH, false>), dim3((unsigned)decode_blocks), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((generic_decode_kernel<DH, false, 1>), grid, block, 0, stream, p);
     }
+decode_launched:
     if (blocks > 0) {
         GenericParams t = p;
         if (decode_blocks > 0) t.first_seq = p.split_seqs, t.split_seqs = 0, t.nsplit = 1;
@@ -610,7 +667,7 @@ static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max
     if (p.split_seqs > 0 && p.rep <= 16 && (p.pages.page_shift == 0 || p.pages.page_shift >= 4)) {
         // generic_decode_kernel takes them; the tile kernel the rest of the batch
         if (p.nsplit == 1) p.piece_tokens = 0x7fffffc0; // the whole sequence
-        decode_blocks = ((int64_t)p.split_seqs * p.nsplit * p.kv_heads + 3) / 4;
+        decode_blocks = ((int64_t)p.split_seqs * p.nsplit * (p.kv_heads / generic_decode_heads_per_wave(p, head_dim)) + 3) / 4;
         const int64_t groups = tiles * (int64_t)(p.batch - p.split_seqs);
         blocks = (groups + 7) / 8 * 8 * p.kv_heads;
     } else {

@@ -131,7 +131,10 @@ def test_cache_prefill_paged_and_layout_3():
     _, got = check(b, t, "cache-prefill, paged slab", cache_prefill=1, paged=paged)
     assert np.array_equal(got["output"].view(np.uint16), flat["output"].view(np.uint16))
     _, got3 = check(b, t, "cache-prefill, cache_layout 3", cache_prefill=1, layout=3)
-    assert np.array_equal(got3["output"].view(np.uint16), flat["output"].view(np.uint16))
+    # (the decode tokens' kernel takes two kv heads per wave where they are neighbours in the slab, one in layout 3:
+    # another order of summation, so those rows are only held to the oracle's tolerance)
+    nd = b.decoding_batches
+    assert np.array_equal(got3["output"][nd:].view(np.uint16), flat["output"][nd:].view(np.uint16))
 
 
 @pytest.mark.parametrize("Dh,mask_on", [(64, False), (96, True), (256, False), (128, True)])
