@@ -589,13 +589,16 @@ void generic_decode_kernel(const GenericParams p) {
     }
 }
 
-// Combines the pieces of a decode sequence's row: out = sum_s w_s o_s / sum_s w_s l_s, w_s = exp2(m_s - max m). One
-// wave per row (query head of a decode token), a lane per four channels.
+// Combines the pieces of a decode sequence's row: out = sum_s w_s o_s / sum_s w_s l_s, w_s = exp2(m_s - max m). A
+// thread per four channels of a row (query head of a decode token), kGenMergeRows<DH> rows to a workgroup.
 template <int DH>
-__global__ __launch_bounds__(64) void generic_merge_kernel(const GenericParams p) {
-    const int64_t row = blockIdx.x; // token * num_heads + head over the decode tokens
-    const int d4 = threadIdx.x * 4;
-    if (d4 >= DH) return;
+constexpr int kGenMergeRows = 256 / (DH / 4);
+template <int DH>
+__global__ __launch_bounds__(256) void generic_merge_kernel(const GenericParams p) {
+    const int r_in_block = threadIdx.x / (DH / 4);
+    const int64_t row = (int64_t)blockIdx.x * kGenMergeRows<DH> + r_in_block; // token * num_heads + head over the decode tokens
+    const int d4 = (threadIdx.x - r_in_block * (DH / 4)) * 4;
+    if (r_in_block >= kGenMergeRows<DH> || row >= (int64_t)p.split_seqs * p.num_heads) return;
     const int64_t b = row / p.num_heads;
     const int64_t kvlen = p.kvstarts[b + 1] - p.kvstarts[b];
     int n = (int)((kvlen + p.piece_tokens - 1) / p.piece_tokens); // the pieces that exist
@@ -647,7 +650,9 @@ decode_launched:
         hipLaunchKernelGGL(generic_attention_kernel<DH>, dim3((unsigned)blocks), dim3(256), 0, stream, t);
     }
     if (p.nsplit > 1 && p.split_seqs > 0)
-        hipLaunchKernelGGL(generic_merge_kernel<DH>, dim3((unsigned)(p.split_seqs * p.num_heads)), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL(generic_merge_kernel<DH>,
+                           dim3((unsigned)(((int64_t)p.split_seqs * p.num_heads + kGenMergeRows<DH> - 1) / kGenMergeRows<DH>)),
+                           dim3(256), 0, stream, p);
 }
 
 bool generic_head_dim_supported(int head_dim) {
