@@ -57,7 +57,7 @@ constexpr int kGenRows = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <int DH>
-__global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : DH <= 192 ? 2 : 1) void generic_attention_kernel(const GenericParams p) {
+__global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2) void generic_attention_kernel(const GenericParams p) {
     constexpr int BN = DH <= 128 ? 64 : 32; // kv tokens per tile
     constexpr int LDK = DH + 8; // halves per LDS row (padding spreads the rows over the banks)
     constexpr int KC = DH / 16;
@@ -132,7 +132,13 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : D
     const half_t* mrow =
         p.mask ? p.mask + (int64_t)head * p.mask_stride_h + (s0 + tok) * p.mask_stride_q + kv_first : nullptr;
 
-    float m_run = -INFINITY, l_part = 0.f;
+    // The running maximum is kept in the domain the scores are held in: raw products (times `cs` = scale_log2 inside
+    // the exponentials) without a mask, exp2-domain values (cs = 1) with one. The row's sum of probabilities comes out
+    // of the matrix cores (a row of ones as the A operand against P^T: every component of l_acc holds it), which also
+    // adds up the four lane groups' shares.
+    const float cs = mrow ? 1.0f : p.scale_log2;
+    float m_run = -INFINITY;
+    float4_t l_acc = {0.f, 0.f, 0.f, 0.f};
     float4_t o[KC];
 #pragma unroll
     for (int i = 0; i < KC; ++i) o[i] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -207,59 +213,68 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : D
     // a wave none of whose 16 rows exists (a decode sequence fills rep rows of the tile's 64) only helps to stage the
     // tiles: its arithmetic would be thrown away, and it would take the matrix cores from the waves that have rows
     const bool wave_has_rows = row0 + wave * 16 < rows;
-    // one K/V tile for the lane's row: NTB blocks of 16 tokens from block tb0 on
-    auto tile_step = [&](auto ntb, const int tb0, const int64_t kv0) {
-        constexpr int NTB = decltype(ntb)::value;
-        // ---- scores of the lane's row against tokens kv0 + 16 * tb + 4 * g + i, in the exp2 domain
-        float s[NTB][4];
+    // one K/V tile for the lane's row
+    auto tile_step = [&](const int64_t kv0) {
+        // keys kv0 .. kv0 + lim of the tile are visible to the lane's row; a tile all of whose keys are visible to all of
+        // the wave's rows (every tile but a causal sequence's last ones, and a ragged tile's) skips the comparisons
+        const int64_t rel = row_limit - kv0;
+        const int lim4 = (int)(rel < -1 ? -1 : rel > BN ? BN : rel) - 4 * g;
+        const bool all_visible = __all(lim4 + 4 * g >= BN - 1);
+        // ---- scores of the lane's row against tokens kv0 + 16 * tb + 4 * g + i
+        float s[TB][4];
         float mx = -INFINITY;
 #pragma unroll
-        for (int t = 0; t < NTB; ++t) {
-            const int tb = tb0 + t;
+        for (int tb = 0; tb < TB; ++tb) {
             float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kc = 0; kc < KC; ++kc) {
                 const half4_t a = *reinterpret_cast<const half4_t*>(&Ks[(16 * tb + r_lane) * LDK + 16 * kc + 4 * g]);
                 acc = __builtin_amdgcn_mfma_f32_16x16x16f16(a, qf[kc], acc, 0, 0, 0);
             }
+            if (mrow) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int64_t j = kv0 + 16 * tb + 4 * g + i;
+                    // (a masked-out key's mask entry is not read: it may lie past the row's end)
+                    acc[i] = 16 * tb + i <= lim4 ? __builtin_fmaf(acc[i], p.scale_log2, (float)mrow[j] * kLog2e) : -INFINITY;
+                }
+            } else if (!all_visible) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] = 16 * tb + i <= lim4 ? acc[i] : -INFINITY;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int64_t j = kv0 + 16 * tb + 4 * g + i;
-                float v = acc[i] * p.scale_log2;
-                if (j <= row_limit) {
-                    if (mrow) v += (float)mrow[j] * kLog2e;
-                } else {
-                    v = -INFINITY;
-                }
-                s[t][i] = v;
-                mx = fmaxf(mx, v);
+                s[tb][i] = acc[i];
+                mx = fmaxf(mx, acc[i]);
             }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float m_new = fmaxf(m_run, mx);
-        // a row that has seen nothing but masked keys so far keeps max -inf: its probabilities are zero, not NaN
-        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
-        half4_t pf[NTB];
-        float psum = 0.f;
+        // a row that has seen nothing but masked keys so far keeps max -inf: against 0 in the exponents its
+        // probabilities are exp2(-inf) = 0, not NaN
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs);
+        const float shift = -m_safe * cs;
+        half4_t pf[TB];
 #pragma unroll
-        for (int t = 0; t < NTB; ++t) {
+        for (int tb = 0; tb < TB; ++tb) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[t][i] - m_new);
-                const half_t h = (half_t)e;
-                pf[t][i] = h;
-                psum += (float)h; // the sum of what the second product multiplies
-            }
+            for (int i = 0; i < 4; ++i) pf[tb][i] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][i], cs, shift));
         }
-        l_part = l_part * alpha + psum;
         m_run = m_new;
+        const half4_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+        if (!__all(alpha == 1.0f)) { // (the maximum has moved for some row of the wave)
+            l_acc *= alpha;
+#pragma unroll
+            for (int db = 0; db < KC; ++db) o[db] *= alpha;
+        }
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) l_acc = __builtin_amdgcn_mfma_f32_16x16x16f16(ones, pf[tb], l_acc, 0, 0, 0);
 #pragma unroll
         for (int db = 0; db < KC; ++db) {
-            o[db] *= alpha;
 #pragma unroll
-            for (int t = 0; t < NTB; ++t) {
-                const int tb = tb0 + t;
+            for (int tb = 0; tb < TB; ++tb) {
                 // V^T operand: lane (block g, j) receives channel 16 * db + j of tokens 16 * tb + 4 * g .. + 3 when
                 // lane 4 * i + c of the block addresses token 16 * tb + 4 * g + i, channels 16 * db + 4 * c .. + 3
                 const half_t* src = &Vs[(16 * tb + 4 * g + (r_lane >> 2)) * LDK + 16 * db + 4 * (r_lane & 3)];
@@ -267,7 +282,7 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : D
                     __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)src);
                 half4_t a;
                 __builtin_memcpy(&a, &raw, 8);
-                o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf[t], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf[tb], o[db], 0, 0, 0);
             }
         }
     };
@@ -278,11 +293,9 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : D
         if (kv0 + BN < kv_end) fetch(kv0 + BN);
         __syncthreads();
         if (!wave_has_rows) continue;
-        tile_step(std::integral_constant<int, TB>{}, 0, kv0);
+        tile_step(kv0);
     }
-    float l = l_part;
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
+    const float l = l_acc[0];
     if (!valid) return;
     if (pieces) {
         const int64_t prow = ((int64_t)b * p.num_heads + head) * p.nsplit + split;
@@ -290,7 +303,7 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : D
 #pragma unroll
         for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[db];
         if (g == 0) {
-            p.part_ml[prow * 2] = m_run; // -inf for a piece without (unmasked) keys: weight 0 in the merge
+            p.part_ml[prow * 2] = m_run * cs; // -inf for a piece without (unmasked) keys: weight 0 in the merge
             p.part_ml[prow * 2 + 1] = l;
         }
         return;
@@ -342,7 +355,7 @@ struct GenDecodeShape {
 
 template <int DH, bool MASK, int HP>
 __global__ __launch_bounds__(256, (HP > 1 ? 2 : (GenDecodeShape<DH, HP>::kMinWaves) -
-                                                     (MASK && (GenDecodeShape<DH, HP>::kMinWaves) > 1 ? 1 : 0)))
+                                                     (MASK && (GenDecodeShape<DH, HP>::kMinWaves) > 2 ? 1 : 0)))
 void generic_decode_kernel(const GenericParams p) {
     constexpr int KC = DH / 16; // 16-channel blocks of a head's output
     // A token's row (of the wave's HP heads) goes to its four lanes by quarters: lane g holds bytes g * CPL .. + CPL - 1,
@@ -452,6 +465,8 @@ void generic_decode_kernel(const GenericParams p) {
         return h;
     };
 
+    constexpr float kOne = 1.0f;
+    const float cs = MASK ? kOne : p.scale_log2; // what the exponentials multiply the held scores by
     float m_run[HP], l_part[HP];
     float4_t o[HP][KC];
 #pragma unroll
@@ -491,33 +506,33 @@ void generic_decode_kernel(const GenericParams p) {
     auto block_step = [&](const int64_t kv0) {
         half4_t pf[HP];
         float alpha[HP];
+        // tokens kv0 + 4 * g + i of the block exist for i < left (only the piece's last block is ragged)
+        const int left = (int)(kv_end - kv0 < 16 ? kv_end - kv0 : 16) - 4 * g;
 #pragma unroll
         for (int h = 0; h < HP; ++h) {
-            // ---- scores of the lane's row against tokens kv0 + 4 * g + i, in the exp2 domain
+            // ---- scores of the lane's row against tokens kv0 + 4 * g + i: raw products without a mask (the scale goes
+            // into the exponentials' multiply-add), exp2-domain values with one
             float sc[4];
             float mx = -INFINITY;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int64_t j = kv0 + 4 * g + i;
-                float v = acc[h][i] * p.scale_log2;
-                if (j < kv_end) {
-                    if (MASK) v += mask4[h][i];
-                } else {
-                    v = -INFINITY;
-                }
+                float v = MASK ? __builtin_fmaf(acc[h][i], p.scale_log2, mask4[h][i]) : acc[h][i];
+                if (kv0 + 16 > kv_end) v = i < left ? v : -INFINITY; // (wave-uniform condition)
                 sc[i] = v;
                 mx = fmaxf(mx, v);
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16));
             mx = fmaxf(mx, __shfl_xor(mx, 32));
             const float m_new = fmaxf(m_run[h], mx);
-            // a row that has seen nothing but masked keys so far keeps max -inf: its probabilities are zero, not NaN
-            alpha[h] = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run[h] - m_new);
+            // a row that has seen nothing but masked keys so far keeps max -inf: against 0 in the exponents its
+            // probabilities are exp2(-inf) = 0, not NaN
+            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+            alpha[h] = __builtin_amdgcn_exp2f((m_run[h] - m_safe) * cs);
+            const float shift = -m_safe * cs;
             float psum = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float e = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[i] - m_new);
-                const half_t x = (half_t)e;
+                const half_t x = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], cs, shift));
                 pf[h][i] = x;
                 psum += (float)x; // the sum of what the second product multiplies
             }
@@ -573,7 +588,7 @@ void generic_decode_kernel(const GenericParams p) {
 #pragma unroll
             for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[h][db];
             if (g == 0) {
-                p.part_ml[prow * 2] = m_run[h];
+                p.part_ml[prow * 2] = m_run[h] * cs; // (the merge works in the exp2 domain)
                 p.part_ml[prow * 2 + 1] = l;
             }
             continue;
