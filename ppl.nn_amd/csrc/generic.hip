@@ -122,12 +122,14 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
         kv_end = kv_begin + p.piece_tokens < kvlen ? kv_begin + p.piece_tokens : kvlen;
     }
 
-    // Q^T as the B operand of the score product: channels 16 * kc + 4 * g .. + 3 of the lane's row
-    half4_t qf[KC];
+    // Q^T as the B operand of the score product (v_mfma_f32_16x16x32_f16: 32 channels a step, 8 of them per lane):
+    // channels 32 * kc + 8 * g .. + 7 of the lane's row
+    constexpr int KC2 = DH / 32;
+    half8_t qf[KC2];
     {
-        const half_t* qp = p.q + ((s0 + tok) * p.num_heads + head) * DH + 4 * g;
+        const half_t* qp = p.q + ((s0 + tok) * p.num_heads + head) * DH + 8 * g;
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc) qf[kc] = *reinterpret_cast<const half4_t*>(qp + 16 * kc);
+        for (int kc = 0; kc < KC2; ++kc) qf[kc] = *reinterpret_cast<const half8_t*>(qp + 32 * kc);
     }
     const half_t* mrow =
         p.mask ? p.mask + (int64_t)head * p.mask_stride_h + (s0 + tok) * p.mask_stride_q + kv_first : nullptr;
@@ -227,9 +229,9 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
         for (int tb = 0; tb < TB; ++tb) {
             float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc) {
-                const half4_t a = *reinterpret_cast<const half4_t*>(&Ks[(16 * tb + r_lane) * LDK + 16 * kc + 4 * g]);
-                acc = __builtin_amdgcn_mfma_f32_16x16x16f16(a, qf[kc], acc, 0, 0, 0);
+            for (int kc = 0; kc < KC2; ++kc) {
+                const half8_t a = *reinterpret_cast<const half8_t*>(&Ks[(16 * tb + r_lane) * LDK + 32 * kc + 8 * g]);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kc], acc, 0, 0, 0);
             }
             if (mrow) {
 #pragma unroll
@@ -263,26 +265,39 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
             for (int i = 0; i < 4; ++i) pf[tb][i] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][i], cs, shift));
         }
         m_run = m_new;
-        const half4_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
         if (!__all(alpha == 1.0f)) { // (the maximum has moved for some row of the wave)
             l_acc *= alpha;
 #pragma unroll
             for (int db = 0; db < KC; ++db) o[db] *= alpha;
         }
+        // The second product takes 32 tokens a step: the lane's k-indices 8 * g + e are tokens 16 * tb + 4 * g + e
+        // (e < 4) and 16 * (tb + 1) + 4 * g + e - 4 of a pair of 16-token blocks, in the P^T operand (straight from
+        // the score registers) and in the V^T operand alike.
+        static_assert(TB % 2 == 0, "pairs of 16-token blocks");
+        const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f,
+                              (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+        half8_t pp[TB / 2];
 #pragma unroll
-        for (int tb = 0; tb < TB; ++tb) l_acc = __builtin_amdgcn_mfma_f32_16x16x16f16(ones, pf[tb], l_acc, 0, 0, 0);
+        for (int t2 = 0; t2 < TB / 2; ++t2) {
+            pp[t2] = half8_t{pf[2 * t2][0], pf[2 * t2][1], pf[2 * t2][2], pf[2 * t2][3],
+                             pf[2 * t2 + 1][0], pf[2 * t2 + 1][1], pf[2 * t2 + 1][2], pf[2 * t2 + 1][3]};
+            l_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pp[t2], l_acc, 0, 0, 0);
+        }
 #pragma unroll
         for (int db = 0; db < KC; ++db) {
 #pragma unroll
-            for (int tb = 0; tb < TB; ++tb) {
+            for (int t2 = 0; t2 < TB / 2; ++t2) {
                 // V^T operand: lane (block g, j) receives channel 16 * db + j of tokens 16 * tb + 4 * g .. + 3 when
                 // lane 4 * i + c of the block addresses token 16 * tb + 4 * g + i, channels 16 * db + 4 * c .. + 3
-                const half_t* src = &Vs[(16 * tb + 4 * g + (r_lane >> 2)) * LDK + 16 * db + 4 * (r_lane & 3)];
-                const short4_t raw =
+                const half_t* src = &Vs[(32 * t2 + 4 * g + (r_lane >> 2)) * LDK + 16 * db + 4 * (r_lane & 3)];
+                const short4_t lo =
                     __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)src);
-                half4_t a;
-                __builtin_memcpy(&a, &raw, 8);
-                o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pf[tb], o[db], 0, 0, 0);
+                const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) short4_t*)(src + 16 * LDK));
+                half8_t a;
+                __builtin_memcpy(&a, &lo, 8);
+                __builtin_memcpy(reinterpret_cast<char*>(&a) + 8, &hi, 8);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pp[t2], o[db], 0, 0, 0);
             }
         }
     };
