@@ -155,44 +155,54 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
         uint4 k, v; // fp16 source: 8 halves each; slab: .x/.y = 8 int8, .z = the group's scale (fp16 bits)
     };
     RawChunk raw[NCH];
-    // contiguous slab region: the sequence's first slab token, looked up once
-    const int64_t seq_tok0 = from_slab && p.pages.page_shift == 0 ? p.pages.cachestarts[b] : 0;
+    // Where the thread's chunks of the current tile start: halves into k16 / v16, or bytes into the slab (K row; the V
+    // row is stride_kv further). Tiles are fetched in order, so the offsets move on by one tile's worth per fetch; only
+    // a paged slab looks every token up.
+    const bool paged = from_slab && p.pages.page_shift != 0;
+    const int64_t seq_tok0 = from_slab && !paged ? p.pages.cachestarts[b] : 0;
+    const int64_t tile_stride = from_slab ? (int64_t)BN * p.addr.stride_s : (int64_t)BN * p.kv_heads * DH;
+    int64_t koff[NCH];
+#pragma unroll
+    for (int n = 0; n < NCH; ++n) {
+        const int c = tid + 256 * n;
+        const int r = c / CH, ch = c - r * CH;
+        koff[n] = from_slab ? p.addr.row(seq_tok0 + kv_begin + r, 0, kvh) + ch * 8
+                            : ((k16_row0 + kv_begin + r) * p.kv_heads + kvh) * DH + ch * 8;
+    }
     auto fetch = [&](int64_t kv0) {
+        const int64_t left64 = kvlen - kv0;
+        const int left = left64 > BN ? BN : (int)left64; // tokens of the tile that exist
 #pragma unroll
         for (int n = 0; n < NCH; ++n) {
             const int c = tid + 256 * n;
             const int r = c / CH, ch = c - r * CH;
-            const int64_t j = kv0 + r;
-            raw[n].k = raw[n].v = make_uint4(0, 0, 0, 0);
-            if (c < BN * CH && j < kvlen) {
+            if (c < BN * CH && r < left) {
                 if (from_slab) {
-                    const int64_t t_slab = p.pages.page_shift == 0 ? seq_tok0 + j : p.pages.token(b, j);
-                    const int64_t rk = p.addr.row(t_slab, 0, kvh), rv = p.addr.row(t_slab, 1, kvh);
-                    const uint2 qk = *reinterpret_cast<const uint2*>(p.cache + rk + ch * 8);
-                    const uint2 qv = *reinterpret_cast<const uint2*>(p.cache + rv + ch * 8);
-                    uint16_t sk, sv;
-                    __builtin_memcpy(&sk, &p.scale[rk / kQuantGroup + ch], 2);
-                    __builtin_memcpy(&sv, &p.scale[rv / kQuantGroup + ch], 2);
+                    int64_t rk = koff[n];
+                    if (paged) rk = p.addr.row(p.pages.token(b, kv0 + r), 0, kvh) + ch * 8;
+                    const int64_t rv = rk + p.addr.stride_kv;
+                    const uint2 qk = *reinterpret_cast<const uint2*>(p.cache + rk);
+                    const uint2 qv = *reinterpret_cast<const uint2*>(p.cache + rv);
+                    uint16_t sk, sv; // (rk = row + 8 * ch: the group's scale is element rk / 8)
+                    __builtin_memcpy(&sk, &p.scale[rk / kQuantGroup], 2);
+                    __builtin_memcpy(&sv, &p.scale[rv / kQuantGroup], 2);
                     raw[n].k = make_uint4(qk.x, qk.y, sk, 0);
                     raw[n].v = make_uint4(qv.x, qv.y, sv, 0);
                 } else {
-                    const int64_t off = ((k16_row0 + j) * p.kv_heads + kvh) * DH + ch * 8;
-                    raw[n].k = *reinterpret_cast<const uint4*>(p.k16 + off);
-                    raw[n].v = *reinterpret_cast<const uint4*>(p.v16 + off);
+                    raw[n].k = *reinterpret_cast<const uint4*>(p.k16 + koff[n]);
+                    raw[n].v = *reinterpret_cast<const uint4*>(p.v16 + koff[n]);
                 }
+            } else {
+                raw[n].k = raw[n].v = make_uint4(0, 0, 0, 0);
             }
+            koff[n] += tile_stride;
         }
     };
     auto dequant = [&](const uint4& x) { // slab chunk -> 8 halves, fp16(float(q) * float(scale)) as everywhere
         half_t sc;
         const uint16_t bits = (uint16_t)x.z;
         __builtin_memcpy(&sc, &bits, 2);
-        const float sf = (float)sc;
-        const uint32_t w[2] = {x.x, x.y};
-        half8_t o;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = (half_t)((float)(int)(int8_t)((w[i >> 2] >> (8 * (i & 3))) & 0xff) * sf);
-        return o;
+        return dequant8(x.x, x.y, sc);
     };
     auto stash = [&]() {
 #pragma unroll
