@@ -1,17 +1,21 @@
-// The attention kernel for everything the specialised kernels (decode.hip, prefill.hip: head_dim 128, at most 16 query
+// The attention kernels for everything the specialised kernels (decode.hip, prefill.hip: head_dim 128, at most 16 query
 // heads per kv head, no mask) do not take: any head_dim that is a multiple of 32 up to 256, any number of query heads
-// per kv head, and an additive attn_mask. One kernel serves decode sequences, prompts and MultiHeadAttention.
+// per kv head, and an additive attn_mask; for MultiHeadCacheAttention and MultiHeadAttention.
 //
-// Rows of a workgroup are (query token, query head of the kv head) pairs of ONE (sequence, kv head): row r of the
-// sequence is token r / rep, head kvh * rep + r % rep, so the K/V tile a workgroup stages in LDS is shared by all query
-// heads of its kv head, and a decode sequence (one token) fills rep rows of a tile instead of one. 64 rows per
-// workgroup, 16 per wave. Per K/V tile: S^T = K Q^T and O^T += V^T P^T with v_mfma_f32_16x16x16_f16, a query row
-// living in the 16 lanes' same column throughout (row statistics are per lane, reductions only over the four 16-lane
-// groups); P never leaves registers (the result layout of the first product is the B operand layout of the second);
-// V^T operands come from row-major V through ds_read_b64_tr_b16. K/V come from the int8 slab (dequantised on the way
-// into LDS, value = fp16(float(q) * float(scale)) as everywhere) or from packed fp16 rows.
-// The next K/V tile is requested from memory before the current one is computed. No split of long sequences: this
-// path is for coverage, the tuned kernels for speed.
+// generic_attention_kernel (the tile kernel: prompts, MultiHeadAttention, decode tokens with more than 16 query heads
+// per kv head). Rows of a workgroup are (query token, query head of the kv head) pairs of ONE (sequence, kv head): row
+// r of the sequence is token r / rep, head kvh * rep + r % rep, so the K/V tile a workgroup stages in LDS is shared by
+// all query heads of its kv head, and a decode sequence (one token) fills rep rows of a tile instead of one. 64 rows
+// per workgroup, 16 per wave. Per K/V tile: S^T = K Q^T and O^T += V^T P^T with v_mfma_f32_16x16x32_f16, a query row
+// living in the 16 lanes' same column throughout (row maxima are per lane, reduced only over the four 16-lane groups;
+// row sums come out of the matrix cores); P never leaves registers (the result layout of the first product is the B
+// operand layout of the second); V^T operands come from row-major V through ds_read_b64_tr_b16. K/V come from the
+// int8 slab (dequantised on the way into LDS, value = fp16(float(q) * float(scale)) as everywhere) or from packed fp16
+// rows. The next K/V tile is requested from memory before the current one is computed.
+//
+// generic_decode_kernel (decode sequences with at most 16 query heads per kv head): a wave per (sequence, one or two
+// kv heads, piece of the keys), K straight from the slab into the matrix-core operands; generic_merge_kernel combines
+// the pieces of a sequence. Described where they are defined.
 #include "common.h"
 
 #include <type_traits>
