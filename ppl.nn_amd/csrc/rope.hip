@@ -3,7 +3,8 @@
 //
 // Both are streaming kernels (HBM roofline): RotaryPositionEmbedding reads and writes every query and key element
 // once, 16 bytes per lane; the angle of a (position, channel pair) is formed in float64 (position * theta^(-2i/d),
-// reduced mod 2*pi before it is narrowed), because a float32 product loses the low bits of a 100k-token position.
+// reduced mod 2*pi before it is narrowed), because a float32 product loses the low bits of a 100k-token position;
+// once per token (workgroup), shared through LDS.
 // Pair i rotates by position * theta^(-2i / rotary_dim); its two channels are (2i, 2i + 1) or (i, i + rotary_dim / 2),
 // the caller's pair_layout; channels >= rotary_dim pass through.
 //
@@ -41,15 +42,19 @@ struct RopeParams {
 };
 
 constexpr double kTwoPi = 6.283185307179586476925286766559;
+constexpr int kMaxRotaryPairs = 1024; // rotary_dim <= head_dim <= 2048 (checked at the entry point)
 
 template <bool WRITE_KV>
 __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
+    // cosine and sine of the token's rotary_dim / 2 angles: each is formed once per workgroup (a float64 exp2, a
+    // reduction mod 2 pi, cosf and sinf: several hundred instructions, which every lane used to repeat for its own pairs
+    // and which then took longer than the kernel's memory traffic) and handed to the lanes through LDS
+    __shared__ float cos_tab[kMaxRotaryPairs], sin_tab[kMaxRotaryPairs];
     const int64_t t = blockIdx.x; // packed token
     const int cpr = p.head_dim / 8; // 16-byte chunks per head row
     const int rows_per_pass = 256 / cpr;
     const int slot = threadIdx.x / cpr;
     const int chunk = threadIdx.x - slot * cpr;
-    if (slot >= rows_per_pass) return;
 
     // (every lane of the workgroup looks for the same token: one table read per lane and a count, one memory round
     // trip instead of a binary search's chain of them)
@@ -75,16 +80,22 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     const bool upper = p.half_split && 8 * chunk >= half;
     const int npairs = p.half_split ? 8 : 4;
     const int pair0 = p.half_split ? 8 * chunk - (upper ? half : 0) : 4 * chunk;
+    for (int i = threadIdx.x; i < half; i += 256) {
+        const double inv_freq = exp2(-(2.0 * i / (double)p.rotary_dim) * log2_theta);
+        double a = pos * inv_freq;
+        a -= kTwoPi * rint(a / kTwoPi);
+        cos_tab[i] = cosf((float)a);
+        sin_tab[i] = sinf((float)a);
+    }
+    __syncthreads();
+    if (slot >= rows_per_pass) return;
     float cs[8], sn[8];
     if (rotate) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             if (j < npairs) {
-                const double inv_freq = exp2(-(2.0 * (pair0 + j) / (double)p.rotary_dim) * log2_theta);
-                double a = pos * inv_freq;
-                a -= kTwoPi * rint(a / kTwoPi);
-                cs[j] = cosf((float)a);
-                sn[j] = sinf((float)a);
+                cs[j] = cos_tab[pair0 + j];
+                sn[j] = sin_tab[pair0 + j];
             }
         }
     }
