@@ -169,15 +169,9 @@ __global__ __launch_bounds__(256) void kv_stage_prefill_kernel(const StageParams
         half_t sc;
         const uint16_t sbits = (uint16_t)(sw[g >> 1] >> (16 * (g & 1)));
         __builtin_memcpy(&sc, &sbits, 2);
-        const float sf = (float)sc;
-        half_t o[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int qi = (int)(int8_t)((qw[2 * g + (i >> 2)] >> (8 * (i & 3))) & 0xff);
-            o[i] = (half_t)((float)qi * sf); // the fp32 product is exact; one rounding to fp16
-        }
+        const half8_t o = dequant8(qw[2 * g], qw[2 * g + 1], sc); // = fp16(float(q) * float(scale)), one rounding
         uint4 packed;
-        __builtin_memcpy(&packed, o, 16);
+        __builtin_memcpy(&packed, &o, 16);
         dst[g] = packed;
     }
 }
@@ -233,18 +227,21 @@ struct GatherParams {
     int64_t total_groups; // total_kv_tokens * 2 * kv_heads * groups_per_head
 };
 
+// A thread takes four groups (32 channels) of one (token, K or V, head): 32 bytes of int8 and four scales in, 64 bytes
+// of fp16 out; the index arithmetic (three divisions) is spent once per 32 channels.
 __global__ __launch_bounds__(256) void kv_gather_dequant_kernel(const GatherParams p) {
-    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (g >= p.total_groups) return;
-    const int gph = p.groups_per_head;
-    const int per_kv = p.kv_heads * gph;
+    const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // unit of four groups
+    if (u >= p.total_groups / 4) return;
+    const int uph = p.groups_per_head / 4; // units per head (head_dim is a multiple of 32)
+    const int per_kv = p.kv_heads * uph;
     const int per_tok = 2 * per_kv;
-    const int64_t j = g / per_tok; // packed kv-token index
-    const int r = (int)(g - j * per_tok);
+    // packed kv-token index (a 32-bit division where the numbers allow it)
+    const int64_t j = (uint64_t)u >> 32 ? u / per_tok : (int64_t)((uint32_t)u / (uint32_t)per_tok);
+    const int r = (int)(u - j * per_tok);
     const int kv = r / per_kv;
     const int r2 = r - kv * per_kv;
-    const int head = r2 / gph;
-    const int grp = r2 - head * gph;
+    const int head = r2 / uph;
+    const int grp = (r2 - head * uph) * 4; // first of the unit's four groups
     int b;
     {
         const int64_t j0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(j >> 32)) << 32) |
@@ -256,19 +253,23 @@ __global__ __launch_bounds__(256) void kv_gather_dequant_kernel(const GatherPara
     }
     const int64_t tok = p.cachestarts[b] + (j - p.kvstarts[b]);
     const int64_t row = p.addr.row(tok, kv, head);
-    const uint2 q = *reinterpret_cast<const uint2*>(p.cache + row + grp * 8);
-    const float s = (float)p.scale[row / kQuantGroup + grp];
-    half_t o[8];
-    const uint32_t w[2] = {q.x, q.y};
+    const uint4* src = reinterpret_cast<const uint4*>(p.cache + row + grp * 8); // rows and grp * 8: multiples of 16
+    const uint4 q0 = src[0], q1 = src[1];
+    const uint32_t* ssrc = reinterpret_cast<const uint32_t*>(p.scale + row / kQuantGroup + grp);
+    const uint32_t sw[2] = {ssrc[0], ssrc[1]};
+    const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    uint4* dst = reinterpret_cast<uint4*>((kv ? p.value_out : p.key_out) +
+                                          ((j * p.kv_heads + head) * p.groups_per_head + grp) * 8);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int qi = (int)(int8_t)((w[i >> 2] >> (8 * (i & 3))) & 0xff);
-        o[i] = (half_t)((float)qi * s); // the fp32 product is exact; one rounding to fp16
+    for (int g = 0; g < 4; ++g) {
+        half_t sc;
+        const uint16_t sbits = (uint16_t)(sw[g >> 1] >> (16 * (g & 1)));
+        __builtin_memcpy(&sc, &sbits, 2);
+        const half8_t o = dequant8(qw[2 * g], qw[2 * g + 1], sc); // = fp16(float(q) * float(scale)), one rounding
+        uint4 packed;
+        __builtin_memcpy(&packed, &o, 16);
+        dst[g] = packed;
     }
-    uint4 packed;
-    __builtin_memcpy(&packed, o, 16);
-    half_t* dst = (kv ? p.value_out : p.key_out) + ((j * p.kv_heads + head) * gph + grp) * 8;
-    *reinterpret_cast<uint4*>(dst) = packed;
 }
 
 pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream_t stream) {
@@ -286,7 +287,7 @@ pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream
     p.kv_heads = w->num_kv_heads;
     p.groups_per_head = w->head_dim / kQuantGroup;
     p.total_groups = a->total_kv_tokens * 2 * (int64_t)w->num_kv_heads * p.groups_per_head;
-    const int64_t blocks = (p.total_groups + 255) / 256;
+    const int64_t blocks = (p.total_groups / 4 + 255) / 256;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "kv_gather_dequant: too many groups");
     hipLaunchKernelGGL(kv_gather_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("kv_gather_dequant");
