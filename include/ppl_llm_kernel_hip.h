@@ -401,6 +401,15 @@ pplhip_retcode pplhip_probe_mfma_f16(const void* d_operands, void* d_out, int32_
 pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_out, int32_t workgroups,
                                      uint64_t* bytes_read, void* stream);
 
+/*
+ * Verification aid (no counterpart in the reference): the quantiser forms x / s as x * (1 / s), one division per
+ * group instead of eight. This call enumerates every absmax (all positive fp16 up to +inf, i.e. every scale the rule
+ * max(fp16(absmax / 127), fp16(1e-5)) can produce) with every fp16 x of no larger magnitude or NaN, runs each pair through
+ * the library's own quantiser and ADDS to `*d_mismatches` (device, 8 bytes, cleared by the caller) the number of pairs
+ * whose int8 differs from int8(rint(fp16(x / s))) formed by a correctly rounded division. 0 is the contract.
+ */
+pplhip_retcode pplhip_probe_quantizer(uint64_t* d_mismatches, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -133,6 +133,7 @@ PROTOTYPES = {
     "pplhip_advance_slots": (_i32, [_p, _p, _i32, _p]),
     "pplhip_probe_mfma_f16": (_i32, [_p, _p, _i32, _i32, C.POINTER(C.c_double), _p]),
     "pplhip_probe_hbm_read": (_i32, [_p, C.c_uint64, _p, _i32, C.POINTER(C.c_uint64), _p]),
+    "pplhip_probe_quantizer": (_i32, [_p, _p]),
 }
 
 

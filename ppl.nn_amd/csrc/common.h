@@ -75,10 +75,15 @@ __device__ inline void quantize_group8(const uint4 raw, uint2* q_out, half_t* s_
     const half_t eps = (half_t)1e-5f;
     if ((float)s < (float)eps) s = eps;
     const float sf = (float)s;
+    // x / s as x * (1 / s): one correctly rounded division per group instead of eight. The fp32 products differ from
+    // the fp32 quotients in the last bits, the int8 results do not: for every fp16 x (all 65 536 patterns) and every
+    // scale the rule can produce (all fp16 from eps to +inf) both ways give the same q, checked by enumerating the
+    // pairs on the device with this file's compiler flags (no contraction, IEEE division).
+    const float rs = 1.0f / sf;
     uint32_t w[2] = {0u, 0u};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const float ratio = (float)(half_t)((float)x[i] / sf);
+        const float ratio = (float)(half_t)((float)x[i] * rs);
         float r = rintf(ratio);
         r = fminf(fmaxf(r, -128.f), 127.f);
         const int qi = (int)r;

@@ -90,3 +90,36 @@ extern "C" pplhip_retcode pplhip_probe_mfma_f16(const void* d_operands, void* d_
     if (flops) *flops = (double)workgroups * 4.0 * iterations * kProbeMfmaPerIter * (2.0 * 32 * 32 * 16);
     return PPLHIP_RC_SUCCESS;
 }
+
+// ---- the quantiser's quotients, enumerated
+// quantize_group8 forms x / s as x * (1 / s). For every absmax A (all positive fp16 up to +inf: every scale the rule
+// can produce) and every fp16 x of no larger magnitude (and every NaN, which the maximum ignores), the group
+// {A, x, 0, ...} goes through quantize_group8 and the int8 it gives x is compared with int8(rint(fp16(x / s))) formed
+// by a correctly rounded fp32 division.
+__global__ __launch_bounds__(256) void probe_quantizer_kernel(unsigned long long* mismatches) {
+    const uint32_t a_bits = blockIdx.x + 1; // 0x0001 .. 0x7c00
+    unsigned long long bad = 0;
+    for (uint32_t xb = threadIdx.x; xb < 65536; xb += 256) {
+        const uint32_t mag = xb & 0x7fffu;
+        if (mag > a_bits && mag <= 0x7c00u) continue; // larger magnitude than the absmax
+        uint2 q;
+        half_t s;
+        quantize_group8(make_uint4(a_bits | xb << 16, 0, 0, 0), &q, &s);
+        const uint16_t x16 = (uint16_t)xb;
+        half_t x;
+        __builtin_memcpy(&x, &x16, 2);
+        float r = rintf((float)(half_t)((float)x / (float)s));
+        r = fminf(fmaxf(r, -128.f), 127.f);
+        if ((uint32_t)((int)r & 0xff) != ((q.x >> 8) & 0xffu)) ++bad;
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
+extern "C" pplhip_retcode pplhip_probe_quantizer(uint64_t* d_mismatches, void* stream) {
+    if (!d_mismatches) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "probe: null counter");
+    hipLaunchKernelGGL(probe_quantizer_kernel, dim3(0x7c00), dim3(256), 0, (hipStream_t)stream,
+                       (unsigned long long*)d_mismatches);
+    PPLHIP_CHECK_LAUNCH("probe_quantizer");
+    return PPLHIP_RC_SUCCESS;
+}
+

@@ -50,6 +50,51 @@ def test_quantize_write_all_finite_absmax_bit_exact(hiplib, olib):
     assert np.array_equal(scale_d.cpu().view(torch.int16).numpy().view(np.uint16), scale_o.view(np.uint16))
 
 
+def test_quantizer_quotients_enumerated(hiplib):
+    """x * (1 / s) against x / s over every (absmax, x) pair of fp16 values, inside the library: no int8 differs."""
+    import torch
+    bad = torch.zeros(1, dtype=torch.int64, device="cuda")
+    harness.pkg.check(hiplib.pplhip_probe_quantizer(harness.dev_ptr(bad), None), "probe_quantizer")
+    torch.cuda.synchronize()
+    assert int(bad.item()) == 0
+
+
+def test_quantize_write_every_value_against_a_spread_of_scales(hiplib, olib):
+    """The device forms x / s as x * (1 / s), one division per group instead of eight; that the int8 results are those
+    of the division for EVERY fp16 x and EVERY scale was established by enumerating all pairs on the device. Here: 200
+    absmax values spread over the finite range (and the extremes), each with every fp16 value of no larger magnitude
+    as its companions, through the write kernel against the oracle's divisions."""
+    import torch
+    pos = np.arange(0, 0x7c00, dtype=np.uint16)
+    picks = np.unique(np.concatenate([pos[:: len(pos) // 190], [1, 2, 0x03ff, 0x0400, 0x7bff, 0x7bfe, 0x3c00]]))
+    picks = picks[picks > 0].astype(np.uint16)
+    groups = []
+    for a in picks:
+        mag = np.arange(0, int(a) + 1, dtype=np.uint16)  # bit patterns 0 .. a are the magnitudes <= absmax
+        xs = np.concatenate([mag, mag | np.uint16(0x8000)])
+        pad = (-len(xs)) % 7
+        xs = np.concatenate([xs, np.zeros(pad, np.uint16)]).reshape(-1, 7)
+        groups.append(np.concatenate([np.full((len(xs), 1), a, np.uint16), xs], axis=1))
+    groups = np.concatenate(groups).view(np.float16)  # [n, 8], first element = the group's absmax
+    n_tok = groups.shape[0] // 16
+    key = np.ascontiguousarray(groups[:n_tok * 16].reshape(n_tok, 1, 128))
+    val = np.ascontiguousarray(-key[::-1])
+    print(f"case every value x {len(picks)} scales: {n_tok} tokens", flush=True)
+    b = workloads.Batch(1, 1, 128, [n_tok], [0], 0)
+    cache_o, scale_o = harness.new_slab(b)
+    zeros = np.zeros(1, np.int64)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, key, val, b.seqstarts, zeros, b.cachestarts, cache_o, scale_o)
+    assert olib.oracle_kv_quantize_write(C.byref(w)) == 0
+    cache_d, scale_d = harness.to_dev(harness.new_slab(b)[0]), harness.to_dev(harness.new_slab(b)[1])
+    kd, vd = harness.to_dev(key), harness.to_dev(val)
+    ss, cs, sp = harness.to_dev(b.seqstarts), harness.to_dev(b.cachestarts), harness.to_dev(zeros)
+    w = harness.fill_write_args(cabi.KvWriteArgs(), b, kd, vd, ss, sp, cs, cache_d, scale_d, ptr=harness.dev_ptr)
+    harness.pkg.check(hiplib.pplhip_kv_quantize_write(C.byref(w), None), "kv_quantize_write")
+    torch.cuda.synchronize()
+    assert np.array_equal(cache_d.cpu().numpy(), cache_o)
+    assert np.array_equal(scale_d.cpu().view(torch.int16).numpy().view(np.uint16), scale_o.view(np.uint16))
+
+
 @pytest.mark.parametrize("H,KVH", [(4, 4), (8, 2), (8, 1), (32, 8), (16, 1), (40, 40)])
 def test_small_mixed_batches(H, KVH):
     b = workloads.Batch(H, KVH, 128, [1, 1, 1, 1, 9, 130, 64, 1], [40, 0 + 1, 300, 63, 0, 0, 0, 0], 4,
