@@ -58,6 +58,17 @@ def test_noalloc_matches_forward_on_two_calls_in_a_row(hiplib):
     _run_both(hiplib, small, seed=72)
 
 
+def test_noalloc_matches_forward_on_the_general_path(hiplib):
+    """head_dim 64: the decode sequences' pieces (general attention path) lie in the scratch array; again two calls
+    in a row, the second smaller."""
+    assert hiplib.pplhip_init() == 0
+    big = workloads.Batch(16, 4, 64, [1] * 12 + [90], list(range(2000, 2000 + 12 * 53, 53)) + [0], 12,
+                          name="general, first (larger)")
+    small = workloads.Batch(16, 4, 64, [1] * 3 + [20], [700, 130, 1500, 0], 3, name="general, second (smaller)")
+    _run_both(hiplib, big, seed=73)
+    _run_both(hiplib, small, seed=74)
+
+
 def test_noalloc_rejects_what_needs_a_caller_workspace(hiplib):
     b = workloads.Batch(32, 8, 128, [1, 1, 512, 512], [100, 900, 4096, 0], 2)
     a = cabi.MhcaArgs()
