@@ -647,19 +647,31 @@ __global__ __launch_bounds__(256) void generic_merge_kernel(const GenericParams 
     const int64_t kvlen = p.kvstarts[b + 1] - p.kvstarts[b];
     int n = (int)((kvlen + p.piece_tokens - 1) / p.piece_tokens); // the pieces that exist
     if (n > p.nsplit) n = p.nsplit;
-    float M = -INFINITY;
-    for (int s = 0; s < n; ++s) M = fmaxf(M, p.part_ml[(row * p.nsplit + s) * 2]);
+    // four pieces' loads go out together; the pieces are folded into a running (maximum, sum, accumulator)
+    float M = -INFINITY, L = 0.f;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    float L = 0.f;
-    if (M != -INFINITY) { // (all pieces without unmasked keys: the row has no distribution -> zeros)
-        for (int s = 0; s < n; ++s) {
-            const int64_t pr = row * p.nsplit + s;
-            const float w = __builtin_amdgcn_exp2f(p.part_ml[pr * 2] - M);
-            acc += *reinterpret_cast<const float4_t*>(p.part_o + pr * DH + d4) * w;
-            L += p.part_ml[pr * 2 + 1] * w;
+    for (int s0 = 0; s0 < n; s0 += 4) {
+        float2 ml[4];
+        float4_t o4[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t pr = row * p.nsplit + (s0 + k < n ? s0 + k : n - 1);
+            ml[k] = *reinterpret_cast<const float2*>(p.part_ml + pr * 2);
+            o4[k] = *reinterpret_cast<const float4_t*>(p.part_o + pr * DH + d4);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float m_new = fmaxf(M, ml[k].x);
+            // (a piece without unmasked keys has maximum -inf and weight 0; while nothing else was seen, nothing moves)
+            if (s0 + k < n && m_new != -INFINITY) {
+                const float wa = __builtin_amdgcn_exp2f(M - m_new), wb = __builtin_amdgcn_exp2f(ml[k].x - m_new);
+                acc = acc * wa + o4[k] * wb;
+                L = L * wa + ml[k].y * wb;
+                M = m_new;
+            }
         }
     }
-    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    const float inv = L > 0.f ? 1.0f / L : 0.f; // (no piece with unmasked keys: zeros)
     const half4_t r = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv), (half_t)(acc[2] * inv), (half_t)(acc[3] * inv)};
     *reinterpret_cast<half4_t*>(p.out + row * DH + d4) = r;
 }
