@@ -236,6 +236,21 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
         const int64_t rel = row_limit - kv0;
         const int lim4 = (int)(rel < -1 ? -1 : rel > BN ? BN : rel) - 4 * g;
         const bool all_visible = __all(lim4 + 4 * g >= BN - 1);
+        // the tile's mask entries of the lane's row, requested before the score products and without a branch per
+        // element: an index past the row's last key is pulled back onto it (that entry exists; its score is masked
+        // out by the comparison below)
+        float mk[TB][4];
+        if (mrow) {
+            const int64_t last = kvlen - 1;
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int64_t j = kv0 + 16 * tb + 4 * g + i;
+                    mk[tb][i] = (float)mrow[j < last ? j : last] * kLog2e;
+                }
+            }
+        }
         // ---- scores of the lane's row against tokens kv0 + 16 * tb + 4 * g + i
         float s[TB][4];
         float mx = -INFINITY;
@@ -249,11 +264,8 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
             }
             if (mrow) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int64_t j = kv0 + 16 * tb + 4 * g + i;
-                    // (a masked-out key's mask entry is not read: it may lie past the row's end)
-                    acc[i] = 16 * tb + i <= lim4 ? __builtin_fmaf(acc[i], p.scale_log2, (float)mrow[j] * kLog2e) : -INFINITY;
-                }
+                for (int i = 0; i < 4; ++i)
+                    acc[i] = 16 * tb + i <= lim4 ? __builtin_fmaf(acc[i], p.scale_log2, mk[tb][i]) : -INFINITY;
             } else if (!all_visible) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) acc[i] = 16 * tb + i <= lim4 ? acc[i] : -INFINITY;
