@@ -58,10 +58,19 @@ struct GenericParams {
 };
 
 constexpr int kGenRows = 64;
+// head dims at which a wave takes two blocks of 16 rows (tiles of 128 rows): measured on four 2 048-token prompts,
+// one block against two: head_dim 32 135 / 142 us, 64 176 / 194 us, 96 301 / 268 us, 128 (with a mask) 405 / 398 us;
+// above 128 two blocks' accumulators do not fit the registers
+constexpr bool gen_two_row_blocks(int head_dim) { return head_dim >= 96 && head_dim <= 128; }
 constexpr float kLog2e = 1.4426950408889634f;
 
-template <int DH>
-__global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2) void generic_attention_kernel(const GenericParams p) {
+// RB: blocks of 16 rows per wave (the workgroup's tile has 64 * RB rows). The staging of a K/V tile, its barriers and
+// a tile's bookkeeping cost every wave the same whatever its rows, and every K and V operand read from LDS feeds RB
+// matrix-core instructions; two blocks' state costs a wave per SIMD (see gen_two_row_blocks).
+template <int DH, int RB>
+__global__ __launch_bounds__(256, (RB == 2 ? 2 : DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2))
+void generic_attention_kernel(const GenericParams p) {
+    constexpr int GR = kGenRows * RB; // rows of the workgroup's tile
     constexpr int BN = DH <= 128 ? 64 : 32; // kv tokens per tile
     constexpr int LDK = DH + 8; // halves per LDS row (padding spreads the rows over the banks)
     constexpr int KC = DH / 16;
@@ -100,7 +109,7 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
     const int64_t kv_first = p.kvstarts[b];
     const int64_t kvlen = p.kvstarts[b + 1] - kv_first;
     const int64_t rows = L * p.rep;
-    const int64_t row0 = (int64_t)tile * kGenRows;
+    const int64_t row0 = (int64_t)tile * GR;
     if (row0 >= rows || kvlen <= 0) return;
     const int64_t sp = kvlen > L ? kvlen - L : 0;
     const bool from_slab = b < p.first_fp16_seq;
@@ -109,15 +118,22 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r_lane = lane & 15, g = lane >> 4;
-    const int64_t my_row_raw = row0 + wave * 16 + r_lane;
-    const bool valid = my_row_raw < rows;
-    const int64_t my_row = valid ? my_row_raw : rows - 1;
-    const int64_t tok = my_row / p.rep;
-    const int head = kvh * p.rep + (int)(my_row - tok * p.rep);
-    // keys 0 .. row_limit are visible to this lane's row
+    // the lane's rows: one in each of the wave's RB blocks of 16
+    bool valid[RB];
+    int64_t tok[RB], row_limit[RB];
+    int head[RB];
     const int64_t all = kvlen - 1;
-    const int64_t row_limit = !valid ? -1 : (p.is_causal ? (sp + tok < all ? sp + tok : all) : all);
-    const int64_t last_row = (row0 + kGenRows - 1 < rows - 1) ? row0 + kGenRows - 1 : rows - 1;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        const int64_t my_row_raw = row0 + (wave * RB + rb) * 16 + r_lane;
+        valid[rb] = my_row_raw < rows;
+        const int64_t my_row = valid[rb] ? my_row_raw : rows - 1;
+        tok[rb] = my_row / p.rep;
+        head[rb] = kvh * p.rep + (int)(my_row - tok[rb] * p.rep);
+        // keys 0 .. row_limit are visible to this lane's row
+        row_limit[rb] = !valid[rb] ? -1 : (p.is_causal ? (sp + tok[rb] < all ? sp + tok[rb] : all) : all);
+    }
+    const int64_t last_row = (row0 + GR - 1 < rows - 1) ? row0 + GR - 1 : rows - 1;
     int64_t kv_end = p.is_causal ? ((sp + last_row / p.rep + 1 < kvlen) ? sp + last_row / p.rep + 1 : kvlen) : kvlen;
     int64_t kv_begin = 0;
     if (pieces) { // (a decode sequence: one token, which sees every key)
@@ -129,25 +145,33 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
     // Q^T as the B operand of the score product (v_mfma_f32_16x16x32_f16: 32 channels a step, 8 of them per lane):
     // channels 32 * kc + 8 * g .. + 7 of the lane's row
     constexpr int KC2 = DH / 32;
-    half8_t qf[KC2];
-    {
-        const half_t* qp = p.q + ((s0 + tok) * p.num_heads + head) * DH + 8 * g;
+    half8_t qf[RB][KC2];
+    const half_t* mrow[RB];
+    const bool masked = p.mask != nullptr;
 #pragma unroll
-        for (int kc = 0; kc < KC2; ++kc) qf[kc] = *reinterpret_cast<const half8_t*>(qp + 32 * kc);
+    for (int rb = 0; rb < RB; ++rb) {
+        const half_t* qp = p.q + ((s0 + tok[rb]) * p.num_heads + head[rb]) * DH + 8 * g;
+#pragma unroll
+        for (int kc = 0; kc < KC2; ++kc) qf[rb][kc] = *reinterpret_cast<const half8_t*>(qp + 32 * kc);
+        mrow[rb] = masked ? p.mask + (int64_t)head[rb] * p.mask_stride_h + (s0 + tok[rb]) * p.mask_stride_q + kv_first
+                          : nullptr;
     }
-    const half_t* mrow =
-        p.mask ? p.mask + (int64_t)head * p.mask_stride_h + (s0 + tok) * p.mask_stride_q + kv_first : nullptr;
 
     // The running maximum is kept in the domain the scores are held in: raw products (times `cs` = scale_log2 inside
     // the exponentials) without a mask, exp2-domain values (cs = 1) with one. The row's sum of probabilities comes out
     // of the matrix cores (a row of ones as the A operand against P^T: every component of l_acc holds it), which also
     // adds up the four lane groups' shares.
-    const float cs = mrow ? 1.0f : p.scale_log2;
-    float m_run = -INFINITY;
-    float4_t l_acc = {0.f, 0.f, 0.f, 0.f};
-    float4_t o[KC];
+    const float cs = masked ? 1.0f : p.scale_log2;
+    float m_run[RB];
+    float4_t l_acc[RB];
+    float4_t o[RB][KC];
 #pragma unroll
-    for (int i = 0; i < KC; ++i) o[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < RB; ++rb) {
+        m_run[rb] = -INFINITY;
+        l_acc[rb] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < KC; ++i) o[rb][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     // A thread's share of a K/V tile: NCH 16-byte chunks (one quantisation group each) of K and of V, as they come from
     // memory. The next tile's are requested before the current tile is computed and go to LDS (dequantised) when it is
@@ -228,73 +252,72 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
     };
     // a wave none of whose 16 rows exists (a decode sequence fills rep rows of the tile's 64) only helps to stage the
     // tiles: its arithmetic would be thrown away, and it would take the matrix cores from the waves that have rows
-    const bool wave_has_rows = row0 + wave * 16 < rows;
-    // one K/V tile for the lane's row
+    const bool wave_has_rows = row0 + wave * 16 * RB < rows;
+    // one K/V tile for the lane's rows
     auto tile_step = [&](const int64_t kv0) {
         // keys kv0 .. kv0 + lim of the tile are visible to the lane's row; a tile all of whose keys are visible to all of
         // the wave's rows (every tile but a causal sequence's last ones, and a ragged tile's) skips the comparisons
-        const int64_t rel = row_limit - kv0;
-        const int lim4 = (int)(rel < -1 ? -1 : rel > BN ? BN : rel) - 4 * g;
-        const bool all_visible = __all(lim4 + 4 * g >= BN - 1);
-        // the tile's mask entries of the lane's row, requested before the score products and without a branch per
+        int lim4[RB];
+        bool vis = true;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int64_t rel = row_limit[rb] - kv0;
+            lim4[rb] = (int)(rel < -1 ? -1 : rel > BN ? BN : rel) - 4 * g;
+            vis = vis && lim4[rb] + 4 * g >= BN - 1;
+        }
+        const bool all_visible = __all(vis);
+        // the tile's mask entries of the lane's rows, requested before the score products and without a branch per
         // element: an index past the row's last key is pulled back onto it (that entry exists; its score is masked
         // out by the comparison below)
-        float mk[TB][4];
-        if (mrow) {
+        float mk[RB][TB][4];
+        if (masked) {
             const int64_t last = kvlen - 1;
 #pragma unroll
-            for (int tb = 0; tb < TB; ++tb) {
+            for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int64_t j = kv0 + 16 * tb + 4 * g + i;
-                    mk[tb][i] = (float)mrow[j < last ? j : last] * kLog2e;
+                for (int tb = 0; tb < TB; ++tb) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int64_t j = kv0 + 16 * tb + 4 * g + i;
+                        mk[rb][tb][i] = (float)mrow[rb][j < last ? j : last] * kLog2e;
+                    }
                 }
             }
         }
-        // ---- scores of the lane's row against tokens kv0 + 16 * tb + 4 * g + i
-        float s[TB][4];
-        float mx = -INFINITY;
+        // ---- scores of the lane's rows against tokens kv0 + 16 * tb + 4 * g + i
+        float s[RB][TB][4];
+        float mx[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) mx[rb] = -INFINITY;
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb) {
-            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+            float4_t acc[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) acc[rb] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kc = 0; kc < KC2; ++kc) {
                 const half8_t a = *reinterpret_cast<const half8_t*>(&Ks[(16 * tb + r_lane) * LDK + 32 * kc + 8 * g]);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[kc], acc, 0, 0, 0);
-            }
-            if (mrow) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    acc[i] = 16 * tb + i <= lim4 ? __builtin_fmaf(acc[i], p.scale_log2, mk[tb][i]) : -INFINITY;
-            } else if (!all_visible) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] = 16 * tb + i <= lim4 ? acc[i] : -INFINITY;
+                for (int rb = 0; rb < RB; ++rb)
+                    acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[rb][kc], acc[rb], 0, 0, 0);
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                s[tb][i] = acc[i];
-                mx = fmaxf(mx, acc[i]);
+            for (int rb = 0; rb < RB; ++rb) {
+                if (masked) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[rb][i] = 16 * tb + i <= lim4[rb] ? __builtin_fmaf(acc[rb][i], p.scale_log2, mk[rb][tb][i])
+                                                             : -INFINITY;
+                } else if (!all_visible) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[rb][i] = 16 * tb + i <= lim4[rb] ? acc[rb][i] : -INFINITY;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s[rb][tb][i] = acc[rb][i];
+                    mx[rb] = fmaxf(mx[rb], acc[rb][i]);
+                }
             }
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // a row that has seen nothing but masked keys so far keeps max -inf: against 0 in the exponents its
-        // probabilities are exp2(-inf) = 0, not NaN
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs);
-        const float shift = -m_safe * cs;
-        half4_t pf[TB];
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pf[tb][i] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][i], cs, shift));
-        }
-        m_run = m_new;
-        if (!__all(alpha == 1.0f)) { // (the maximum has moved for some row of the wave)
-            l_acc *= alpha;
-#pragma unroll
-            for (int db = 0; db < KC; ++db) o[db] *= alpha;
         }
         // The second product takes 32 tokens a step: the lane's k-indices 8 * g + e are tokens 16 * tb + 4 * g + e
         // (e < 4) and 16 * (tb + 1) + 4 * g + e - 4 of a pair of 16-token blocks, in the P^T operand (straight from
@@ -302,13 +325,47 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
         static_assert(TB % 2 == 0, "pairs of 16-token blocks");
         const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f,
                               (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
-        half8_t pp[TB / 2];
+        half8_t pp[RB][TB / 2];
+        bool still = true;
+        float alpha[RB];
 #pragma unroll
-        for (int t2 = 0; t2 < TB / 2; ++t2) {
-            pp[t2] = half8_t{pf[2 * t2][0], pf[2 * t2][1], pf[2 * t2][2], pf[2 * t2][3],
-                             pf[2 * t2 + 1][0], pf[2 * t2 + 1][1], pf[2 * t2 + 1][2], pf[2 * t2 + 1][3]};
-            l_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pp[t2], l_acc, 0, 0, 0);
+        for (int rb = 0; rb < RB; ++rb) {
+            float m = mx[rb];
+            m = fmaxf(m, __shfl_xor(m, 16));
+            m = fmaxf(m, __shfl_xor(m, 32));
+            const float m_new = fmaxf(m_run[rb], m);
+            // a row that has seen nothing but masked keys so far keeps max -inf: against 0 in the exponents its
+            // probabilities are exp2(-inf) = 0, not NaN
+            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+            alpha[rb] = __builtin_amdgcn_exp2f((m_run[rb] - m_safe) * cs);
+            const float shift = -m_safe * cs;
+            half4_t pf[TB];
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    pf[tb][i] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][tb][i], cs, shift));
+            }
+            m_run[rb] = m_new;
+            still = still && alpha[rb] == 1.0f;
+#pragma unroll
+            for (int t2 = 0; t2 < TB / 2; ++t2)
+                pp[rb][t2] = half8_t{pf[2 * t2][0], pf[2 * t2][1], pf[2 * t2][2], pf[2 * t2][3],
+                                     pf[2 * t2 + 1][0], pf[2 * t2 + 1][1], pf[2 * t2 + 1][2], pf[2 * t2 + 1][3]};
         }
+        if (!__all(still)) { // (the maximum has moved for some row of the wave)
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                l_acc[rb] *= alpha[rb];
+#pragma unroll
+                for (int db = 0; db < KC; ++db) o[rb][db] *= alpha[rb];
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int t2 = 0; t2 < TB / 2; ++t2)
+                l_acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pp[rb][t2], l_acc[rb], 0, 0, 0);
 #pragma unroll
         for (int db = 0; db < KC; ++db) {
 #pragma unroll
@@ -323,7 +380,9 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
                 half8_t a;
                 __builtin_memcpy(&a, &lo, 8);
                 __builtin_memcpy(reinterpret_cast<char*>(&a) + 8, &hi, 8);
-                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pp[t2], o[db], 0, 0, 0);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+                    o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pp[rb][t2], o[rb][db], 0, 0, 0);
             }
         }
     };
@@ -336,27 +395,30 @@ __global__ __launch_bounds__(256, DH <= 32 ? 5 : DH <= 64 ? 4 : DH <= 96 ? 3 : 2
         if (!wave_has_rows) continue;
         tile_step(kv0);
     }
-    const float l = l_acc[0];
-    if (!valid) return;
-    if (pieces) {
-        const int64_t prow = ((int64_t)b * p.num_heads + head) * p.nsplit + split;
-        float* dst = p.part_o + prow * DH + 4 * g;
 #pragma unroll
-        for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[db];
-        if (g == 0) {
-            p.part_ml[prow * 2] = m_run * cs; // -inf for a piece without (unmasked) keys: weight 0 in the merge
-            p.part_ml[prow * 2 + 1] = l;
+    for (int rb = 0; rb < RB; ++rb) {
+        const float l = l_acc[rb][0];
+        if (!valid[rb]) continue;
+        if (pieces) {
+            const int64_t prow = ((int64_t)b * p.num_heads + head[rb]) * p.nsplit + split;
+            float* dst = p.part_o + prow * DH + 4 * g;
+#pragma unroll
+            for (int db = 0; db < KC; ++db) *reinterpret_cast<float4_t*>(dst + 16 * db) = o[rb][db];
+            if (g == 0) {
+                p.part_ml[prow * 2] = m_run[rb] * cs; // -inf for a piece without (unmasked) keys: weight 0 in the merge
+                p.part_ml[prow * 2 + 1] = l;
+            }
+            continue;
         }
-        return;
-    }
-    // a row whose keys were all masked out has no distribution: zeros
-    const float inv_l = l > 0.f ? 1.0f / l : 0.f;
-    half_t* dst = p.out + ((s0 + tok) * p.num_heads + head) * DH + 4 * g;
+        // a row whose keys were all masked out has no distribution: zeros
+        const float inv_l = l > 0.f ? 1.0f / l : 0.f;
+        half_t* dst = p.out + ((s0 + tok[rb]) * p.num_heads + head[rb]) * DH + 4 * g;
 #pragma unroll
-    for (int db = 0; db < KC; ++db) {
-        const half4_t r = {(half_t)(o[db][0] * inv_l), (half_t)(o[db][1] * inv_l), (half_t)(o[db][2] * inv_l),
-                           (half_t)(o[db][3] * inv_l)};
-        *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
+        for (int db = 0; db < KC; ++db) {
+            const half4_t r = {(half_t)(o[rb][db][0] * inv_l), (half_t)(o[rb][db][1] * inv_l),
+                               (half_t)(o[rb][db][2] * inv_l), (half_t)(o[rb][db][3] * inv_l)};
+            *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
+        }
     }
 }
 
@@ -694,7 +756,7 @@ static int generic_decode_heads_per_wave(const GenericParams& p, int head_dim) {
 }
 
 template <int DH>
-static void launch_one(const GenericParams& p, int64_t blocks, int64_t decode_blocks, hipStream_t stream) {
+static void launch_one(const GenericParams& p, int64_t blocks, int64_t decode_blocks, int row_blocks, hipStream_t stream) {
     if (decode_blocks > 0) { // the decode sequences, a wave per (sequence, kv head or pair of them, piece)
         const dim3 grid((unsigned)decode_blocks), block(256);
         if constexpr (DH <= 96) {
@@ -715,8 +777,15 @@ decode_launched:
     if (blocks > 0) {
         GenericParams t = p;
         if (decode_blocks > 0) t.first_seq = p.split_seqs, t.split_seqs = 0, t.nsplit = 1;
-        hipLaunchKernelGGL(generic_attention_kernel<DH>, dim3((unsigned)blocks), dim3(256), 0, stream, t);
+        if constexpr (gen_two_row_blocks(DH)) {
+            if (row_blocks == 2) {
+                hipLaunchKernelGGL((generic_attention_kernel<DH, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, t);
+                goto tiles_launched;
+            }
+        }
+        hipLaunchKernelGGL((generic_attention_kernel<DH, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, t);
     }
+tiles_launched:
     if (p.nsplit > 1 && p.split_seqs > 0)
         hipLaunchKernelGGL(generic_merge_kernel<DH>,
                            dim3((unsigned)(((int64_t)p.split_seqs * p.num_heads + kGenMergeRows<DH> - 1) / kGenMergeRows<DH>)),
@@ -731,7 +800,9 @@ static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max
     if (!generic_head_dim_supported(head_dim))
         PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 32 between 32 and 256", head_dim);
     p.scale_log2 = kLog2e / sqrtf((float)head_dim);
-    const int64_t tiles = (max_seqlen * p.rep + kGenRows - 1) / kGenRows;
+    // tiles of 128 rows (two blocks of 16 per wave) where a sequence has more than 64 rows
+    const int row_blocks = gen_two_row_blocks(head_dim) && max_seqlen * p.rep > kGenRows ? 2 : 1;
+    const int64_t tiles = (max_seqlen * p.rep + kGenRows * row_blocks - 1) / (kGenRows * row_blocks);
     if (tiles <= 0 || p.batch <= 0) return PPLHIP_RC_SUCCESS;
     // p.split_seqs: the decode sequences (the first of the batch, one new token each, all of whose keys are in the slab)
     if (p.nsplit < 1) p.nsplit = 1;
@@ -753,14 +824,14 @@ static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max
         PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many row tiles");
     p.tiles_max = (int32_t)tiles;
     switch (head_dim) {
-        case 32: launch_one<32>(p, blocks, decode_blocks, stream); break;
-        case 64: launch_one<64>(p, blocks, decode_blocks, stream); break;
-        case 96: launch_one<96>(p, blocks, decode_blocks, stream); break;
-        case 128: launch_one<128>(p, blocks, decode_blocks, stream); break;
-        case 160: launch_one<160>(p, blocks, decode_blocks, stream); break;
-        case 192: launch_one<192>(p, blocks, decode_blocks, stream); break;
-        case 224: launch_one<224>(p, blocks, decode_blocks, stream); break;
-        default: launch_one<256>(p, blocks, decode_blocks, stream); break;
+        case 32: launch_one<32>(p, blocks, decode_blocks, row_blocks, stream); break;
+        case 64: launch_one<64>(p, blocks, decode_blocks, row_blocks, stream); break;
+        case 96: launch_one<96>(p, blocks, decode_blocks, row_blocks, stream); break;
+        case 128: launch_one<128>(p, blocks, decode_blocks, row_blocks, stream); break;
+        case 160: launch_one<160>(p, blocks, decode_blocks, row_blocks, stream); break;
+        case 192: launch_one<192>(p, blocks, decode_blocks, row_blocks, stream); break;
+        case 224: launch_one<224>(p, blocks, decode_blocks, row_blocks, stream); break;
+        default: launch_one<256>(p, blocks, decode_blocks, row_blocks, stream); break;
     }
     PPLHIP_CHECK_LAUNCH("generic_attention");
     return PPLHIP_RC_SUCCESS;
