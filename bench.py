@@ -210,7 +210,12 @@ def cpu_baseline(db, threads, min_seconds=10.0, max_prepare=24):
                        f"resident in host memory")
 
 
-def mfma_sustained(lib, pkg):
+def probe_check(probes, rc, what):
+    if rc:
+        raise RuntimeError("%s failed: %d: %s" % (what, rc, probes.pplhip_probe_last_error().decode()))
+
+
+def mfma_sustained(probes):
     """TFLOP/s of a bare v_mfma_f32_32x32x16_f16 loop on the whole chip, with all-zero and with random fp16 operands:
     the clock the chip holds depends on how many operand bits toggle."""
     import torch
@@ -222,14 +227,14 @@ def mfma_sustained(lib, pkg):
     for name, ops in (("zeros", torch.zeros(2048 * 8, dtype=torch.float16, device="cuda")),
                       ("random_normal", torch.randn(2048 * 8, generator=g, dtype=torch.float16, device="cuda"))):
         flops = C.c_double()
-        call = lambda i: pkg.check(lib.pplhip_probe_mfma_f16(C.c_void_p(ops.data_ptr()), C.c_void_p(dst.data_ptr()),
-                                                              1024, 2000, C.byref(flops), stream), "probe")
+        call = lambda i: probe_check(probes, probes.pplhip_probe_mfma_f16(
+            C.c_void_p(ops.data_ptr()), C.c_void_p(dst.data_ptr()), 1024, 2000, C.byref(flops), stream), "mfma probe")
         mean_ms, med_ms, _ = timed_robust(call, min_warmup=3, min_iters=10, min_ms=100.0, batches=5)
         out[name] = flops.value / (med_ms * 1e-3) / 1e12
     return out
 
 
-def hbm_sustained(lib, pkg):
+def hbm_sustained(probes):
     """GB/s of a plain streaming read of 2 GiB (eight times the memory-side cache) by 512 / 2048 / 8192 workgroups:
     the practical ceiling of this box beside the published HBM peak."""
     import torch
@@ -240,8 +245,8 @@ def hbm_sustained(lib, pkg):
     for wgs in (512, 2048, 8192):
         dst = torch.empty(wgs * 256, dtype=torch.int32, device="cuda")
         got = C.c_uint64()
-        call = lambda i: pkg.check(lib.pplhip_probe_hbm_read(C.c_void_p(src.data_ptr()), n, C.c_void_p(dst.data_ptr()),
-                                                              wgs, C.byref(got), stream), "hbm probe")
+        call = lambda i: probe_check(probes, probes.pplhip_probe_hbm_read(
+            C.c_void_p(src.data_ptr()), n, C.c_void_p(dst.data_ptr()), wgs, C.byref(got), stream), "hbm probe")
         _, med_ms, _ = timed_robust(call, min_warmup=3, min_iters=20, min_ms=100.0, batches=5)
         out["%d_workgroups" % wgs] = got.value / (med_ms * 1e-3) / 1e9
     del src
@@ -438,6 +443,7 @@ def main():
     import torch
     pkg = entry.load_package()
     lib = pkg.load_library()
+    probes = pkg.load_probe_library()  # roofline probes: measurement aids, not part of the drop-in ABI
     from ppl_nn_amd import workloads
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
@@ -486,7 +492,7 @@ def main():
                      "median_ms_per_launch_long_run": dec_med_ms, "long_run_calls": dec_n,
                      "traffic_source": "recorded rocprofv3 --pmc summary under profiles/ (not re-measured in this run)"},
     }
-    stream_gbs = hbm_sustained(lib, pkg)
+    stream_gbs = hbm_sustained(probes)
     result["hbm_read_sustained_GBs"] = dict(
         stream_gbs, note="plain streaming read of 2 GiB measured in this run; the published peak is %.0f" % HBM_PEAK_GBS)
     result["roofline"]["frac_of_sustained_hbm_read"] = gbs / max(stream_gbs.values())
@@ -494,7 +500,7 @@ def main():
     def frac(tflops):
         return tflops / MFMA_FP16_PEAK_TFLOPS
 
-    sustained = mfma_sustained(lib, pkg) if pre_b is not None else None
+    sustained = mfma_sustained(probes) if pre_b is not None else None
     if sustained:
         result["mfma_f16_sustained_tflops"] = dict(
             sustained, note="bare v_mfma_f32_32x32x16_f16 loop on all CUs, measured in this run; the published peak is "

@@ -73,6 +73,9 @@ pplhip_retcode pplhip_init(void);
  * Sequences [0, decoding_batches) are decode steps (exactly one new token each) and attend over the int8 cache,
  * the just-written token included; sequences [decoding_batches, batch) are prefill and attend over the fp16
  * current_key/current_value (or over the cache when cache_prefill != 0, which also allows start_pos > 0).
+ * Without cache_prefill a prefill sequence's keys are exactly its seqlen new tokens on every kernel path: cached
+ * history (start_pos > 0) is not attended to, although its new tokens are still written behind it in the slab and
+ * kvstarts still places the sequence's columns in an attn_mask.
  */
 typedef struct pplhip_mhca_args {
     const void* d_query;
@@ -288,7 +291,7 @@ pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* args, void* stream);
  * rotary_position_embedding_kernel.cc:99-108, which sends NONE to LINEAR and everything else to NONE; this library
  * takes the value at its name.)
  * head_dim and rotary_dim must be multiples of 8, head_dim <= 2048; the half-split layout needs rotary_dim to be a
- * multiple of 16 and head_dim <= 512.
+ * multiple of 16. rotated_query / rotated_key may alias query / key (in-place rotation) in both layouts.
  */
 enum {
     PPLHIP_ROPE_PAIRS_INTERLEAVED = 0,
@@ -382,33 +385,37 @@ pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot
                                     void* stream);
 
 /*
- * Measurement aid (no counterpart in the reference): enqueues `workgroups` x 4 wavefronts that each issue
- * `iterations` x 16 independent v_mfma_f32_32x32x16_f16 on the operands at `d_operands` (2048 x 16 bytes of fp16,
- * device, 16-byte aligned) and write one float per lane to `d_out` (workgroups x 256 floats). `*flops` (host, may be
- * NULL) receives the floating-point operations of the launch. Timing it gives the matrix-core rate this chip sustains
- * for THAT operand data: with random operands the clock is held well below the one the published peak assumes.
+ * Consistency check of the tables of one MultiHeadCacheAttention call, for debugging a scheduler (the attention
+ * kernels trust the tables: one bad entry is an out-of-range slab access, i.e. a GPU fault rather than a wrong
+ * number). The reference has no device-side counterpart; its host harness builds the tables it trusts itself
+ * (tools/benchmark_llama/generation_state.cc:60-192), and its debug builds synchronise after every op
+ * (src/ppl/nn/engines/llm_cuda/kernel.cc:169-177) so that a fault names the op. One small launch reads `args`'
+ * seqstarts / kvstarts / cachestarts / start_pos (never the slab, never the activations) and writes to `d_flag`
+ * (device, 2 x int32): d_flag[0] = one of PPLHIP_TABLES_* (0 = consistent), d_flag[1] = the first offending sequence
+ * (-1 if none). Checked per sequence b: seqlen >= 1; kvlen >= seqlen; start_pos >= 0 and kvlen == start_pos + seqlen;
+ * a decode sequence (b < decoding_batches) has exactly one new token at packed index b; seqlen <= max_seqlen and
+ * kvlen <= max_kvlen; every slab token the sequence owns lies in [0, max_slab_tokens) -- cachestarts[b] + kvlen in the
+ * contiguous mode, every used page of its page-table row (and enough entries in that row) in the paged mode; and
+ * seqstarts[0] == kvstarts[0] == 0, seqstarts[batch] == total_new_tokens. `max_slab_tokens` is the slab's token extent
+ * (MaxT of the cache tensor). Only the table pointers, sizes, cache_mode / page_size / cachestart_stride_b of `args` are
+ * read.
  */
-pplhip_retcode pplhip_probe_mfma_f16(const void* d_operands, void* d_out, int32_t workgroups, int32_t iterations,
-                                     double* flops, void* stream);
-
-/*
- * Measurement aid (no counterpart in the reference): `workgroups` workgroups each stream their own contiguous share
- * of the `bytes` at `d_src` (device, 16-byte aligned) with plain 16-byte loads, eight in flight per lane, and write one
- * word per lane to `d_out` (workgroups x 256 words). `*bytes_read` (host, may be NULL) receives what the launch read
- * (shares are rounded down to whole rounds of 32 KiB). Timed over a buffer much larger than the memory-side cache it
- * gives the streaming-read rate the chip sustains, the practical ceiling beside the published 8 TB/s.
- */
-pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_out, int32_t workgroups,
-                                     uint64_t* bytes_read, void* stream);
-
-/*
- * Verification aid (no counterpart in the reference): the quantiser forms x / s as x * (1 / s), one division per
- * group instead of eight. This call enumerates every absmax (all positive fp16 up to +inf, i.e. every scale the rule
- * max(fp16(absmax / 127), fp16(1e-5)) can produce) with every fp16 x of no larger magnitude or NaN, runs each pair through
- * the library's own quantiser and ADDS to `*d_mismatches` (device, 8 bytes, cleared by the caller) the number of pairs
- * whose int8 differs from int8(rint(fp16(x / s))) formed by a correctly rounded division. 0 is the contract.
- */
-pplhip_retcode pplhip_probe_quantizer(uint64_t* d_mismatches, void* stream);
+enum {
+    PPLHIP_TABLES_OK = 0,
+    PPLHIP_TABLES_BAD_SEQSTARTS = 1,        /* not starting at 0, not increasing, or total != total_new_tokens */
+    PPLHIP_TABLES_BAD_KVSTARTS = 2,         /* not starting at 0, or a kv length below the sequence's new tokens */
+    PPLHIP_TABLES_KVLEN_MISMATCH = 3,       /* kvlen != start_pos + seqlen, or start_pos < 0 */
+    PPLHIP_TABLES_BAD_DECODE_ORDER = 4,     /* a decode sequence without exactly one new token at packed index b */
+    PPLHIP_TABLES_MAX_EXCEEDED = 5,         /* seqlen > max_seqlen or kvlen > max_kvlen */
+    PPLHIP_TABLES_SLAB_RANGE = 6,           /* a slab token outside [0, max_slab_tokens) */
+    PPLHIP_TABLES_PAGE_TABLE_TOO_SHORT = 7  /* paged mode: the sequence needs more pages than its table row holds */
+};
+pplhip_retcode pplhip_check_tables(const pplhip_mhca_args* args, int64_t max_slab_tokens, int32_t* d_flag, void* stream);
+/* The same rules, same codes and same choice of the reported finding (the lowest sequence, then the lowest code)
+ * for a scheduler that builds its tables in host memory, as the reference's harness does before it uploads them
+ * (tools/benchmark_llama/text_generator.cc:233-291): the four table pointers of `args` are HOST pointers here, `flag`
+ * is 2 x int32 in host memory, and no device is touched. */
+pplhip_retcode pplhip_check_tables_host(const pplhip_mhca_args* args, int64_t max_slab_tokens, int32_t* flag);
 
 #ifdef __cplusplus
 }

@@ -200,9 +200,12 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
         for (int h = 0; h < H; ++h) {
             const int kvh = h / rep;
             const int64_t s0 = a->d_seqstarts[b], seqlen = a->d_seqstarts[b + 1] - s0;
-            const int64_t sp = a->d_start_pos[b];
-            const int64_t kvlen = a->d_kvstarts[b + 1] - a->d_kvstarts[b];
             const bool from_cache = (b < a->decoding_batches) || a->enable_cache_prefill;
+            // A prefill sequence of a call without cache-prefill attends over the fp16 rows it brings: exactly seqlen
+            // keys, query t seeing keys 0..t. Cached history (start_pos > 0) is not looked at on that path; kvstarts
+            // only places the sequence's columns in an attn_mask.
+            const int64_t sp = from_cache ? a->d_start_pos[b] : 0;
+            const int64_t kvlen = from_cache ? a->d_kvstarts[b + 1] - a->d_kvstarts[b] : seqlen;
             // materialise this (sequence, kv head)'s keys and values as doubles
             std::vector<double> K((size_t)kvlen * Dh), V((size_t)kvlen * Dh);
             for (int64_t j = 0; j < kvlen; ++j) {
@@ -212,7 +215,7 @@ int oracle_mhca_forward(const pplhip_mhca_args* a, double* out_f64) {
                     dequant_row(cv.row(tok, 0, kvh), cv.srow(tok, 0, kvh), Dh, &K[j * Dh]);
                     dequant_row(cv.row(tok, 1, kvh), cv.srow(tok, 1, kvh), Dh, &V[j * Dh]);
                 } else {
-                    // fp16 path: key j of the sequence is packed row seqstarts[b] + j (start_pos must be 0)
+                    // fp16 path: key j of the sequence is packed row seqstarts[b] + j
                     const uint16_t* kr = CK + ((s0 + j) * KVH + kvh) * Dh;
                     const uint16_t* vr = CV + ((s0 + j) * KVH + kvh) * Dh;
                     for (int d = 0; d < Dh; ++d) {

@@ -11,8 +11,10 @@ from . import cabi
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libppl_llm_kernel_hip.so")
 CONSERVATIVE_WAITS_LIB_PATH = os.path.join(_HERE, "lib", "libppl_llm_kernel_hip_conservative_waits.so")
+PROBES_LIB_PATH = os.path.join(_HERE, "lib", "libppl_llm_kernel_hip_probes.so")
 _LIB = None
 _CHECK_LIB = None
+_PROBES = None
 
 
 class LibraryMissing(RuntimeError):
@@ -51,6 +53,19 @@ def load_conservative_waits_library():
     return _CHECK_LIB
 
 
+def load_probe_library():
+    """The roofline probes and the quantiser enumeration (measurement / verification aids; not part of the drop-in
+    ABI): for the benchmark and the tests only."""
+    global _PROBES
+    if _PROBES is None:
+        if not os.path.exists(PROBES_LIB_PATH):
+            raise LibraryMissing(f"{PROBES_LIB_PATH} is not built; run `python __graft_entry__.py`")
+        load_library()
+        _PROBES = cabi.bind(ctypes.CDLL(PROBES_LIB_PATH), cabi.PROBE_PROTOTYPES)
+        _assert_single_hip_runtime()
+    return _PROBES
+
+
 def _assert_single_hip_runtime():
     paths = set()
     try:
@@ -87,6 +102,7 @@ def load_engine_library():
             "pplnn_hip_last_error": (ctypes.c_char_p, []),
             "pplnn_hip_set_log_level": (None, [ctypes.c_int]),
             "pplnn_hip_engine_create": (vp, [u32, u32]),
+            "pplnn_hip_engine_create_on_stream": (vp, [u32, u32, vp]),
             "pplnn_hip_engine_name": (ctypes.c_char_p, [vp]),
             "pplnn_hip_engine_configure_u32": (u32, [vp, u32, u32]),
             "pplnn_hip_engine_destroy": (None, [vp]),
@@ -108,6 +124,8 @@ def load_engine_library():
             "pplnn_hip_runtime_input": (vp, [vp, u32]),
             "pplnn_hip_runtime_output": (vp, [vp, u32]),
             "pplnn_hip_runtime_run": (u32, [vp]),
+            "pplnn_hip_runtime_run_async": (u32, [vp]),
+            "pplnn_hip_runtime_synchronize": (u32, [vp]),
             "pplnn_hip_runtime_set_profiling": (u32, [vp, u32]),
             "pplnn_hip_runtime_profiling": (u32, [vp, ctypes.POINTER(u64), ctypes.POINTER(u32), u32]),
             "pplnn_hip_runtime_destroy": (None, [vp]),

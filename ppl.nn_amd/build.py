@@ -10,7 +10,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # attention.hip is decode.hip + prefill.hip in one translation unit (it includes them: a call with decode sequences and
 # prompts runs both kinds of workgroup in one launch)
-KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "attention.hip", "pack.hip", "rope.hip", "probe.hip", "generic.hip"]
+KERNEL_SOURCES = ["api.hip", "kv_quant.hip", "attention.hip", "pack.hip", "rope.hip", "generic.hip"]
 KERNEL_INCLUDED = ["decode.hip", "prefill.hip"]
 
 HIP_FLAGS = [
@@ -37,7 +37,7 @@ def build_kernels(force=False, verbose=False, conservative_waits=False):
     tag = "_conservative_waits" if conservative_waits else ""
     out = os.path.join(LIBDIR, f"libppl_llm_kernel_hip{tag}.so")
     srcs = [os.path.join(CSRC, s) for s in KERNEL_SOURCES]
-    deps = srcs + [os.path.join(CSRC, s) for s in KERNEL_INCLUDED] + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "exports.map"),
+    deps = srcs + [os.path.join(CSRC, s) for s in KERNEL_INCLUDED] + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "table_check.h"), os.path.join(CSRC, "exports.map"),
                    os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip.h")]
     if not force and not _newer(out, deps):
         return out
@@ -66,8 +66,29 @@ def build_kernels(force=False, verbose=False, conservative_waits=False):
     return out
 
 
+def build_probes(force=False, verbose=False):
+    """The roofline probes and the quantiser enumeration: measurement / verification aids of the benchmark and one
+    test, in a library of their own so that the product library's ABI does not carry them."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    out = os.path.join(LIBDIR, "libppl_llm_kernel_hip_probes.so")
+    src = os.path.join(CSRC, "probe.hip")
+    deps = [src, os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip_probes.h"),
+            os.path.join(HERE, "..", "include", "ppl_llm_kernel_hip.h")]
+    if not force and not _newer(out, deps):
+        return out
+    cmd = [HIPCC] + HIP_FLAGS + ["-shared", "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), src, "-o", out]
+    if verbose:
+        print(" ".join(cmd))
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        print(p.stdout, file=sys.stderr)
+        raise RuntimeError("hipcc failed")
+    return out
+
+
 def build_all(force=False, verbose=False):
     build_kernels(force=force, verbose=verbose)
+    build_probes(force=force, verbose=verbose)
     build_kernels(force=force, verbose=verbose, conservative_waits=True)
     engine_build = os.path.join(HERE, "engine", "build_engine.py")
     if os.path.exists(engine_build):

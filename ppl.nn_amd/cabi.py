@@ -131,15 +131,25 @@ PROTOTYPES = {
     "pplhip_kv_cache_forward": (_i32, [C.POINTER(KvCacheArgs), _p]),
     "pplhip_pack_tables": (_i32, [C.POINTER(PackArgs), _p]),
     "pplhip_advance_slots": (_i32, [_p, _p, _i32, _p]),
+    "pplhip_check_tables": (_i32, [C.POINTER(MhcaArgs), _i64, _p, _p]),
+    "pplhip_check_tables_host": (_i32, [C.POINTER(MhcaArgs), _i64, _p]),
+}
+
+# the measurement / verification aids of libppl_llm_kernel_hip_probes.so (include/ppl_llm_kernel_hip_probes.h)
+PROBE_PROTOTYPES = {
+    "pplhip_probe_last_error": (C.c_char_p, []),
     "pplhip_probe_mfma_f16": (_i32, [_p, _p, _i32, _i32, C.POINTER(C.c_double), _p]),
     "pplhip_probe_hbm_read": (_i32, [_p, C.c_uint64, _p, _i32, C.POINTER(C.c_uint64), _p]),
     "pplhip_probe_quantizer": (_i32, [_p, _p]),
 }
 
+TABLES_OK, TABLES_BAD_SEQSTARTS, TABLES_BAD_KVSTARTS, TABLES_KVLEN_MISMATCH = 0, 1, 2, 3
+TABLES_BAD_DECODE_ORDER, TABLES_MAX_EXCEEDED, TABLES_SLAB_RANGE, TABLES_PAGE_TABLE_TOO_SHORT = 4, 5, 6, 7
 
-def bind(lib):
+
+def bind(lib, prototypes=None):
     """Attach prototypes to a loaded CDLL; raises AttributeError when a declared symbol is missing."""
-    for name, (res, args) in PROTOTYPES.items():
+    for name, (res, args) in (PROTOTYPES if prototypes is None else prototypes).items():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

@@ -78,6 +78,14 @@ static bool needs_general_kernel(int head_dim, int num_heads, int num_kv_heads, 
     return head_dim != 128 || num_heads / num_kv_heads > 16 || mask != nullptr;
 }
 
+// Workspace of the tuned decode path for `ranges` ranges: partial accumulators and (max, sum) pairs per (slot, head),
+// slots = ranges + decode sequences, then one int per range (its first sequence).
+static uint64_t decode_workspace_bytes(const pplhip_mhca_args* a, int64_t ranges) {
+    if (a->decoding_batches <= 0 || ranges <= 0) return 0;
+    const uint64_t rows = ((uint64_t)ranges + (uint64_t)a->decoding_batches) * a->num_heads;
+    return rows * (a->head_dim + 2) * sizeof(float) + (uint64_t)ranges * sizeof(int32_t);
+}
+
 static pplhip_retcode validate_mask(const void* mask, int64_t stride_h, int64_t stride_q) {
     if (!mask) return PPLHIP_RC_SUCCESS;
     if ((uintptr_t)mask & 1) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "attn_mask must be 2-byte aligned");
@@ -232,9 +240,7 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         if (ranges > 0x3fffffff) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many ranges");
         plan->decode_num_ranges = (int32_t)ranges;
         plan->decode_heads_per_block = hpb;
-        const uint64_t rows = ((uint64_t)ranges + (uint64_t)nd) * a->num_heads;
-        // partial accumulators and (max, sum) pairs per (slot, head), then one int per range (its first sequence)
-        plan->workspace_bytes = rows * (a->head_dim + 2) * sizeof(float) + (uint64_t)ranges * sizeof(int32_t);
+        plan->workspace_bytes = decode_workspace_bytes(a, ranges);
     }
     // ---- prefill
     plan->prefill_q_tile = 128;
@@ -260,6 +266,22 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
     const bool general = needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask);
     if ((plan->general_kernel != 0) != general || (!general && a->decoding_batches > 0 && plan->decode_num_ranges <= 0))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
+    // the plan is checked against the arguments before anything is enqueued: a rejected call leaves the slab untouched,
+    // and the kernels never write past the workspace the plan declares
+    if (general) {
+        if (plan->general_decode_splits < 0 || plan->general_decode_splits > 64 ||
+            generic_workspace_bytes(a, plan->general_decode_splits) > plan->workspace_bytes)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
+    } else {
+        const uint64_t decode_bytes = decode_workspace_bytes(a, plan->decode_num_ranges);
+        bool ok = plan->decode_num_ranges >= 0 && !(plan->decode_num_ranges & 7) && decode_bytes <= plan->workspace_bytes;
+        if (ok && plan->prefill_staging) { // fp16 staging rows of a cache-prefill call, behind the decode partials
+            const uint64_t first = (uint64_t)(uint32_t)plan->prefill_staging_offset_256 * 256;
+            const uint64_t rows = (uint64_t)prefill_staging_tokens(a) * 2 * a->num_kv_heads * a->head_dim * sizeof(uint16_t);
+            ok = plan->prefill_staging_offset_256 >= 0 && first >= decode_bytes && first + rows <= plan->workspace_bytes;
+        }
+        if (!ok) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
+    }
     hipStream_t s = (hipStream_t)stream;
     pplhip_kv_write_args w;
     write_args_from_mhca(a, &w);
@@ -268,9 +290,6 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
         // attend over the slab
         pplhip_retcode rcw = launch_kv_quantize_write(&w, s);
         if (rcw != PPLHIP_RC_SUCCESS) return rcw;
-        if (plan->general_decode_splits < 0 || plan->general_decode_splits > 64 ||
-            generic_workspace_bytes(a, plan->general_decode_splits) > plan->workspace_bytes)
-            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
         return launch_generic_mhca(a, plan->general_decode_splits, d_workspace, s);
     }
     // the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens) into the
@@ -344,9 +363,6 @@ static pplhip_retcode validate_rope(const pplhip_rope_args* a, bool* empty) {
     if (a->pair_layout == PPLHIP_ROPE_PAIRS_HALF_SPLIT && rotary_dim % 16)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "rotary_dim %d: must be a multiple of 16 for the half-split pair layout",
                     rotary_dim);
-    // (the two halves of a pair are read and written by lanes of one wavefront, which keeps in-place rotation safe)
-    if (a->pair_layout == PPLHIP_ROPE_PAIRS_HALF_SPLIT && a->head_dim > 512)
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: at most 512 for the half-split pair layout", a->head_dim);
     if (a->num_heads <= 0 || a->num_key_heads <= 0)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "num_heads %d / num_key_heads %d", a->num_heads, a->num_key_heads);
     if (!(a->theta > 0.f)) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "theta must be positive");
@@ -437,6 +453,30 @@ pplhip_retcode pplhip_pack_tables(const pplhip_pack_args* a, void* stream) {
         !a->d_cachestarts || !a->d_start_pos || !a->d_batch_slots || !a->d_header)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null table pointer");
     return launch_pack_tables(a, (hipStream_t)stream);
+}
+
+static pplhip_retcode validate_check_tables(const pplhip_mhca_args* a, int64_t max_slab_tokens, const int32_t* flag) {
+    if (!a || !flag) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block or flag pointer");
+    if (a->batch < 0 || a->decoding_batches < 0 || a->decoding_batches > a->batch || max_slab_tokens < 0)
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "check_tables: batch %lld, decoding_batches %lld, max_slab_tokens %lld",
+                    (long long)a->batch, (long long)a->decoding_batches, (long long)max_slab_tokens);
+    if (a->batch >= (int64_t(1) << 31)) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "check_tables: too many sequences");
+    if (a->batch > 0 && (!a->d_seqstarts || !a->d_kvstarts || !a->d_cachestarts || !a->d_start_pos))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null table pointer");
+    return validate_cache_mode(a->cache_mode, a->page_size, a->cachestart_stride_b);
+}
+
+pplhip_retcode pplhip_check_tables(const pplhip_mhca_args* a, int64_t max_slab_tokens, int32_t* d_flag, void* stream) {
+    const pplhip_retcode rc = validate_check_tables(a, max_slab_tokens, d_flag);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    return launch_check_tables(a, max_slab_tokens, d_flag, (hipStream_t)stream);
+}
+
+pplhip_retcode pplhip_check_tables_host(const pplhip_mhca_args* a, int64_t max_slab_tokens, int32_t* flag) {
+    const pplhip_retcode rc = validate_check_tables(a, max_slab_tokens, flag);
+    if (rc != PPLHIP_RC_SUCCESS) return rc;
+    check_tables_host(a, max_slab_tokens, flag);
+    return PPLHIP_RC_SUCCESS;
 }
 
 pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot_newlen, int32_t num_slots,

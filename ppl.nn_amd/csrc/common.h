@@ -195,6 +195,8 @@ pplhip_retcode launch_position_index(const int64_t* d_seqstarts, const int64_t* 
                                      int64_t total_tokens, int64_t* d_out, hipStream_t stream);
 pplhip_retcode launch_pack_tables(const pplhip_pack_args* a, hipStream_t stream);
 pplhip_retcode launch_advance_slots(int64_t* kvlen, const int64_t* newlen, int n, hipStream_t stream);
+pplhip_retcode launch_check_tables(const pplhip_mhca_args* a, int64_t max_slab_tokens, int32_t* d_flag, hipStream_t stream);
+void check_tables_host(const pplhip_mhca_args* a, int64_t max_slab_tokens, int32_t* flag);
 
 } // namespace pplhip
 

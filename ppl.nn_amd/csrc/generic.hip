@@ -40,6 +40,8 @@ struct GenericParams {
     half_t* out; // [S, H, DH]
     int32_t batch, num_heads, kv_heads, rep;
     int32_t first_fp16_seq; // sequences [0, first_fp16_seq) read the slab, the others the fp16 rows
+    int32_t k16_holds_new_tokens; // the fp16 rows are the sequences' NEW tokens only (MultiHeadCacheAttention's
+                                  // current_key / current_value), packed by seqstarts: such a sequence has seqlen keys
     int32_t is_causal;
     int32_t tiles_max; // row tiles of the longest sequence
     float scale_log2; // log2(e) / sqrt(DH)
@@ -107,12 +109,16 @@ void generic_attention_kernel(const GenericParams p) {
     const int64_t s0 = p.seqstarts[b];
     const int64_t L = p.seqstarts[b + 1] - s0;
     const int64_t kv_first = p.kvstarts[b];
-    const int64_t kvlen = p.kvstarts[b + 1] - kv_first;
+    const bool from_slab = b < p.first_fp16_seq;
+    // The prompts of a MultiHeadCacheAttention call without cache-prefill attend over the fp16 rows they bring:
+    // current_key / current_value hold exactly L rows for the sequence, whatever kvstarts says (a start_pos > 0 is
+    // history that such a call does not look at), so its keys are those L rows. kvstarts still places the sequence's
+    // columns in an attn_mask.
+    const int64_t kvlen = (!from_slab && p.k16_holds_new_tokens) ? L : p.kvstarts[b + 1] - kv_first;
     const int64_t rows = L * p.rep;
     const int64_t row0 = (int64_t)tile * GR;
     if (row0 >= rows || kvlen <= 0) return;
     const int64_t sp = kvlen > L ? kvlen - L : 0;
-    const bool from_slab = b < p.first_fp16_seq;
     const int64_t k16_row0 = from_slab ? 0 : p.k16_starts[b];
 
     const int tid = threadIdx.x;
@@ -893,6 +899,7 @@ pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* 
     // decode sequences always attend over the slab; prompts only in a cache-prefill call (otherwise over the fp16 rows
     // they bring, like the specialised path)
     p.first_fp16_seq = a->enable_cache_prefill ? (int32_t)a->batch : (int32_t)a->decoding_batches;
+    p.k16_holds_new_tokens = 1;
     p.is_causal = a->is_causal;
     const int64_t max_rows_tokens = a->batch > a->decoding_batches ? a->max_seqlen : 1;
     return launch_generic(p, a->head_dim, max_rows_tokens, stream);
@@ -923,6 +930,7 @@ pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream) 
     p.kv_heads = a->num_kv_heads;
     p.rep = a->num_heads / a->num_kv_heads;
     p.first_fp16_seq = 0;
+    p.k16_holds_new_tokens = 0; // key / value hold every key of a sequence, packed by kvstarts
     p.is_causal = a->is_causal;
     return launch_generic(p, a->head_dim, a->max_seqlen, stream);
 }

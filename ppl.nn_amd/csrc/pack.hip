@@ -3,6 +3,7 @@
 // At most 1024 slots, so one workgroup does everything in LDS; the kernel is latency-bound (a few microseconds)
 // and replaces eight host-to-device uploads per step.
 #include "common.h"
+#include "table_check.h"
 
 namespace pplhip {
 
@@ -138,6 +139,52 @@ pplhip_retcode launch_advance_slots(int64_t* kvlen, const int64_t* newlen, int n
     hipLaunchKernelGGL(advance_slots_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, kvlen, newlen, n);
     PPLHIP_CHECK_LAUNCH("advance_slots");
     return PPLHIP_RC_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Consistency check of one call's tables (a debugging aid: the attention kernels trust the tables, and one bad entry
+// is an out-of-range slab access). Reads the tables only; never touches the slab. One workgroup walks the sequences;
+// the lowest (sequence, code) pair found wins, so the report does not depend on thread timing.
+__global__ __launch_bounds__(256) void check_tables_kernel(const TableView p, int32_t* flag) {
+    __shared__ unsigned long long first_bad;
+    if (threadIdx.x == 0) first_bad = check_table_ends(p);
+    __syncthreads();
+    for (int64_t b = threadIdx.x; b < p.batch; b += blockDim.x) {
+        const int code = check_table_sequence(p, b);
+        if (code != PPLHIP_TABLES_OK) atomicMin(&first_bad, (unsigned long long)table_finding(b, code));
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const bool bad = first_bad != kNoTableFinding;
+        flag[0] = bad ? (int32_t)(first_bad & 0xff) : PPLHIP_TABLES_OK; // [0] = code, [1] = first offending sequence
+        flag[1] = bad ? (int32_t)(first_bad >> 8) : -1;
+    }
+}
+
+TableView table_view_of(const pplhip_mhca_args* a, int64_t max_slab_tokens) {
+    return TableView{a->d_seqstarts, a->d_kvstarts, a->d_cachestarts, a->d_start_pos, a->batch, a->decoding_batches,
+                     a->max_seqlen, a->max_kvlen, a->total_new_tokens, max_slab_tokens, a->cachestart_stride_b,
+                     page_shift_of(a->cache_mode, a->page_size)};
+}
+
+pplhip_retcode launch_check_tables(const pplhip_mhca_args* a, int64_t max_slab_tokens, int32_t* d_flag,
+                                   hipStream_t stream) {
+    hipLaunchKernelGGL(check_tables_kernel, dim3(1), dim3(256), 0, stream, table_view_of(a, max_slab_tokens), d_flag);
+    PPLHIP_CHECK_LAUNCH("check_tables");
+    return PPLHIP_RC_SUCCESS;
+}
+
+// the same rules over tables that live in host memory
+void check_tables_host(const pplhip_mhca_args* a, int64_t max_slab_tokens, int32_t* flag) {
+    const TableView p = table_view_of(a, max_slab_tokens);
+    uint64_t first_bad = check_table_ends(p);
+    for (int64_t b = 0; b < p.batch; ++b) {
+        const int code = check_table_sequence(p, b);
+        if (code != PPLHIP_TABLES_OK && table_finding(b, code) < first_bad) first_bad = table_finding(b, code);
+    }
+    const bool bad = first_bad != kNoTableFinding;
+    flag[0] = bad ? (int32_t)(first_bad & 0xff) : PPLHIP_TABLES_OK;
+    flag[1] = bad ? (int32_t)(first_bad >> 8) : -1;
 }
 
 } // namespace pplhip

@@ -3,9 +3,22 @@
 // the caller supplies. The rate this chip SUSTAINS depends on the operand data (power management lowers the clock when
 // the operands toggle many bits): the benchmark reports the prefill kernel next to the published peak and next to
 // this measured figure for random fp16 operands.
+// Built into a library of its own (the probes are not part of the drop-in ABI); quantize_group8 is the kernel library's
+// own inline quantiser, compiled here with the same flags.
+#include <stdarg.h>
+
 #include "common.h"
+#include "../../include/ppl_llm_kernel_hip_probes.h"
 
 namespace pplhip {
+
+static thread_local char g_probe_error[256] = "";
+void set_error(const char* fmt, ...) { // (this library's copy: PPLHIP_FAIL writes here)
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_probe_error, sizeof(g_probe_error), fmt, ap);
+    va_end(ap);
+}
 
 constexpr int kProbeMfmaPerIter = 16;
 
@@ -62,6 +75,10 @@ __global__ __launch_bounds__(256) void probe_hbm_read_kernel(const u32x4_probe_t
 } // namespace pplhip
 
 using namespace pplhip;
+
+extern "C" const char* pplhip_probe_last_error(void) {
+    return g_probe_error;
+}
 
 extern "C" pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_out, int32_t workgroups,
                                                 uint64_t* bytes_read, void* stream) {

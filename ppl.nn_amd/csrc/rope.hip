@@ -88,9 +88,9 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
         sin_tab[i] = sinf((float)a);
     }
     __syncthreads();
-    if (slot >= rows_per_pass) return;
+    const bool lane_has_rows = slot < rows_per_pass; // 256 need not be a multiple of the chunks per row
     float cs[8], sn[8];
-    if (rotate) {
+    if (rotate && lane_has_rows) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             if (j < npairs) {
@@ -102,20 +102,32 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     // rows of a token: query heads, key heads and, when the launch also fills the slab, value heads
     const int rows = p.num_heads + p.num_key_heads * (WRITE_KV ? 2 : 1);
     const int64_t slab_tok = WRITE_KV ? p.pages.token(b, sp + (t - s0)) : 0;
-    for (int r = slot; r < rows; r += rows_per_pass) {
+    // Half-split pairs rotated in place (outputs aliasing inputs): a lane reads its partner's chunk, which the partner
+    // overwrites. Within a wavefront every lane's loads are issued before any lane's store. When the chunks per row do
+    // not divide 64 (head_dim 80, 96, 160, ...) a row's lanes can sit in two wavefronts, so a pass then loads, meets
+    // at a workgroup barrier, and stores: every thread walks the same number of passes.
+    const bool sync_pass = p.half_split && (kWave % cpr) != 0;
+    for (int r0 = 0; r0 < rows; r0 += rows_per_pass) {
+        const int r = r0 + slot;
+        const bool active = lane_has_rows && r < rows;
         const bool is_value = WRITE_KV && r >= p.num_heads + p.num_key_heads;
         const bool is_key = r >= p.num_heads && !is_value;
         const int head = is_value ? r - p.num_heads - p.num_key_heads : (is_key ? r - p.num_heads : r);
         const int64_t off = ((t * (is_key || is_value ? p.num_key_heads : p.num_heads) + head) * (int64_t)p.head_dim) + 8 * chunk;
         const half_t* src = is_value ? p.v : (is_key ? p.k : p.q);
-        const uint4 raw = *reinterpret_cast<const uint4*>(src + off);
+        const bool rotated = active && rotate && !is_value && !(is_key && p.bypass_key);
+        uint4 raw = make_uint4(0, 0, 0, 0), other = make_uint4(0, 0, 0, 0);
+        if (active) raw = *reinterpret_cast<const uint4*>(src + off);
+        // the other halves of this lane's pairs
+        if (rotated && p.half_split) other = *reinterpret_cast<const uint4*>(src + off + (upper ? -half : half));
+        if (sync_pass) __syncthreads();
+        if (!active) continue;
         uint4 res = raw;
-        if (rotate && !is_value && !(is_key && p.bypass_key)) {
+        if (rotated) {
             half_t x[8], y[8];
             __builtin_memcpy(x, &raw, 16);
             if (p.half_split) {
-                half_t o[8]; // the other halves of this lane's pairs
-                const uint4 other = *reinterpret_cast<const uint4*>(src + off + (upper ? -half : half));
+                half_t o[8];
                 __builtin_memcpy(o, &other, 16);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {

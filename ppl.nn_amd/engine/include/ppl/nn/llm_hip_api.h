@@ -216,6 +216,13 @@ enum {
         channels (2i, 2i+1); 1 = channel i with channel i + rotary_dim/2 ("rotate_half"). The op has no attribute for
         it and the reference's kernel is not in its tree, so the integrator states what the checkpoint was exported for */
     ENGINE_CONF_ROPE_PAIR_LAYOUT = 1006,
+    /** uint32_t, llm_hip only, debugging: before MultiHeadCacheAttention trusts its tables, run the kernel library's
+        table check (pplhip_check_tables) against the cache tensor's token extent, wait for it, and fail the op with
+        RC_INVALID_VALUE (naming the rule and the sequence) instead of launching attention on a bad table */
+    ENGINE_CONF_DEBUG_CHECK_TABLES = 1007,
+    /** uint32_t, llm_hip only, debugging: wait for the stream after every op and report the op a device error belongs
+        to; what the reference's debug builds do unconditionally (src/ppl/nn/engines/llm_cuda/kernel.cc:169-177) */
+    ENGINE_CONF_DEBUG_SYNC_AFTER_OP = 1008,
     ENGINE_CONF_INTERNAL_MAX,
 };
 

@@ -24,6 +24,14 @@ void* pplnn_hip_engine_create(uint32_t device_id, uint32_t mm_policy) {
     options.mm_policy = mm_policy;
     return llm::hip::EngineFactory::Create(options);
 }
+// every Runtime of the engine enqueues on the caller's stream (EngineOptions::runtime_stream) instead of one of its own
+void* pplnn_hip_engine_create_on_stream(uint32_t device_id, uint32_t mm_policy, void* stream) {
+    llm::hip::EngineOptions options;
+    options.device_id = device_id;
+    options.mm_policy = mm_policy;
+    options.runtime_stream = stream;
+    return llm::hip::EngineFactory::Create(options);
+}
 const char* pplnn_hip_engine_name(void* e) { return static_cast<Engine*>(e)->GetName(); }
 uint32_t pplnn_hip_engine_configure_u32(void* e, uint32_t option, uint32_t value) {
     return static_cast<Engine*>(e)->Configure(option, value);
@@ -86,6 +94,8 @@ uint32_t pplnn_hip_runtime_output_count(void* r) { return static_cast<Runtime*>(
 void* pplnn_hip_runtime_input(void* r, uint32_t i) { return static_cast<Runtime*>(r)->GetInputTensor(i); }
 void* pplnn_hip_runtime_output(void* r, uint32_t i) { return static_cast<Runtime*>(r)->GetOutputTensor(i); }
 uint32_t pplnn_hip_runtime_run(void* r) { return static_cast<Runtime*>(r)->Run(); }
+uint32_t pplnn_hip_runtime_run_async(void* r) { return static_cast<Runtime*>(r)->RunAsync(); }
+uint32_t pplnn_hip_runtime_synchronize(void* r) { return static_cast<Runtime*>(r)->Synchronize(); }
 uint32_t pplnn_hip_runtime_set_profiling(void* r, uint32_t on) {
     return static_cast<Runtime*>(r)->Configure(RUNTIME_CONF_SET_KERNEL_PROFILING_FLAG, on);
 }

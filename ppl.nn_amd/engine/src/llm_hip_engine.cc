@@ -35,25 +35,38 @@ struct EngineConfig final { // src/ppl/nn/engines/llm_cuda/engine_config.h:25-36
     // which channels RotaryPositionEmbedding rotates together (PPLHIP_ROPE_PAIRS_*): not an attribute of the op, so
     // the integrator states it per engine for the checkpoint family being served
     int32_t rope_pair_layout = PPLHIP_ROPE_PAIRS_INTERLEAVED;
+    // debugging aids (off by default): the device-side table check in front of MultiHeadCacheAttention, and a wait for
+    // the stream after every op (the reference's debug builds: kernel.cc:169-177)
+    bool debug_check_tables = false;
+    bool debug_sync_after_op = false;
 };
 
 // The strides of an attn_mask tensor in the C ABI's terms: shape [S, K] (one mask for all heads) or [H, S, K] (one per
 // head), K >= kvstarts[batch] (exporters pad the last extent to a multiple of 8).
-static RetCode MaskStrides(const TensorImpl* mask, int num_heads, int64_t* stride_h, int64_t* stride_q) {
+// The kernels index the mask unchecked, so what can be checked on the host is: fp16 elements, one row per packed query
+// token (`tokens` of them), and at least `min_keys` columns (the longest sequence's keys; the packed key total is only
+// known on the device).
+static RetCode MaskStrides(const TensorImpl* mask, int num_heads, int64_t tokens, int64_t min_keys, int64_t* stride_h,
+                           int64_t* stride_q) {
     const TensorShape* sh = mask->GetShape();
     const uint32_t n = sh->GetDimCount();
-    if (n == 2) {
-        *stride_h = 0;
-        *stride_q = sh->GetDim(1);
-        return RC_SUCCESS;
+    if (sh->GetDataType() != DATATYPE_FLOAT16) {
+        LOG(ERROR) << "attn_mask must be fp16";
+        return RC_INVALID_VALUE;
     }
-    if (n == 3 && (sh->GetDim(0) == num_heads || sh->GetDim(0) == 1)) {
-        *stride_h = sh->GetDim(0) == 1 ? 0 : sh->GetDim(1) * sh->GetDim(2);
-        *stride_q = sh->GetDim(2);
-        return RC_SUCCESS;
+    if (!((n == 2) || (n == 3 && (sh->GetDim(0) == num_heads || sh->GetDim(0) == 1)))) {
+        LOG(ERROR) << "attn_mask must be [tokens, keys] or [num_heads, tokens, keys]";
+        return RC_INVALID_VALUE;
     }
-    LOG(ERROR) << "attn_mask must be [tokens, keys] or [num_heads, tokens, keys]";
-    return RC_INVALID_VALUE;
+    const int64_t rows = sh->GetDim(n - 2), cols = sh->GetDim(n - 1);
+    if (rows < tokens || cols < min_keys) {
+        LOG(ERROR) << "attn_mask holds " << rows << " rows x " << cols << " keys; the call has " << tokens
+                   << " query tokens and sequences of up to " << min_keys << " keys";
+        return RC_INVALID_VALUE;
+    }
+    *stride_h = (n == 3 && sh->GetDim(0) != 1) ? rows * cols : 0;
+    *stride_q = cols;
+    return RC_SUCCESS;
 }
 
 // ---------------------------------------------------------------- device
@@ -196,6 +209,14 @@ public:
             timed_ = true;
         }
         if (rc != RC_SUCCESS) return rc;
+        if (GetEngineConfig().debug_sync_after_op) { // kernel.cc:169-177 (the reference's debug builds)
+            const hipError_t serr = hipStreamSynchronize(stream);
+            if (serr != hipSuccess) {
+                LOG(ERROR) << "hipStreamSynchronize after kernel[" << GetName() << "] failed: " << (int)serr << ", "
+                           << hipGetErrorString(serr);
+                return RC_DEVICE_RUNTIME_ERROR;
+            }
+        }
         const hipError_t err = hipGetLastError(); // kernel.cc:179-185
         if (err != hipSuccess) {
             LOG(ERROR) << "exec kernel[" << GetName() << "] of type[" << GetType().domain << ":" << GetType().name
@@ -384,7 +405,8 @@ protected:
         a.d_current_value = current_value->GetBufferPtr();
         a.d_attn_mask = attn_mask_data;
         if (attn_mask_data) {
-            const RetCode mrc = MaskStrides(attn_mask, param_->num_heads, &a.attn_mask_stride_h, &a.attn_mask_stride_q);
+            const RetCode mrc = MaskStrides(attn_mask, param_->num_heads, query->GetShape()->GetDim(0), max_kvlen_val,
+                                            &a.attn_mask_stride_h, &a.attn_mask_stride_q);
             if (mrc != RC_SUCCESS) return mrc;
         }
         a.d_seqstarts = seqstarts->GetBufferPtr<int64_t>();
@@ -419,6 +441,13 @@ protected:
         auto krc = CheckKernelRc(pplhip_mhca_prepare(&a, &plan), GetName());
         if (krc != PPLHIP_RC_SUCCESS) return (RetCode)krc;
 
+        if (GetEngineConfig().debug_check_tables) {
+            // token extent of the slab: dim 0 of (MaxT, L, 2, H, Dh), dim 3 of (L, 2, H, MaxT, Dh)
+            const int64_t max_slab_tokens = cache->GetShape()->GetDim(param_->cache_layout == 0 ? 0 : 3);
+            const RetCode trc = CheckTables(a, max_slab_tokens);
+            if (trc != RC_SUCCESS) return trc;
+        }
+
         BufferDesc tmp;
         auto status = GetHipDevice()->AllocTmpBuffer(plan.workspace_bytes, &tmp);
         if (status != RC_SUCCESS) {
@@ -433,6 +462,35 @@ protected:
     }
 
 private:
+    // ENGINE_CONF_DEBUG_CHECK_TABLES: the kernels trust seqstarts / kvstarts / cachestarts / start_pos, and one bad entry
+    // is an out-of-range slab access. The check reads the tables only; attention is not launched when it finds
+    // something.
+    RetCode CheckTables(const pplhip_mhca_args& a, int64_t max_slab_tokens) {
+        static const char* const kRule[] = {
+            "consistent", "seqstarts (must start at 0, increase, and end at the query's token count)",
+            "kvstarts (must start at 0; a sequence has at least its new tokens as keys)",
+            "kvlen != start_pos + seqlen (or start_pos < 0)",
+            "a decode sequence must bring exactly one new token, packed at its sequence index",
+            "seqlen > max_seqlen or kvlen > max_kvlen", "a slab token outside the cache tensor's token extent",
+            "the page table row is shorter than the sequence's pages"};
+        BufferDesc flag_buf;
+        auto status = GetHipDevice()->AllocTmpBuffer(2 * sizeof(int32_t), &flag_buf);
+        if (status != RC_SUCCESS) return status;
+        int32_t flag[2] = {0, -1};
+        auto krc = CheckKernelRc(pplhip_check_tables(&a, max_slab_tokens, (int32_t*)flag_buf.addr, GetStream()), GetName());
+        if (krc == PPLHIP_RC_SUCCESS) status = GetHipDevice()->CopyToHost(flag, flag_buf, sizeof(flag)); // waits
+        GetHipDevice()->FreeTmpBuffer(&flag_buf);
+        if (krc != PPLHIP_RC_SUCCESS) return (RetCode)krc;
+        if (status != RC_SUCCESS) return status;
+        if (flag[0] != PPLHIP_TABLES_OK) {
+            LOG(ERROR) << "kernel[" << GetName() << "]: inconsistent tables at sequence " << flag[1] << ": "
+                       << (flag[0] > 0 && flag[0] < 8 ? kRule[flag[0]] : "unknown rule") << " (slab of "
+                       << max_slab_tokens << " tokens)";
+            return RC_INVALID_VALUE;
+        }
+        return RC_SUCCESS;
+    }
+
     const opmx::MultiHeadCacheAttentionParam* param_;
 };
 
@@ -602,7 +660,9 @@ protected:
         a.d_value = value->GetBufferPtr();
         a.d_attn_mask = attn_mask_data;
         if (attn_mask_data) {
-            const RetCode mrc = MaskStrides(attn_mask, param_->num_heads, &a.attn_mask_stride_h, &a.attn_mask_stride_q);
+            // (the packed keys of all sequences are the rows of `key`: the mask must have a column for each)
+            const RetCode mrc = MaskStrides(attn_mask, param_->num_heads, query->GetShape()->GetDim(0),
+                                            key->GetShape()->GetDim(0), &a.attn_mask_stride_h, &a.attn_mask_stride_q);
             if (mrc != RC_SUCCESS) return mrc;
         }
         a.d_seqstarts = seqstarts->GetBufferPtr<int64_t>();
@@ -1008,6 +1068,8 @@ public:
                 }
                 break;
             }
+            case ENGINE_CONF_DEBUG_CHECK_TABLES: config_.debug_check_tables = va_arg(args, uint32_t) ? true : false; break;
+            case ENGINE_CONF_DEBUG_SYNC_AFTER_OP: config_.debug_sync_after_op = va_arg(args, uint32_t) ? true : false; break;
             default:
                 LOG(ERROR) << "invalid option[" << option << "] >= [" << (uint32_t)ENGINE_CONF_INTERNAL_MAX << "]";
                 rc = RC_INVALID_VALUE;

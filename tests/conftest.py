@@ -24,3 +24,10 @@ def hiplib():
     """The HIP kernel library through its C ABI; GPU tests fail (not skip) when it is not built."""
     import harness
     return harness.pkg.load_library()
+
+
+@pytest.fixture(scope="session")
+def probelib():
+    """The measurement / verification aids (roofline probes, quantiser enumeration): a library of their own."""
+    import harness
+    return harness.pkg.load_probe_library()

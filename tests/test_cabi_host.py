@@ -10,10 +10,11 @@ import harness
 from harness import cabi, workloads
 
 HEADER = os.path.join(harness.ROOT, "include", "ppl_llm_kernel_hip.h")
+PROBES_HEADER = os.path.join(harness.ROOT, "include", "ppl_llm_kernel_hip_probes.h")
 
 
-def header_text():
-    with open(HEADER) as f:
+def header_text(path=HEADER):
+    with open(path) as f:
         return f.read()
 
 
@@ -25,6 +26,18 @@ def test_library_exports_every_declared_symbol(hiplib):
         assert hasattr(hiplib, name)
     assert hiplib.pplhip_version() >= 100
     assert hiplib.pplhip_last_error() is not None
+    assert not any("probe" in name for name in declared)  # the drop-in ABI carries no measurement aids
+
+
+def test_probe_library_exports_every_declared_symbol(probelib):
+    txt = re.sub(r"/\*.*?\*/", "", header_text(PROBES_HEADER), flags=re.S)
+    declared = set(re.findall(r"\b(pplhip_[a-z0-9_]+)\s*\(", txt))
+    assert declared == set(cabi.PROBE_PROTOTYPES), declared ^ set(cabi.PROBE_PROTOTYPES)
+    for name in declared:
+        assert hasattr(probelib, name)
+    assert probelib.pplhip_probe_last_error() == b""
+    assert probelib.pplhip_probe_quantizer(None, None) == cabi.RC_INVALID_VALUE  # host-side check, no device call
+    assert b"null counter" in probelib.pplhip_probe_last_error()
 
 
 @pytest.mark.parametrize("cname,cls", [("pplhip_mhca_args", cabi.MhcaArgs), ("pplhip_mhca_plan", cabi.MhcaPlan),

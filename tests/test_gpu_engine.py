@@ -424,3 +424,84 @@ def test_debug_dumps_and_step_replay(hiplib, tmp_path):
     bad[0] = str(tmp_path / "query.dat")
     assert eng.pplnn_hip_runtime_set_inputs_from_files(s.rt, ",".join(bad).encode()) == cabi.RC_INVALID_VALUE  # name
     s.close()
+
+
+def test_engine_debug_options_check_tables_and_sync(hiplib):
+    """ENGINE_CONF_DEBUG_CHECK_TABLES (1007): a bad table entry fails the op with RC_INVALID_VALUE before any attention
+    kernel is launched (the check reads the tables only, so nothing faults), good tables run as usual; with
+    ENGINE_CONF_DEBUG_SYNC_AFTER_OP (1008) every op is followed by a wait for the stream. The slab is poisoned with a
+    pattern first: a refused call must leave every byte of it as it was."""
+    import torch
+    eng = harness.pkg.load_engine_library()
+    eng.pplnn_hip_set_log_level(4)
+    b = workloads.Batch(8, 2, 128, [1, 1, 70], [300, 9, 0], 2, slack_tokens=1, name="engine_debug")
+    t = workloads.make_tensors(b, seed=15)
+    ref = harness.run_oracle(b, t)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    before = cache.clone()
+
+    def run(tables, configure):
+        s = Session(eng, ow.mhca_model(8, 2, 128, 1, 0), configure=configure)
+        for i, name in enumerate(("query", "current_key", "current_value")):
+            s.set_device_tensor(i, harness.to_dev(t[name]))
+        for i, tab in enumerate(tables):
+            s.set_table(3 + i, tab)
+        for i, v in enumerate((b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+            s.set_host_scalar(7 + i, v)
+        s.set_device_tensor(10, cache)
+        s.set_device_tensor(11, scale)
+        rc = eng.pplnn_hip_runtime_run(s.rt)
+        out = s.output(0, np.float16) if rc == 0 else None
+        s.close()
+        return rc, out
+
+    good = (b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)
+    past_the_slab = b.cachestarts.copy()
+    past_the_slab[2] = b.max_tokens - 3  # the prompt's 70 tokens would run past the end of the cache tensor
+    wrong_kvlen = b.start_pos.copy()
+    wrong_kvlen[0] = 299
+    for name, tables in (("slab range", (b.seqstarts, b.kvstarts, past_the_slab, b.start_pos)),
+                         ("kvlen", (b.seqstarts, b.kvstarts, b.cachestarts, wrong_kvlen))):
+        print(f"case engine check_tables: {name}", flush=True)
+        rc, _ = run(tables, [(1007, 1), (1008, 1)])
+        assert rc == cabi.RC_INVALID_VALUE
+        assert b"inconsistent tables" in eng.pplnn_hip_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(cache, before), "a refused call wrote to the slab"
+    rc, out = run(good, [(1007, 1), (1008, 1)])
+    assert rc == 0, eng.pplnn_hip_last_error()
+    harness.assert_attn_close(out, ref["output_f64"])
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), ref["cache"])
+
+
+def test_engine_rejects_masks_it_cannot_index(hiplib):
+    """attn_mask is indexed unchecked by the kernels: the engine refuses an fp32 mask, one with fewer rows than query
+    tokens, and one with fewer columns than the longest sequence has keys."""
+    eng = harness.pkg.load_engine_library()
+    eng.pplnn_hip_set_log_level(4)
+    import torch
+    b = workloads.Batch(8, 2, 64, [1, 40], [90, 0], 1, name="engine_mask_checks")
+    t = workloads.make_tensors(b, seed=16)
+    cache, scale = _prepare_slab(b, t, hiplib)
+    S, K = b.total_new_tokens, int(b.kvstarts[-1])
+
+    def run(mask):
+        s = Session(eng, ow.mhca_model(8, 2, 64, 1, 0, mask_rank=2))
+        for i, name in enumerate(("query", "current_key", "current_value")):
+            s.set_device_tensor(i, harness.to_dev(t[name]))
+        for i, tab in enumerate((b.seqstarts, b.kvstarts, b.cachestarts, b.start_pos)):
+            s.set_table(3 + i, tab)
+        for i, v in enumerate((b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+            s.set_host_scalar(7 + i, v)
+        s.set_device_tensor(10, cache)
+        s.set_device_tensor(11, scale)
+        s.set_device_tensor(12, mask)
+        rc = eng.pplnn_hip_runtime_run(s.rt)
+        s.close()
+        return rc
+
+    f16 = dict(dtype=torch.float16, device="cuda")
+    assert run(torch.zeros((S, (K + 7) // 8 * 8), **f16)) == 0, eng.pplnn_hip_last_error()
+    assert run(torch.zeros((S - 1, (K + 7) // 8 * 8), **f16)) == cabi.RC_INVALID_VALUE
+    assert run(torch.zeros((S, b.max_kvlen - 1), **f16)) == cabi.RC_INVALID_VALUE

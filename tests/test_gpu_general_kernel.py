@@ -200,3 +200,22 @@ def test_key_value_cache_op_other_head_dim(hiplib, olib):
     f16 = lambda x: x.cpu().view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(cd.cpu().numpy(), co) and np.array_equal(f16(sd), so.view(np.uint16))
     assert np.array_equal(f16(kd), ko.view(np.uint16)) and np.array_equal(f16(vd), vo.view(np.uint16))
+
+
+@pytest.mark.parametrize("Dh", [64, 128])
+def test_prompt_with_history_but_no_cache_prefill_sees_its_new_tokens_only(Dh):
+    """A prompt with start_pos > 0 in a call WITHOUT cache-prefill (a chunk whose history the caller chose not to
+    attend to): current_key / current_value hold only its seqlen rows, so its keys are those rows on every path. The
+    general path (here through an all-zero mask at head_dim 128, and natively at 64) must agree with the oracle and,
+    at head_dim 128, with the tuned path; the last sequence's rows end exactly at the end of current_key."""
+    b = workloads.Batch(8, 2, Dh, [1, 1, 70, 33, 130], [40, 900, 300, 0, 77], 2, num_layer=2, layer_idx=1,
+                        name="general_prompt_history")
+    t = workloads.make_tensors(b, seed=91 + Dh)
+    zero_mask = np.zeros((b.total_new_tokens, (int(b.kvstarts[-1]) + 7) // 8 * 8), np.float16)
+    ref, got = check(b, t, f"prompt history, no cache-prefill, Dh {Dh}", mask=zero_mask)
+    if Dh == 128:
+        tuned = harness.run_device(b, t)
+        harness.assert_attn_close(tuned["output"], ref["output_f64"], what="tuned path")
+        assert np.array_equal(tuned["cache"], got["cache"])
+    else:
+        check(b, t, f"prompt history, no cache-prefill, no mask, Dh {Dh}")

@@ -53,10 +53,11 @@ def test_rope_vs_oracle(hiplib, olib, H, KVH, Dh, rd):
 
 
 @pytest.mark.parametrize("H,KVH,Dh,rd", [(32, 8, 128, 0), (8, 8, 128, 64), (6, 2, 64, 0), (5, 1, 80, 32), (4, 4, 256, 0),
-                                         (2, 2, 512, 0)])
+                                         (2, 2, 512, 0), (24, 4, 96, 0), (22, 6, 80, 0), (20, 8, 160, 0), (3, 1, 1024, 0)])
 def test_rope_half_split_layout_vs_oracle(hiplib, olib, H, KVH, Dh, rd):
-    """Pairs (i, i + rotary_dim / 2) instead of consecutive channels, out of place and in place (the two halves of a
-    pair are handled by two lanes of one wavefront)."""
+    """Pairs (i, i + rotary_dim / 2) instead of consecutive channels, out of place and in place. At head_dim 80, 96
+    and 160 a head row's lanes straddle two wavefronts (10, 12, 20 lanes a row) once a pass holds more than a few
+    rows, and at 1024 a row is two wavefronts wide: the in-place result must still equal the out-of-place one."""
     rng = np.random.default_rng(21)
     seqlens = np.array([1, 1, 37, 1, 130, 5])
     start = np.array([131071, 0, 0, 4095, 900, 65536])
@@ -65,21 +66,25 @@ def test_rope_half_split_layout_vs_oracle(hiplib, olib, H, KVH, Dh, rd):
     q = rng.standard_normal((T, H, Dh)).astype(np.float16)
     k = rng.standard_normal((T, KVH, Dh)).astype(np.float16)
     kw = dict(theta=500000.0, rotary_dim=rd, pair_layout=cabi.ROPE_PAIRS_HALF_SPLIT)
+    outs = []
     for inplace in (False, True):
         (qo, ko), (gq, gk) = run_both(hiplib, olib, q, k, seqlens, start, inplace=inplace, **kw)
         close(gq, qo, f"rotated_query in-place={inplace}")
         close(gk, ko, f"rotated_key in-place={inplace}")
         r = rd or Dh
         assert np.array_equal(gq[..., r:], q[..., r:]) and np.array_equal(gk[..., r:], k[..., r:])
+        outs.append((gq, gk))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1]), \
+        "in-place rotation differs from out-of-place"
     (io, _), _ = run_both(hiplib, olib, q, k, seqlens, start, theta=500000.0, rotary_dim=rd)
     assert not np.array_equal(io, qo)  # not the interleaved layout's result
 
 
 def test_rope_layout_is_validated(hiplib):
-    q = np.zeros((1, 1, 1024), np.float16)
+    q = np.zeros((1, 1, 4096), np.float16)
     a = harness.fill_rope_args(cabi.RopeArgs(), q, q, [1], [0], q, q, pair_layout=cabi.ROPE_PAIRS_HALF_SPLIT,
                                ptr=lambda t: C.c_void_p(0x1000))
-    assert hiplib.pplhip_rope_forward(C.byref(a), None) == cabi.RC_UNSUPPORTED  # head_dim > 512
+    assert hiplib.pplhip_rope_forward(C.byref(a), None) == cabi.RC_UNSUPPORTED  # head_dim > 2048
     a.head_dim, a.rotary_dim = 128, 24
     assert hiplib.pplhip_rope_forward(C.byref(a), None) == cabi.RC_INVALID_VALUE  # rotary_dim % 16
     a.rotary_dim, a.pair_layout = 0, 7
