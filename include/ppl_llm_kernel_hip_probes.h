@@ -46,6 +46,16 @@ pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_
  */
 pplhip_retcode pplhip_probe_quantizer(uint64_t* d_mismatches, void* stream);
 
+/*
+ * Verification aid, host only (no device call): the element offset of row (token, kv, head) of layer `layer` in the
+ * int8 slab and of the row's first scale in the scale tensor, formed by the library's own addressing (the struct every
+ * kernel folds its slab offsets with). A test compares it with arbitrary-precision arithmetic over strides up to
+ * 2^34, i.e. slabs far beyond 4 GiB: tok*stride_s + layer*stride_l + kv*stride_kv + head*stride_h, and that / 8.
+ */
+pplhip_retcode pplhip_probe_slab_row(int64_t stride_s, int64_t stride_l, int64_t stride_h, int64_t stride_kv, int32_t layer,
+                                     int64_t token, int32_t kv, int32_t head, int64_t* cache_element,
+                                     int64_t* scale_element);
+
 #ifdef __cplusplus
 }
 #endif

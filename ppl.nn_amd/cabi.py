@@ -141,6 +141,7 @@ PROBE_PROTOTYPES = {
     "pplhip_probe_mfma_f16": (_i32, [_p, _p, _i32, _i32, C.POINTER(C.c_double), _p]),
     "pplhip_probe_hbm_read": (_i32, [_p, C.c_uint64, _p, _i32, C.POINTER(C.c_uint64), _p]),
     "pplhip_probe_quantizer": (_i32, [_p, _p]),
+    "pplhip_probe_slab_row": (_i32, [_i64, _i64, _i64, _i64, _i32, _i64, _i32, _i32, C.POINTER(_i64), C.POINTER(_i64)]),
 }
 
 TABLES_OK, TABLES_BAD_SEQSTARTS, TABLES_BAD_KVSTARTS, TABLES_KVLEN_MISMATCH = 0, 1, 2, 3

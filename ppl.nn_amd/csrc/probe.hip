@@ -80,6 +80,18 @@ extern "C" const char* pplhip_probe_last_error(void) {
     return g_probe_error;
 }
 
+// The slab addressing every kernel uses (CacheAddr::row, compiled here for the host): element offset of a row of the
+// int8 slab and of its first scale. Host only, no device call.
+extern "C" pplhip_retcode pplhip_probe_slab_row(int64_t stride_s, int64_t stride_l, int64_t stride_h, int64_t stride_kv,
+                                                int32_t layer, int64_t token, int32_t kv, int32_t head,
+                                                int64_t* cache_element, int64_t* scale_element) {
+    if (!cache_element || !scale_element) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "probe: null result pointer");
+    const CacheAddr addr{stride_s, stride_l, stride_h, stride_kv, layer};
+    *cache_element = addr.row(token, kv, head);
+    *scale_element = *cache_element / kQuantGroup;
+    return PPLHIP_RC_SUCCESS;
+}
+
 extern "C" pplhip_retcode pplhip_probe_hbm_read(const void* d_src, uint64_t bytes, void* d_out, int32_t workgroups,
                                                 uint64_t* bytes_read, void* stream) {
     if (!d_src || !d_out || workgroups <= 0) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "probe: null buffer or no workgroups");

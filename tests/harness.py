@@ -152,15 +152,19 @@ def to_dev(a):
 
 
 def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layout=0, staging=None, lib=None,
-               mask=None):
+               mask=None, slab=None):
     """Same call through the C ABI on cuda:0. staging=0 clears plan.prefill_staging (the caller's way to keep a
     cache-prefill call on the kernel that reads the int8 slab itself). lib: another build of the kernel library than
-    the product one."""
+    the product one. slab: (cache, scale) device tensors the caller made (a slab too large to mirror on the host);
+    they are then inspected by the caller and not copied back."""
     import torch
     lib = lib or pkg.load_library()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cache_h, scale_h = new_slab(b, paged, layout)
-    cache, scale = to_dev(cache_h), to_dev(scale_h)
+    if slab is None:
+        cache_h, scale_h = new_slab(b, paged, layout)
+        cache, scale = to_dev(cache_h), to_dev(scale_h)
+    else:
+        cache, scale = slab
     d = {k: to_dev(v) for k, v in t.items()}
     tabs = dict(seqstarts=b.seqstarts, kvstarts=b.kvstarts,
                 cachestarts=np.ascontiguousarray(paged.table) if paged else b.cachestarts, start_pos=b.start_pos,
@@ -185,8 +189,10 @@ def run_device(b, t, cache_prefill=0, split_k=1, plan_out=None, paged=None, layo
     torch.cuda.synchronize()
     if plan_out is not None:
         plan_out.append(plan)
-    return dict(cache=cache.cpu().numpy(), scale=scale.cpu().view(torch.int16).numpy().view(np.float16),
-                output=out.cpu().view(torch.int16).numpy().view(np.float16))
+    output = out.cpu().view(torch.int16).numpy().view(np.float16)
+    if slab is not None:
+        return dict(output=output)
+    return dict(cache=cache.cpu().numpy(), scale=scale.cpu().view(torch.int16).numpy().view(np.float16), output=output)
 
 
 def mha_inputs(b, t):

@@ -277,3 +277,31 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(harness.pkg, "LIB_PATH", "/nonexistent/libppl_llm_kernel_hip.so")
     with pytest.raises(harness.pkg.LibraryMissing):
         harness.pkg.load_library()
+
+
+def test_slab_addressing_is_64_bit(probelib):
+    """The struct every kernel forms its slab offsets with, compiled for the host, against Python's integers: both
+    cache layouts at sizes whose offsets need up to 45 bits, and random strides up to 2^34 elements."""
+    import random
+    rng = random.Random(7)
+    row, srow = C.c_int64(), C.c_int64()
+    cases = []
+    for L, KVH, Dh, tokens in ((32, 8, 128, 70000), (80, 8, 128, 2 ** 22), (1, 8, 128, 2 ** 22 + 4099), (48, 40, 256, 2 ** 21)):
+        for st in (cabi.cache_strides_layout0(L, KVH, Dh), cabi.cache_strides_layout3(L, KVH, Dh, tokens)):
+            for _ in range(50):
+                cases.append((st["cache_stride_s"], st["cache_stride_l"], st["cache_stride_h"], st["cache_stride_kv"],
+                              rng.randrange(L), rng.randrange(tokens), rng.randrange(2), rng.randrange(KVH)))
+            cases.append((st["cache_stride_s"], st["cache_stride_l"], st["cache_stride_h"], st["cache_stride_kv"],
+                          L - 1, tokens - 1, 1, KVH - 1))
+    for _ in range(500):
+        cases.append(tuple(16 * rng.randrange(1, 2 ** 30) for _ in range(4)) +
+                     (rng.randrange(128), rng.randrange(2 ** 22), rng.randrange(2), rng.randrange(64)))
+    beyond = 0
+    for ss, sl, sh, skv, layer, tok, kv, head in cases:
+        want = tok * ss + layer * sl + kv * skv + head * sh
+        if want >= 2 ** 63:
+            continue
+        assert probelib.pplhip_probe_slab_row(ss, sl, sh, skv, layer, tok, kv, head, C.byref(row), C.byref(srow)) == 0
+        assert row.value == want and srow.value == want // 8, (ss, sl, sh, skv, layer, tok, kv, head)
+        beyond += want > 2 ** 32
+    assert beyond > 400
