@@ -37,6 +37,10 @@ def parse():
     ap.add_argument("--split-k", type=int, default=1)
     ap.add_argument("--no-other-configs", action="store_true", help="skip the cfg1 / cfg3 decode runs")
     ap.add_argument("--no-churn", action="store_true", help="skip the cfg4 continuous-batching churn run")
+    ap.add_argument("--churn-only", action="store_true",
+                    help="run only the cfg4 churn loop and print its entry (the command of the churn kernel trace)")
+    ap.add_argument("--no-engine", action="store_true", help="skip the run through the llm_hip host engine")
+    ap.add_argument("--no-layer-slab", action="store_true", help="skip the decode runs inside a 32-layer slab")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy (the reference point for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this same command)")
@@ -46,7 +50,10 @@ def parse():
 class DeviceBatch:
     """Device-resident tensors + argument block of one MHCA call; history is quantised by the library itself."""
 
-    def __init__(self, pkg, lib, b, seed, n_slabs, split_k=1, cache_prefill=0):
+    def __init__(self, pkg, lib, b, seed, n_slabs, split_k=1, cache_prefill=0, layout=0, layers=None):
+        """layers: instead of n_slabs separate one-layer slabs, ONE slab of b.num_layer layers whose listed layers all
+        hold the history; the steps rotate over them (distinct memory per step, like the slab rotation, inside a slab
+        of the size a whole model allocates). layout: cache_layout 0 (MaxT, L, 2, KVH, Dh) or 3 (L, 2, KVH, MaxT, Dh)."""
         import torch
         from ppl_nn_amd import cabi
         self.pkg, self.lib, self.b, self.cabi = pkg, lib, b, cabi
@@ -62,14 +69,23 @@ class DeviceBatch:
         self.seqstarts, self.kvstarts = i64(b.seqstarts), i64(b.kvstarts)
         self.cachestarts, self.start_pos = i64(b.cachestarts), i64(b.start_pos)
         histstarts, zeros = i64(b.histstarts), i64(np.zeros(max(b.batch, 1)))
-        shape = (b.max_tokens, b.num_layer, 2, b.num_kv_heads, b.head_dim)
+        if layout == 3:
+            shape = (b.num_layer, 2, b.num_kv_heads, b.max_tokens, b.head_dim)
+            st = cabi.cache_strides_layout3(b.num_layer, b.num_kv_heads, b.head_dim, b.max_tokens)
+        else:
+            shape = (b.max_tokens, b.num_layer, 2, b.num_kv_heads, b.head_dim)
+            st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
         self.slabs = []
         self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         ptr = lambda t: C.c_void_p(t.data_ptr())
-        st = cabi.cache_strides_layout0(b.num_layer, b.num_kv_heads, b.head_dim)
-        for s in range(n_slabs):
+        # (slab, layer) of every step of the rotation
+        places = [(0, l) for l in layers] if layers else [(s, b.layer_idx) for s in range(n_slabs)]
+        for s in range(1 if layers else n_slabs):
             cache = torch.zeros(shape, dtype=torch.int8, device="cuda")
             scale = torch.zeros(shape[:-1] + (b.head_dim // 8,), **f16)
+            self.slabs.append((cache, scale))
+        for slab, layer in places:
+            cache, scale = self.slabs[slab]
             if Hs:
                 hk = torch.randn((Hs, b.num_kv_heads, b.head_dim), generator=g, **f16)
                 hv = torch.randn((Hs, b.num_kv_heads, b.head_dim), generator=g, **f16)
@@ -77,23 +93,23 @@ class DeviceBatch:
                 w.d_current_key, w.d_current_value = ptr(hk), ptr(hv)
                 w.d_seqstarts, w.d_cachestarts, w.d_start_pos = ptr(histstarts), ptr(self.cachestarts), ptr(zeros)
                 w.batch, w.total_new_tokens = b.batch, Hs
-                w.layer_idx, w.num_layer, w.num_kv_heads, w.head_dim = b.layer_idx, b.num_layer, b.num_kv_heads, b.head_dim
+                w.layer_idx, w.num_layer, w.num_kv_heads, w.head_dim = layer, b.num_layer, b.num_kv_heads, b.head_dim
                 for kk, vv in st.items():
                     setattr(w, kk, vv)
                 w.d_cache, w.d_scale = ptr(cache), ptr(scale)
                 pkg.check(lib.pplhip_kv_quantize_write(C.byref(w), self.stream), "history write")
                 torch.cuda.synchronize()
                 del hk, hv
-            self.slabs.append((cache, scale))
         self.args = []
-        for cache, scale in self.slabs:
+        for slab, layer in places:
+            cache, scale = self.slabs[slab]
             a = cabi.MhcaArgs()
             a.d_query, a.d_current_key, a.d_current_value = ptr(self.q), ptr(self.k), ptr(self.v)
             a.d_seqstarts, a.d_kvstarts = ptr(self.seqstarts), ptr(self.kvstarts)
             a.d_cachestarts, a.d_start_pos = ptr(self.cachestarts), ptr(self.start_pos)
             a.is_causal, a.batch, a.decoding_batches = 1, b.batch, b.decoding_batches
             a.max_seqlen, a.max_kvlen = b.max_seqlen, b.max_kvlen
-            a.layer_idx, a.num_layer = b.layer_idx, b.num_layer
+            a.layer_idx, a.num_layer = layer, b.num_layer
             a.num_heads, a.num_kv_heads, a.head_dim = b.num_heads, b.num_kv_heads, b.head_dim
             a.cache_mode, a.page_size = 0, 128
             for kk, vv in st.items():
@@ -374,12 +390,126 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
     flops = sum(h["prefill_flops"] for h in timed)
     # check the on-device state against the host mirror once, after the timed region
     assert np.array_equal(slot_kv.cpu().numpy(), host[-1]["kv"] + host[-1]["nl"]), "slot state diverged"
+    # roofline of a step: the decode sequences' cache bytes at the HBM peak and the prompts' causal flops at the fp16
+    # matrix peak; the step cannot be shorter than the larger of the two and, where the two do not overlap, than their
+    # sum. Both fractions are given against the measured step (pack + attention + advance).
+    new_tokens = sum(h["S"] for h in timed)
+    write_bytes = new_tokens * 2 * KVH * Dh * (2 + 1.25)  # fp16 K/V rows read, int8 + scales written
+    qo_bytes = 2 * new_tokens * H * Dh * 2
+    step_bytes = (dec_bytes + write_bytes + qo_bytes) / steps
+    t_hbm_us = step_bytes / (HBM_PEAK_GBS * 1e9) * 1e6
+    t_mfma_us = flops / steps / (MFMA_FP16_PEAK_TFLOPS * 1e12) * 1e6
     return {"workload": "cfg4 churn: 256 slots x %d steps, H=KVH=40, Dh 128, retire p=0.02, prompts U[32,512], tables "
                         "rebuilt on the GPU every step" % steps,
             "ms_per_step": ms, "pack_tables_us": {"mean": pack_mean * 1e3, "median": pack_med * 1e3},
             "decode_tokens_per_s": dec_tokens / (ms * steps * 1e-3),
             "decode_kv_GB_per_step": dec_bytes / steps / 1e9, "prefill_GFLOP_per_step": flops / steps / 1e9,
-            "decode_GBps_if_step_were_decode_only": dec_bytes / (ms * steps * 1e-3) / 1e9}
+            "decode_GBps_if_step_were_decode_only": dec_bytes / (ms * steps * 1e-3) / 1e9,
+            "roofline": {"bound": "hbm", "algorithmic_bytes_per_step": step_bytes,
+                         "achieved": step_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": t_hbm_us / (ms * 1e3), "hbm_us_at_peak": t_hbm_us, "mfma_us_at_peak": t_mfma_us,
+                         "frac_if_bytes_and_flops_do_not_overlap": (t_hbm_us + t_mfma_us) / (ms * 1e3),
+                         "note": "bytes: int8 K/V + scales of the decode sequences, Q/O, fp16 K/V of the new tokens read "
+                                 "and their int8 rows written; flops: causal prompt attention; step = pack_tables + "
+                                 "one mixed MultiHeadCacheAttention call + advance_slots"}}
+
+
+def engine_run(pkg, lib, db):
+    """The same MultiHeadCacheAttention call through the llm_hip host engine: a one-node OPMX graph loaded by the ONNX
+    wire reader, run by Runtime::RunAsync on the caller's stream (the reference's wrapper reads three host scalars,
+    computes the strides, plans, takes a workspace from the device's buffer manager and frees it again:
+    multi_head_cache_attention_kernel.cc:116-132,218-228), beside the bare C-ABI call on the SAME slab. Also the node's
+    time as the runtime's own profiling reports it (tools/pplnn_llm.cc:892-990 prints these per kernel)."""
+    import torch
+    from ppl_nn_amd import onnx_writer as ow
+    eng = pkg.load_engine_library()
+    b = db.b
+    stream = torch.cuda.current_stream().cuda_stream
+    engine = eng.pplnn_hip_engine_create_on_stream(0, 1, C.c_void_p(stream))
+    builder = eng.pplnn_hip_builder_create()
+    model = ow.mhca_model(b.num_heads, b.num_kv_heads, b.head_dim, b.num_layer, b.layer_idx)
+
+    def ok(rc, what):
+        if rc:
+            raise RuntimeError("%s failed: %d: %s" % (what, rc, eng.pplnn_hip_last_error().decode()))
+    ok(eng.pplnn_hip_builder_load_model(builder, model, len(model)), "load_model")
+    ok(eng.pplnn_hip_builder_set_engine(builder, engine), "set_engine")
+    ok(eng.pplnn_hip_builder_preprocess(builder), "preprocess")
+    rt = eng.pplnn_hip_builder_create_runtime(builder)
+    if not rt:
+        raise RuntimeError("create_runtime failed: " + eng.pplnn_hip_last_error().decode())
+    cache, scale = db.slabs[0]
+    keep = []
+
+    def dims_of(shape):
+        return (C.c_int64 * len(shape))(*shape), len(shape)
+
+    def borrow(i, t):  # caller-owned device memory, like the KV slab
+        tensor = eng.pplnn_hip_runtime_input(rt, i)
+        d, n = dims_of(tuple(t.shape))
+        eng.pplnn_hip_tensor_reshape(tensor, d, n)
+        eng.pplnn_hip_tensor_set_buffer_ptr(tensor, t.data_ptr())
+
+    def host_scalar(i, v):
+        tensor = eng.pplnn_hip_runtime_input(rt, i)
+        eng.pplnn_hip_tensor_use_host_device(tensor)
+        eng.pplnn_hip_tensor_reshape(tensor, None, 0)
+        a = np.array([v], np.int64)
+        keep.append(a)
+        ok(eng.pplnn_hip_tensor_copy_from_host(tensor, a.ctypes.data), "scalar")
+    for i, t in enumerate((db.q, db.k, db.v, db.seqstarts, db.kvstarts, db.cachestarts, db.start_pos)):
+        borrow(i, t)
+    for i, v in enumerate((b.decoding_batches, b.max_seqlen, b.max_kvlen)):
+        host_scalar(7 + i, v)
+    borrow(10, cache)
+    borrow(11, scale)
+
+    def via_engine(i):
+        rc = eng.pplnn_hip_runtime_run_async(rt)
+        if rc:
+            ok(rc, "RunAsync")
+
+    a0, plan = db.args[0], db.plan
+
+    def via_cabi(i):
+        rc = lib.pplhip_mhca_forward(C.byref(a0), C.byref(plan), db.ws_ptr, db.stream)
+        if rc:
+            pkg.check(rc, "mhca_forward")
+    res = {}
+    for rnd in range(2):  # interleaved, the second round is reported
+        e_mean, e_med, e_n = timed_robust(via_engine)
+        c_mean, c_med, c_n = timed_robust(via_cabi)
+    # wall clock of a queue of calls as well: the host side of the engine call must keep ahead of the GPU
+    def wall(fn, n=300):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            fn(i)
+        host = (time.perf_counter() - t0) / n
+        torch.cuda.synchronize()
+        return host * 1e6, (time.perf_counter() - t0) / n * 1e6
+    e_host, e_wall = wall(via_engine)
+    c_host, c_wall = wall(via_cabi)
+    # the runtime's own per-kernel profile (each profiled run waits for its kernel's end event)
+    ok(eng.pplnn_hip_runtime_set_profiling(rt, 1), "profiling on")
+    runs = 50
+    for _ in range(runs):
+        ok(eng.pplnn_hip_runtime_run(rt), "Run")
+    micros, counts = (C.c_uint64 * 4)(), (C.c_uint32 * 4)()
+    nk = eng.pplnn_hip_runtime_profiling(rt, micros, counts, 4)
+    ok(eng.pplnn_hip_runtime_set_profiling(rt, 0), "profiling off")
+    torch.cuda.synchronize()
+    eng.pplnn_hip_runtime_destroy(rt)
+    eng.pplnn_hip_builder_destroy(builder)
+    eng.pplnn_hip_engine_destroy(engine)
+    return {"workload": "decode part of the workload, one slab (no rotation), MultiHeadCacheAttention as a one-node graph",
+            "engine_run_async_us": e_med * 1e3, "cabi_call_us": c_med * 1e3, "engine_minus_cabi_us": (e_med - c_med) * 1e3,
+            "calls_timed": e_n, "host_us_per_engine_call": e_host, "host_us_per_cabi_call": c_host,
+            "wall_us_per_engine_call": e_wall, "wall_us_per_cabi_call": c_wall,
+            "profiling": {"kernels": int(nk), "exec_count": int(counts[0]),
+                          "avg_us_per_run": micros[0] / max(int(counts[0]), 1),
+                          "note": "GetProfilingStatistics of the node: HIP events around the op on an idle stream, "
+                                  "so the host time between the first event and the first launch is inside"}}
 
 
 def rope_cache_write(pkg, lib, b):
@@ -463,6 +593,13 @@ def main():
         dec_b = workloads.cfg3_long_context()
         wname = "cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]"
 
+    if args.churn_only:
+        print(json.dumps({"churn_cfg4": churn_cfg4(pkg, lib)}))
+        return
+    # the two roofline probes run first: what this box sustains, measured before anything else has heated the chip
+    stream_gbs = hbm_sustained(probes)
+    sustained = mfma_sustained(probes) if pre_b is not None else None
+
     dec = DeviceBatch(pkg, lib, dec_b, seed=1, n_slabs=N_SLABS, split_k=args.split_k)
     wall_ms, ev_ms = timed(dec, args.steps, args.warmup)
     _, dec_med_ms, dec_n = timed_robust(dec.step)
@@ -492,7 +629,6 @@ def main():
                      "median_ms_per_launch_long_run": dec_med_ms, "long_run_calls": dec_n,
                      "traffic_source": "recorded rocprofv3 --pmc summary under profiles/ (not re-measured in this run)"},
     }
-    stream_gbs = hbm_sustained(probes)
     result["hbm_read_sustained_GBs"] = dict(
         stream_gbs, note="plain streaming read of 2 GiB measured in this run; the published peak is %.0f" % HBM_PEAK_GBS)
     result["roofline"]["frac_of_sustained_hbm_read"] = gbs / max(stream_gbs.values())
@@ -500,7 +636,6 @@ def main():
     def frac(tflops):
         return tflops / MFMA_FP16_PEAK_TFLOPS
 
-    sustained = mfma_sustained(probes) if pre_b is not None else None
     if sustained:
         result["mfma_f16_sustained_tflops"] = dict(
             sustained, note="bare v_mfma_f32_32x32x16_f16 loop on all CUs, measured in this run; the published peak is "
@@ -527,10 +662,31 @@ def main():
         result["fused_mixed_call_ms_mean"] = mix_mean
         del mixed
         result["rope_cache_write"] = rope_cache_write(pkg, lib, full)
+    if not args.no_engine:
+        result["engine_run"] = engine_run(pkg, lib, dec)
     if args.workload == "cfg2" and not args.no_churn:
         del dec.slabs[1:], dec.args[1:]
         torch.cuda.empty_cache()
         result["churn_cfg4"] = churn_cfg4(pkg, lib)
+    if args.workload == "cfg2" and not args.no_layer_slab:
+        # the same decode call inside the slab a whole model allocates (tools/benchmark_llama/text_generator.cc:200-211:
+        # one cache tensor for all layers): 32 layers, the steps rotate over layers 28..31 so that every step reads
+        # memory the previous ones did not (the role the rotated slabs play above)
+        ls = {}
+        for layout, name in ((0, "cache_layout_0 (MaxT, 32, 2, KVH, Dh): 64 KiB between a head group's tokens"),
+                             (3, "cache_layout_3 (32, 2, KVH, MaxT, Dh): a head's tokens 128 bytes apart")):
+            lb = workloads.Batch(32, 8, 128, dec_b.seqlens, dec_b.start_pos, dec_b.decoding_batches, num_layer=32,
+                                 layer_idx=31, name="cfg2 decode part in a 32-layer slab")
+            ldb = DeviceBatch(pkg, lib, lb, seed=1, n_slabs=1, split_k=args.split_k, layout=layout, layers=[28, 29, 30, 31])
+            l_mean, l_med, l_n = timed_robust(ldb.step)
+            l_gbs = lb.decode_bytes() / (l_med * 1e-3) / 1e9
+            ls["cache_layout_%d" % layout] = {"layout": name, "ms_per_step": l_med, "ms_per_step_mean": l_mean,
+                                              "calls_timed": l_n, "achieved_GBs": l_gbs,
+                                              "frac_of_hbm_peak": l_gbs / HBM_PEAK_GBS, "layers_rotated": [28, 29, 30, 31],
+                                              "slab_GB": (ldb.slabs[0][0].numel() + 2 * ldb.slabs[0][1].numel()) / 1e9}
+            del ldb
+            torch.cuda.empty_cache()
+        result["decode_in_32_layer_slab"] = ls
     if args.workload == "cfg2" and not args.no_other_configs:
         # the other decode configurations at their full sizes
         others = {}
