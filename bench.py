@@ -41,6 +41,13 @@ def parse():
                     help="run only the cfg4 churn loop and print its entry (the command of the churn kernel trace)")
     ap.add_argument("--no-engine", action="store_true", help="skip the run through the llm_hip host engine")
     ap.add_argument("--no-layer-slab", action="store_true", help="skip the decode runs inside a 32-layer slab")
+    ap.add_argument("--sections", default="all",
+                    help="comma-separated subset of the secondary measurements to run: probes, prefill (cfg2 prefill "
+                         "part, fused mixed call, rope + cache write), engine, churn, layer_slab, other (cfg1, cfg3, "
+                         "8k prompts, chunked prefill, general kernels), cpu; the headline decode loop always runs")
+    ap.add_argument("--quick", action="store_true",
+                    help="a dozen calls per secondary figure instead of >= 100 calls and >= 200 ms: for counter runs "
+                         "(rocprofv3 --pmc serialises dispatches), not for reported timings")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy (the reference point for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this same command)")
@@ -149,11 +156,16 @@ def timed(db, steps, warmup):
     return wall, e0.elapsed_time(e1) / steps
 
 
+QUICK = False  # --quick: a dozen calls per figure (counter collection), set by main()
+
+
 def timed_robust(step, min_warmup=20, min_iters=100, min_ms=200.0, batches=10):
     """For the secondary figures: at least `min_warmup` untimed calls, then at least `min_iters` calls and `min_ms` of
     device time whatever --steps says, timed with events on the launch stream in `batches` equal batches.
     Returns (mean ms per call, median over the batches of ms per call, calls timed)."""
     import torch
+    if QUICK:
+        min_warmup, min_iters, min_ms, batches = 2, 10, 0.0, 2
     for i in range(min_warmup):
         step(i)
     torch.cuda.synchronize()
@@ -296,8 +308,8 @@ def copy_calibration():
 
 def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
     """Continuous-batching churn (Llama-2-13B shape, H = KVH = 40): 256 slots, every step the tables are rebuilt on
-    the GPU by pplhip_pack_tables from the slot state, one mixed MultiHeadCacheAttention call runs on them, and
-    pplhip_advance_slots grows the slots. The host only supplies the sizes its scheduler knows anyway (batch,
+    the GPU by pplhip_pack_tables from the slot state (the same launch grows the slots for the next step), and one
+    mixed MultiHeadCacheAttention call runs on them. The host only supplies the sizes its scheduler knows anyway (batch,
     decoding_batches, maxima), precomputed for the seeded schedule; no table is uploaded and nothing is read back."""
     import torch
     from ppl_nn_amd import cabi, workloads
@@ -342,7 +354,7 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
     for i, h in enumerate(host):
         pa = cabi.PackArgs()
         pa.d_slot_kvlen, pa.d_slot_newlen, pa.d_slot_cachestart = ptr(slot_kv), ptr(slot_nl[i]), ptr(slot_cs)
-        pa.num_slots = n
+        pa.num_slots, pa.advance_slots = n, 1  # the slot state moves on inside the pack launch
         pa.d_seqstarts, pa.d_kvstarts, pa.d_cachestarts = ptr(seqstarts), ptr(kvstarts), ptr(cachestarts)
         pa.d_start_pos, pa.d_batch_slots, pa.d_header = ptr(start_pos), ptr(batch_slots), ptr(header)
         a = cabi.MhcaArgs()
@@ -368,7 +380,6 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
         slot_kv.copy_(slot_kv_reset[i])  # device-to-device: applies the scheduler's retirements
         rc = lib.pplhip_pack_tables(C.byref(pa), stream)
         rc = rc or lib.pplhip_mhca_forward(C.byref(a), C.byref(plan), ptr(ws), stream)
-        rc = rc or lib.pplhip_advance_slots(ptr(slot_kv), ptr(slot_nl[i]), n, stream)
         if rc:
             pkg.check(rc, "churn step")
 
@@ -383,13 +394,15 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
     # the table rebuild alone (same slot state every call; one workgroup, latency-bound)
-    pack_mean, pack_med, _ = timed_robust(lambda i: lib.pplhip_pack_tables(C.byref(calls[-1][0]), stream), min_ms=50.0)
+    pack_only = calls[-1][0]
+    pack_only.advance_slots = 0  # (timed on a fixed slot state, after the loop's own check below has used it)
     timed = host[warm_steps:]
     dec_tokens = sum(h["nd"] for h in timed)
     dec_bytes = sum(h["dec_kv"] for h in timed) * 2.5 * KVH * Dh
     flops = sum(h["prefill_flops"] for h in timed)
     # check the on-device state against the host mirror once, after the timed region
     assert np.array_equal(slot_kv.cpu().numpy(), host[-1]["kv"] + host[-1]["nl"]), "slot state diverged"
+    pack_mean, pack_med, _ = timed_robust(lambda i: lib.pplhip_pack_tables(C.byref(pack_only), stream), min_ms=50.0)
     # roofline of a step: the decode sequences' cache bytes at the HBM peak and the prompts' causal flops at the fp16
     # matrix peak; the step cannot be shorter than the larger of the two and, where the two do not overlap, than their
     # sum. Both fractions are given against the measured step (pack + attention + advance).
@@ -410,8 +423,8 @@ def churn_cfg4(pkg, lib, steps=100, warm_steps=5):
                          "frac": t_hbm_us / (ms * 1e3), "hbm_us_at_peak": t_hbm_us, "mfma_us_at_peak": t_mfma_us,
                          "frac_if_bytes_and_flops_do_not_overlap": (t_hbm_us + t_mfma_us) / (ms * 1e3),
                          "note": "bytes: int8 K/V + scales of the decode sequences, Q/O, fp16 K/V of the new tokens read "
-                                 "and their int8 rows written; flops: causal prompt attention; step = pack_tables + "
-                                 "one mixed MultiHeadCacheAttention call + advance_slots"}}
+                                 "and their int8 rows written; flops: causal prompt attention; step = pack_tables (which also advances the "
+                                 "slot state) + one mixed MultiHeadCacheAttention call"}}
 
 
 def engine_run(pkg, lib, db):
@@ -593,12 +606,18 @@ def main():
         dec_b = workloads.cfg3_long_context()
         wname = "cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]"
 
+    global QUICK
+    QUICK = args.quick
+    sections = set(x.strip() for x in args.sections.split(","))
+
+    def want(name):
+        return "all" in sections or name in sections
     if args.churn_only:
-        print(json.dumps({"churn_cfg4": churn_cfg4(pkg, lib)}))
+        print(json.dumps({"churn_cfg4": churn_cfg4(pkg, lib, steps=20 if QUICK else 100)}))
         return
     # the two roofline probes run first: what this box sustains, measured before anything else has heated the chip
-    stream_gbs = hbm_sustained(probes)
-    sustained = mfma_sustained(probes) if pre_b is not None else None
+    stream_gbs = hbm_sustained(probes) if want("probes") else None
+    sustained = mfma_sustained(probes) if pre_b is not None and want("probes") else None
 
     dec = DeviceBatch(pkg, lib, dec_b, seed=1, n_slabs=N_SLABS, split_k=args.split_k)
     wall_ms, ev_ms = timed(dec, args.steps, args.warmup)
@@ -629,9 +648,10 @@ def main():
                      "median_ms_per_launch_long_run": dec_med_ms, "long_run_calls": dec_n,
                      "traffic_source": "recorded rocprofv3 --pmc summary under profiles/ (not re-measured in this run)"},
     }
-    result["hbm_read_sustained_GBs"] = dict(
-        stream_gbs, note="plain streaming read of 2 GiB measured in this run; the published peak is %.0f" % HBM_PEAK_GBS)
-    result["roofline"]["frac_of_sustained_hbm_read"] = gbs / max(stream_gbs.values())
+    if stream_gbs:
+        result["hbm_read_sustained_GBs"] = dict(
+            stream_gbs, note="plain streaming read of 2 GiB measured in this run; the published peak is %.0f" % HBM_PEAK_GBS)
+        result["roofline"]["frac_of_sustained_hbm_read"] = gbs / max(stream_gbs.values())
 
     def frac(tflops):
         return tflops / MFMA_FP16_PEAK_TFLOPS
@@ -652,7 +672,7 @@ def main():
         e.update(extra or {})
         return e
 
-    if pre_b is not None:
+    if pre_b is not None and want("prefill"):
         pre = DeviceBatch(pkg, lib, pre_b, seed=2, n_slabs=1)
         result["prefill"] = prefill_entry(pre, pre_b, {"prefill_seqs": pre_b.batch, "prefill_tokens": pre_b.total_new_tokens})
         del pre
@@ -662,13 +682,13 @@ def main():
         result["fused_mixed_call_ms_mean"] = mix_mean
         del mixed
         result["rope_cache_write"] = rope_cache_write(pkg, lib, full)
-    if not args.no_engine:
+    if not args.no_engine and want("engine"):
         result["engine_run"] = engine_run(pkg, lib, dec)
-    if args.workload == "cfg2" and not args.no_churn:
+    if args.workload == "cfg2" and not args.no_churn and want("churn"):
         del dec.slabs[1:], dec.args[1:]
         torch.cuda.empty_cache()
         result["churn_cfg4"] = churn_cfg4(pkg, lib)
-    if args.workload == "cfg2" and not args.no_layer_slab:
+    if args.workload == "cfg2" and not args.no_layer_slab and want("layer_slab"):
         # the same decode call inside the slab a whole model allocates (tools/benchmark_llama/text_generator.cc:200-211:
         # one cache tensor for all layers): 32 layers, the steps rotate over layers 28..31 so that every step reads
         # memory the previous ones did not (the role the rotated slabs play above)
@@ -687,7 +707,7 @@ def main():
             del ldb
             torch.cuda.empty_cache()
         result["decode_in_32_layer_slab"] = ls
-    if args.workload == "cfg2" and not args.no_other_configs:
+    if args.workload == "cfg2" and not args.no_other_configs and want("other"):
         # the other decode configurations at their full sizes
         others = {}
         for name, ob in (("cfg1 Llama-2-7B pure decode (H32/KVH32/Dh128): 64 seqs kv~U[128,2048]",
@@ -741,7 +761,7 @@ def main():
         result["general_kernel"] = gen
     if args.copy_calibration:
         copy_calibration()
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and want("cpu"):
         threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
         result["cpu_baseline"] = cpu_baseline(dec, threads)
     print(json.dumps(result))

@@ -369,7 +369,10 @@ typedef struct pplhip_pack_args {
     const int64_t* d_slot_newlen;
     const int64_t* d_slot_cachestart;
     int32_t num_slots;
-    int32_t reserved;
+    int32_t advance_slots; /* 0: the slot state is only read. 1: once the tables are built the same launch also does what
+                              pplhip_advance_slots does, slot_kvlen[i] += slot_newlen[i] for every active slot (the
+                              attention call that follows reads the packed tables, not the slot state, so the state can
+                              move on right away and a step needs one launch less); d_slot_kvlen is then written */
     int64_t* d_seqstarts;
     int64_t* d_kvstarts;
     int64_t* d_cachestarts;
@@ -380,7 +383,8 @@ typedef struct pplhip_pack_args {
 
 pplhip_retcode pplhip_pack_tables(const pplhip_pack_args* args, void* stream);
 
-/* After a step: slot_kvlen += slot_newlen for every active slot (so the next pack sees the grown sequences). */
+/* After a step: slot_kvlen += slot_newlen for every active slot (so the next pack sees the grown sequences). A launch
+ * of its own; pplhip_pack_args.advance_slots does the same inside the pack launch. */
 pplhip_retcode pplhip_advance_slots(int64_t* d_slot_kvlen, const int64_t* d_slot_newlen, int32_t num_slots,
                                     void* stream);
 

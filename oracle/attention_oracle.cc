@@ -439,6 +439,11 @@ int oracle_pack_tables(const pplhip_pack_args* a) {
     a->d_header[3] = max_kv;
     a->d_header[4] = a->d_seqstarts[b];
     a->d_header[5] = a->d_kvstarts[b];
+    if (a->advance_slots) { // the slot state moves on in the same call (generation_state.cc:127-140: kv lengths grow)
+        int64_t* kv = const_cast<int64_t*>(a->d_slot_kvlen);
+        for (int i = 0; i < n; ++i)
+            if (a->d_slot_newlen[i] > 0) kv[i] += a->d_slot_newlen[i];
+    }
     return PPLHIP_RC_SUCCESS;
 }
 

@@ -109,7 +109,7 @@ ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_DYNAMIC = 0, 1, 2
 class PackArgs(C.Structure):
     _fields_ = [
         ("d_slot_kvlen", _p), ("d_slot_newlen", _p), ("d_slot_cachestart", _p),
-        ("num_slots", _i32), ("reserved", _i32),
+        ("num_slots", _i32), ("advance_slots", _i32),
         ("d_seqstarts", _p), ("d_kvstarts", _p), ("d_cachestarts", _p), ("d_start_pos", _p),
         ("d_batch_slots", _p), ("d_header", _p),
     ]

@@ -10,7 +10,7 @@ namespace pplhip {
 constexpr int kMaxSlots = 1024;
 
 struct PackParams {
-    const int64_t* slot_kvlen;
+    int64_t* slot_kvlen; // written only when `advance` is set
     const int64_t* slot_newlen;
     const int64_t* slot_cachestart;
     int64_t* seqstarts;
@@ -20,6 +20,7 @@ struct PackParams {
     int64_t* batch_slots;
     int64_t* header;
     int32_t n;
+    int32_t advance; // slot_kvlen += slot_newlen once the tables are built
 };
 
 // Inclusive scan of one int64 per thread across the workgroup (Hillis-Steele in LDS, ping-pong buffers).
@@ -107,6 +108,8 @@ __global__ __launch_bounds__(kMaxSlots) void pack_tables_kernel(const PackParams
         p.seqstarts[0] = 0;
         p.kvstarts[0] = 0;
     }
+    // (every thread read its own slot's state at the top and nothing else reads it: the state may move on in place)
+    if (p.advance && in && nl > 0) p.slot_kvlen[tid] = kl + nl;
     if (tid == nt - 1) {
         p.header[0] = batch;
         p.header[1] = nd;
@@ -120,8 +123,9 @@ __global__ __launch_bounds__(kMaxSlots) void pack_tables_kernel(const PackParams
 pplhip_retcode launch_pack_tables(const pplhip_pack_args* a, hipStream_t stream) {
     if (a->num_slots <= 0 || a->num_slots > kMaxSlots)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "pack_tables: num_slots %d outside [1, %d]", a->num_slots, kMaxSlots);
-    PackParams p{a->d_slot_kvlen, a->d_slot_newlen, a->d_slot_cachestart, a->d_seqstarts, a->d_kvstarts,
-                 a->d_cachestarts, a->d_start_pos, a->d_batch_slots, a->d_header, a->num_slots};
+    PackParams p{const_cast<int64_t*>(a->d_slot_kvlen), a->d_slot_newlen, a->d_slot_cachestart, a->d_seqstarts,
+                 a->d_kvstarts, a->d_cachestarts, a->d_start_pos, a->d_batch_slots, a->d_header, a->num_slots,
+                 a->advance_slots != 0};
     int threads = 64;
     while (threads < a->num_slots) threads <<= 1;
     hipLaunchKernelGGL(pack_tables_kernel, dim3(1), dim3(threads), 0, stream, p);

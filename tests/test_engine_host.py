@@ -124,7 +124,10 @@ def test_engine_configure_like_the_reference(eng):
     # 1006 = ENGINE_CONF_ROPE_PAIR_LAYOUT (this engine's own): 0 consecutive channels, 1 half-split
     assert eng.pplnn_hip_engine_configure_u32(e, 1006, 1) == 0 and eng.pplnn_hip_engine_configure_u32(e, 1006, 0) == 0
     assert eng.pplnn_hip_engine_configure_u32(e, 1006, 2) == cabi.RC_INVALID_VALUE
-    assert eng.pplnn_hip_engine_configure_u32(e, 1007, 0) == cabi.RC_INVALID_VALUE
+    # 1007 / 1008: this engine's debugging aids (table check in front of attention, wait after every op)
+    for opt in (1007, 1008):
+        assert eng.pplnn_hip_engine_configure_u32(e, opt, 1) == 0 and eng.pplnn_hip_engine_configure_u32(e, opt, 0) == 0
+    assert eng.pplnn_hip_engine_configure_u32(e, 1009, 0) == cabi.RC_INVALID_VALUE
     eng.pplnn_hip_engine_destroy(e)
     assert not eng.pplnn_hip_engine_create(0, 99)  # unknown mm_policy: factories return nullptr on failure
 

@@ -252,6 +252,42 @@ def test_pack_tables_random_and_churn(hiplib, olib):
         assert np.array_equal(dkv.cpu().numpy(), kv + nl)
 
 
+def test_pack_tables_can_advance_the_slots_in_the_same_launch(hiplib, olib):
+    """pplhip_pack_args.advance_slots: the tables are those of the plain call, and slot_kvlen has moved on by
+    slot_newlen for every active slot when the launch is done (what pplhip_advance_slots does as a second launch).
+    Against the oracle's pack with the same flag, over the churn schedule with the state kept on the device."""
+    import torch
+    import test_oracle_pack as top
+    sch = workloads.ChurnSchedule(seed=2)
+    n = sch.num_slots
+    out = {k: torch.full((m,), -7, dtype=torch.int64, device="cuda") for k, m in
+           dict(seqstarts=n + 1, kvstarts=n + 1, cachestarts=n, start_pos=n, batch_slots=n, header=6).items()}
+    dcs = harness.to_dev(sch.cachestart)
+    for step in range(30):
+        kv, nl = sch.next_step()
+        dkv, dnl = harness.to_dev(kv), harness.to_dev(nl)  # (retirements reset slots: the scheduler's upload)
+        a = cabi.PackArgs()
+        a.d_slot_kvlen, a.d_slot_newlen, a.d_slot_cachestart = dkv.data_ptr(), dnl.data_ptr(), dcs.data_ptr()
+        a.num_slots, a.advance_slots = n, 1
+        a.d_seqstarts, a.d_kvstarts = out["seqstarts"].data_ptr(), out["kvstarts"].data_ptr()
+        a.d_cachestarts, a.d_start_pos = out["cachestarts"].data_ptr(), out["start_pos"].data_ptr()
+        a.d_batch_slots, a.d_header = out["batch_slots"].data_ptr(), out["header"].data_ptr()
+        harness.pkg.check(hiplib.pplhip_pack_tables(C.byref(a), None), "pack_tables")
+        torch.cuda.synchronize()
+        want = top.run_pack(olib.oracle_pack_tables, kv, nl, sch.cachestart)
+        for k in want:
+            assert np.array_equal(out[k].cpu().numpy(), want[k]), (step, k)
+        assert np.array_equal(dkv.cpu().numpy(), kv + nl), step
+    # the oracle with the flag: same tables, state advanced
+    kv, nl = sch.next_step()
+    kv2 = kv.copy()
+    want = top.run_pack(olib.oracle_pack_tables, kv, nl, sch.cachestart)
+    got = top.run_pack(olib.oracle_pack_tables, kv2, nl, sch.cachestart, advance=1)
+    for k in want:
+        assert np.array_equal(got[k], want[k])
+    assert np.array_equal(kv2, kv + nl)
+
+
 @pytest.mark.parametrize("causal", [1, 0])
 def test_multi_head_attention_vs_oracle(causal):
     # decode rows (1 query, long history), chunked rows (kvlen > seqlen), fresh prompts; tiles that straddle 64/128

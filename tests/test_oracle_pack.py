@@ -19,14 +19,14 @@ def brute_force(kvlen, newlen, cachestart):
                 cachestarts=[int(cachestart[i]) for i in order], start_pos=[int(kvlen[i]) for i in order])
 
 
-def run_pack(fn, kvlen, newlen, cachestart):
+def run_pack(fn, kvlen, newlen, cachestart, advance=0):
     n = len(kvlen)
     out = dict(seqstarts=np.full(n + 1, -7, np.int64), kvstarts=np.full(n + 1, -7, np.int64),
                cachestarts=np.full(n, -7, np.int64), start_pos=np.full(n, -7, np.int64),
                batch_slots=np.full(n, -7, np.int64), header=np.full(6, -7, np.int64))
     a = cabi.PackArgs()
     a.d_slot_kvlen, a.d_slot_newlen, a.d_slot_cachestart = kvlen.ctypes.data, newlen.ctypes.data, cachestart.ctypes.data
-    a.num_slots = n
+    a.num_slots, a.advance_slots = n, advance
     a.d_seqstarts, a.d_kvstarts = out["seqstarts"].ctypes.data, out["kvstarts"].ctypes.data
     a.d_cachestarts, a.d_start_pos = out["cachestarts"].ctypes.data, out["start_pos"].ctypes.data
     a.d_batch_slots, a.d_header = out["batch_slots"].ctypes.data, out["header"].ctypes.data
@@ -80,3 +80,19 @@ def test_churn_schedule_invariants():
         assert (nl[kv > 0] == 1).all() and (nl[kv == 0] >= 8).all()
         assert (kv + nl <= 256).all()
         prev_after = kv + nl
+
+
+def test_pack_with_advance_moves_the_slot_state(olib):
+    """advance_slots = 1: the same tables, and afterwards slot_kvlen += slot_newlen for every active slot
+    (generation_state.cc:127-140 grows the kv lengths between steps)."""
+    rng = np.random.default_rng(8)
+    for n in (1, 5, 64, 300):
+        kvlen = (rng.integers(0, 50, n) * (rng.random(n) < 0.7)).astype(np.int64)
+        newlen = np.where(rng.random(n) < 0.2, 0, np.where(kvlen > 0, 1, rng.integers(1, 40, n))).astype(np.int64)
+        cs = (np.arange(n) * 1024).astype(np.int64)
+        plain = run_pack(olib.oracle_pack_tables, kvlen.copy(), newlen, cs)
+        state = kvlen.copy()
+        moved = run_pack(olib.oracle_pack_tables, state, newlen, cs, advance=1)
+        for k in plain:
+            assert np.array_equal(plain[k], moved[k]), k
+        assert np.array_equal(state, kvlen + np.maximum(newlen, 0))
