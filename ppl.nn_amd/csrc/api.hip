@@ -229,13 +229,11 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
         // perfectly filled round) measures best; the knob moves it to half or twice that
         const int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
         // ranges x groups workgroups must not spill over the slots (a second, nearly empty round doubles the time:
-        // 40 kv heads = 10 groups took 56 ranges = 560 workgroups on 512 slots), so everything rounds DOWN to the
-        // multiple of 8 the XCD-aware numbering needs
+        // 40 kv heads = 10 groups took 56 ranges = 560 workgroups on 512 slots), so the quotient rounds DOWN
         int64_t ranges = slots * half_slots / 2 / groups;
         // never more ranges than 128-token pieces of the worst case (every sequence max_kvlen long)
         const int64_t cap = (nd * a->max_kvlen + 127) / 128;
         if (ranges > cap) ranges = cap;
-        ranges = ranges / 8 * 8;
         if (ranges < 8) ranges = 8;
         if (ranges > 0x3fffffff) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many ranges");
         plan->decode_num_ranges = (int32_t)ranges;
@@ -274,7 +272,7 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
             PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
     } else {
         const uint64_t decode_bytes = decode_workspace_bytes(a, plan->decode_num_ranges);
-        bool ok = plan->decode_num_ranges >= 0 && !(plan->decode_num_ranges & 7) && decode_bytes <= plan->workspace_bytes;
+        bool ok = plan->decode_num_ranges >= 0 && decode_bytes <= plan->workspace_bytes;
         if (ok && plan->prefill_staging) { // fp16 staging rows of a cache-prefill call, behind the decode partials
             const uint64_t first = (uint64_t)(uint32_t)plan->prefill_staging_offset_256 * 256;
             const uint64_t rows = (uint64_t)prefill_staging_tokens(a) * 2 * a->num_kv_heads * a->head_dim * sizeof(uint16_t);

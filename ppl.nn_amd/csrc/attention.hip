@@ -55,8 +55,8 @@ pplhip_retcode launch_decode_and_prefill(const pplhip_mhca_args* a, const pplhip
                                            reinterpret_cast<const void*>(mixed_attention_kernel<false, true>),
                                            reinterpret_cast<const void*>(mixed_attention_kernel<true, true>)});
     if (rc != PPLHIP_RC_SUCCESS) return rc;
-    // the decode workgroups come first: they are dispatched at once, and their numbering (workgroup i on XCD i % 8)
-    // holds; their count is a multiple of 8, so the prompts' numbering holds as well
+    // the decode workgroups come first: they are dispatched at once. The prompts' numbering relies on workgroups that
+    // are 8 apart sharing an XCD, which holds behind any number of decode workgroups.
     const dim3 grid((unsigned)(dblocks + pblocks)), block(256);
     const uint32_t nd_blocks = (uint32_t)dblocks;
     const bool direct = dp.hpb == kDecodeWaves;

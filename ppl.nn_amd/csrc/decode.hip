@@ -19,8 +19,7 @@
 // one after the other. Every workgroup therefore streams the same number of bytes, whatever the raggedness of the batch,
 // and there is no tail of long sequences. Inside a workgroup each wave owns one kv head (the workgroup then reads
 // hpb * 128 contiguous bytes of every token) or, with fewer than 4 kv heads, a share of the segment's tokens.
-// Workgroups are numbered so that the head groups of one range start on the same XCD (workgroup i runs on XCD i % 8):
-// their neighbouring rows then meet in one L2 and reach the same DRAM pages together.
+// The head groups of one range are neighbouring workgroups: they start together and reach the same DRAM pages together.
 //
 // LDS layout of one 32-token stage of one wave (10 KiB): K rows [32][128 B], V rows [32][128 B], K scales [32][32 B],
 // V scales [32][32 B]. Inside a K/V row the eight 16 B pieces are XOR-swizzled with (row & 7) by choosing which
@@ -78,7 +77,7 @@ struct DecodeParams {
     CacheAddr addr;
     int32_t nd; // decode sequences (the first nd entries of the tables)
     int32_t num_heads, kv_heads, rep; // rep = num_heads / kv_heads (<= 16)
-    int32_t num_ranges; // S, a multiple of 8
+    int32_t num_ranges; // S
     int32_t hpb; // kv heads per workgroup: min(kv_heads, 4), a power of two dividing kv_heads
     int32_t merge_by_boundary; // merge kernel: blockIdx.y counts range boundaries instead of sequences
     float score_scale; // log2(e) / sqrt(Dh)
@@ -444,10 +443,11 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
     const int groups = p.kv_heads / p.hpb;
-    const int xcd = block & 7;
-    const uint32_t j = block >> 3;
-    const int hg = (int)(j % (uint32_t)groups);
-    const int64_t s_idx = (int64_t)(j / (uint32_t)groups) * 8 + xcd; // range index
+    // Workgroup numbering: the head groups of a range are neighbours. (Numbering them so that they share an XCD, with
+    // the range count rounded down to a multiple of 8 for it, measured the same on every shape -- the head groups read
+    // different bytes of a row, there is nothing for them to share in an L2 -- and left up to 7 x groups slots empty.)
+    const int hg = (int)(block % (uint32_t)groups);
+    const int64_t s_idx = block / (uint32_t)groups; // range index
     // (virtual positions: see kBoundaryTokens)
     const const_tab_t kvstarts = (const_tab_t)p.kvstarts, seqstarts = (const_tab_t)p.seqstarts,
                       cachestarts = (const_tab_t)p.cachestarts;
@@ -966,7 +966,7 @@ static pplhip_retcode decode_setup(const pplhip_mhca_args* a, const pplhip_mhca_
     p.num_ranges = plan->decode_num_ranges;
     p.hpb = decode_heads_per_block(p.kv_heads);
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
-    if (p.num_ranges <= 0 || (p.num_ranges & 7) || plan->decode_heads_per_block != p.hpb)
+    if (p.num_ranges <= 0 || plan->decode_heads_per_block != p.hpb)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: plan was not produced by pplhip_mhca_prepare for these arguments");
     if (ws == nullptr) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: needs the workspace reported by pplhip_mhca_prepare");
     const size_t slots = (size_t)p.num_ranges + nd;
