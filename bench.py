@@ -44,7 +44,8 @@ def parse():
     ap.add_argument("--sections", default="all",
                     help="comma-separated subset of the secondary measurements to run: probes, prefill (cfg2 prefill "
                          "part, fused mixed call, rope + cache write), engine, churn, layer_slab, other (cfg1, cfg3, "
-                         "8k prompts, chunked prefill, general kernels), cpu; the headline decode loop always runs")
+                         "8k prompts, chunked prefill, general kernels), prefill_lengths (32 768 prompt tokens as prompts of 128 ... "
+                         "8 192 tokens), cpu; the headline decode loop always runs")
     ap.add_argument("--quick", action="store_true",
                     help="a dozen calls per secondary figure instead of >= 100 calls and >= 200 ms: for counter runs "
                          "(rocprofv3 --pmc serialises dispatches), not for reported timings")
@@ -759,6 +760,22 @@ def main():
         del gpb
         torch.cuda.empty_cache()
         result["general_kernel"] = gen
+    if args.workload == "cfg2" and want("prefill_lengths"):
+        # 32 768 prompt tokens as prompts of one length: the same 8 192 tile workgroups every time, from 1.5 to 65
+        # 64-key steps each -- separates what a workgroup costs from what a step costs
+        import numpy as _np
+        sweep = {}
+        for plen in (128, 256, 512, 1024, 2048, 4096, 8192):
+            n = 32768 // plen
+            sb = workloads.Batch(32, 8, 128, _np.full(n, plen, _np.int64), _np.zeros(n, _np.int64), 0, name="%dx%d prefill" % (n, plen))
+            sdb = DeviceBatch(pkg, lib, sb, seed=9, n_slabs=1)
+            tiles = n * (plen // 128) * 32
+            steps = n * 32 * sum(2 * (i + 1) for i in range(plen // 128))
+            sweep["%d_prompts_x_%d_tokens" % (n, plen)] = prefill_entry(
+                sdb, sb, {"tile_workgroups": tiles, "workgroup_steps": steps})
+            del sdb
+            torch.cuda.empty_cache()
+        result["prefill_by_prompt_length"] = sweep
     if args.copy_calibration:
         copy_calibration()
     if not args.no_cpu_baseline and want("cpu"):
