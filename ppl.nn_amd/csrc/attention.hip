@@ -46,8 +46,11 @@ pplhip_retcode launch_decode_and_prefill(const pplhip_mhca_args* a, const pplhip
         rc = launch_decode(a, plan, ws, stream);
         return rc != PPLHIP_RC_SUCCESS ? rc : launch_prefill(a, plan, ws, stream);
     }
-    rc = prefill_setup(a, plan, ws, stream, &pp, &pblocks, &from_slab);
+    // the prompts' write-only workgroups (dispatched last, into the launch's tail) take the decode sequences' new
+    // tokens as well: stores from the middle of a decode wave's stream stall it
+    rc = prefill_setup(a, plan, ws, stream, true, &pp, &pblocks, &from_slab);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
+    dp.new_tokens_written_elsewhere = pp.w_cache != nullptr && pp.w_first_token == 0;
     if (dblocks + pblocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many workgroups in one call");
     static std::atomic<uint64_t> lds_opted_in{0};
     rc = reserve_decode_lds(lds_opted_in, {reinterpret_cast<const void*>(mixed_attention_kernel<false, false>),

@@ -80,6 +80,8 @@ struct DecodeParams {
     int32_t num_ranges; // S
     int32_t hpb; // kv heads per workgroup: min(kv_heads, 4), a power of two dividing kv_heads
     int32_t merge_by_boundary; // merge kernel: blockIdx.y counts range boundaries instead of sequences
+    int32_t new_tokens_written_elsewhere; // the launch's write-only workgroups put the decode sequences' new tokens
+                                          // into the slab: the decode waves only patch their stage buffers
     float score_scale; // log2(e) / sqrt(Dh)
 };
 
@@ -703,9 +705,13 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
                             row = (cur.cbase - reinterpret_cast<const char*>(p.cache)) + tl * (int64_t)stride;
                         }
                         row += isv ? kv_off : 0;
-                        *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
-                        p.scale[row / kQuantGroup + grp] = sc;
-                        // (two more stores behind the next stage 0; the waits count only the result rows)
+                        // (two more stores behind the next stage 0; the waits count only the result rows. A store in
+                        // the middle of a wave's stream costs it about a stage: where the launch has write-only
+                        // workgroups anyway, they take these rows.)
+                        if (!p.new_tokens_written_elsewhere) {
+                            *reinterpret_cast<uint2*>(p.cache + row + grp * 8) = qv;
+                            p.scale[row / kQuantGroup + grp] = sc;
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -976,6 +982,7 @@ static pplhip_retcode decode_setup(const pplhip_mhca_args* a, const pplhip_mhca_
     const int64_t blocks = (int64_t)p.num_ranges * (p.kv_heads / p.hpb);
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many tasks");
     p.merge_by_boundary = nd > p.num_ranges - 1;
+    p.new_tokens_written_elsewhere = 0;
     *out = p;
     *out_blocks = blocks;
     return PPLHIP_RC_SUCCESS;

@@ -1069,8 +1069,10 @@ bool prefill_writes_new_tokens(const pplhip_mhca_args* a) {
 
 // Fills the launch parameters of the prompts' attention (and enqueues the staging pass where the plan has one).
 // *blocks: workgroups of the launch; *from_slab: the kernel that dequantises the int8 slab itself has to run it.
+// with_decode_tokens: the write-only workgroups also quantise the decode sequences' new tokens (the first
+// decoding_batches packed tokens); *out has w_first_token == 0 then.
 static pplhip_retcode prefill_setup(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream,
-                                    PrefillParams* out, int64_t* out_blocks, bool* from_slab) {
+                                    bool with_decode_tokens, PrefillParams* out, int64_t* out_blocks, bool* from_slab) {
     const int npre = (int)(a->batch - a->decoding_batches);
     PrefillParams p;
     p.kv_origin = nullptr;
@@ -1112,7 +1114,8 @@ static pplhip_retcode prefill_setup(const pplhip_mhca_args* a, const pplhip_mhca
     if (prefill_writes_new_tokens(a)) {
         p.w_cache = (int8_t*)a->d_cache;
         p.w_scale = (half_t*)a->d_scale;
-        p.w_first_token = a->decoding_batches; // one new token per decode sequence, then the prompts
+        // one new token per decode sequence, then the prompts
+        p.w_first_token = with_decode_tokens ? 0 : a->decoding_batches;
         p.w_end_token = a->total_new_tokens;
         p.w_batch = (int32_t)a->batch;
         p.w_per_tok = 2 * a->num_kv_heads * 4;
@@ -1147,7 +1150,7 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
     PrefillParams p;
     int64_t blocks;
     bool from_slab;
-    const pplhip_retcode rc = prefill_setup(a, plan, ws, stream, &p, &blocks, &from_slab);
+    const pplhip_retcode rc = prefill_setup(a, plan, ws, stream, false, &p, &blocks, &from_slab);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
     const dim3 grid((unsigned)blocks);
     if (from_slab)
