@@ -143,6 +143,7 @@ def load_engine_library():
             "pplnn_x86_set_num_threads": (None, [ctypes.c_int]),
             "pplnn_x86_get_num_threads": (ctypes.c_int, []),
             "pplnn_hip_arena_create_host": (vp, [u64, u64]),
+            "pplnn_hip_arena_create_host_with_policy": (vp, [u64, u64, u32]),
             "pplnn_hip_arena_alloc": (u32, [vp, u64, ctypes.POINTER(vp), ctypes.POINTER(u64)]),
             "pplnn_hip_arena_free": (None, [vp, vp]),
             "pplnn_hip_arena_buffered_bytes": (u64, [vp]),

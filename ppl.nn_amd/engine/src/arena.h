@@ -17,8 +17,14 @@ class ArenaBufferManager final {
 public:
     typedef std::function<void*(uint64_t)> RawAlloc;
     typedef std::function<void(void*)> RawFree;
-    ArenaBufferManager(const RawAlloc& a, const RawFree& f, uint64_t alignment, uint64_t block_bytes)
-        : raw_alloc_(a), raw_free_(f), alignment_(alignment), block_bytes_(block_bytes) {}
+    // How a request picks among the free pieces: the smallest that fits (MM_BEST_FIT, the reference's
+    // bestfit_buffered_device.cc) or the one at the lowest address (MM_COMPACT, buffered_device.cc over the compact
+    // manager: the heap stays packed towards its start). kPlain keeps nothing: every request is a raw allocation
+    // that goes back to the raw allocator when it is freed (MM_PLAIN, plain_device.cc).
+    enum Policy { kBestFit, kCompact, kPlain };
+    ArenaBufferManager(const RawAlloc& a, const RawFree& f, uint64_t alignment, uint64_t block_bytes,
+                       Policy policy = kBestFit)
+        : raw_alloc_(a), raw_free_(f), alignment_(alignment), block_bytes_(block_bytes), policy_(policy) {}
     ~ArenaBufferManager() {
         for (auto& b : blocks_) raw_free_(b.first);
     }
@@ -26,10 +32,16 @@ public:
         std::lock_guard<std::mutex> guard(lock_);
         const uint64_t need = Align(bytes ? bytes : 1);
         auto best = free_by_addr_.end();
-        for (auto it = free_by_addr_.begin(); it != free_by_addr_.end(); ++it) // best fit
-            if (it->second >= need && (best == free_by_addr_.end() || it->second < best->second)) best = it;
+        for (auto it = free_by_addr_.begin(); it != free_by_addr_.end(); ++it) {
+            if (it->second < need) continue;
+            if (policy_ == kCompact) { // the map is ordered by address: the first that fits is the lowest
+                best = it;
+                break;
+            }
+            if (best == free_by_addr_.end() || it->second < best->second) best = it;
+        }
         if (best == free_by_addr_.end()) {
-            const uint64_t block = need > block_bytes_ ? need : block_bytes_;
+            const uint64_t block = (policy_ == kPlain || need > block_bytes_) ? need : block_bytes_;
             void* p = raw_alloc_(block);
             if (!p) {
                 LOG(ERROR) << "arena: raw allocation of " << block << " bytes failed";
@@ -55,6 +67,14 @@ public:
         char* addr = it->first;
         uint64_t size = it->second;
         used_.erase(it);
+        if (policy_ == kPlain) { // the piece is a raw block of its own
+            blocks_.erase(addr);
+            buffered_bytes_ -= size;
+            raw_free_(addr);
+            buffer->addr = nullptr;
+            buffer->desc = 0;
+            return;
+        }
         // coalesce with the neighbours, but never across raw blocks
         auto next = free_by_addr_.lower_bound(addr);
         if (next != free_by_addr_.end() && addr + size == next->first && !IsBlockStart(next->first)) {
@@ -87,6 +107,7 @@ private:
     RawAlloc raw_alloc_;
     RawFree raw_free_;
     uint64_t alignment_, block_bytes_;
+    Policy policy_;
     std::map<char*, uint64_t> blocks_, free_by_addr_, used_;
     uint64_t buffered_bytes_ = 0;
     std::mutex lock_;

@@ -247,6 +247,14 @@ uint32_t pplnn_hip_selftest_registry(void) {
 void* pplnn_hip_arena_create_host(uint64_t alignment, uint64_t block_bytes) {
     return new utils::ArenaBufferManager([](uint64_t n) { return malloc(n); }, [](void* p) { free(p); }, alignment, block_bytes);
 }
+// mm_policy: MM_PLAIN / MM_COMPACT / MM_BEST_FIT of the llm_hip engine options
+void* pplnn_hip_arena_create_host_with_policy(uint64_t alignment, uint64_t block_bytes, uint32_t mm_policy) {
+    const auto policy = mm_policy == llm::hip::MM_PLAIN     ? utils::ArenaBufferManager::kPlain
+                        : mm_policy == llm::hip::MM_COMPACT ? utils::ArenaBufferManager::kCompact
+                                                            : utils::ArenaBufferManager::kBestFit;
+    return new utils::ArenaBufferManager([](uint64_t n) { return malloc(n); }, [](void* p) { free(p); }, alignment,
+                                         block_bytes, policy);
+}
 uint32_t pplnn_hip_arena_alloc(void* a, uint64_t bytes, void** addr, uint64_t* desc) {
     BufferDesc b;
     auto rc = static_cast<utils::ArenaBufferManager*>(a)->Alloc(bytes, &b);

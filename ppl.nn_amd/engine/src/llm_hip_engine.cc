@@ -76,7 +76,7 @@ public:
         arena_.reset();
         if (own_stream_ && stream_) hipStreamDestroy(stream_);
     }
-    RetCode Init(int device_id, void* stream) {
+    RetCode Init(int device_id, void* stream, uint32_t mm_policy = MM_BEST_FIT) {
         device_id_ = device_id;
         int count = 0;
         if (hipGetDeviceCount(&count) != hipSuccess || device_id >= count) {
@@ -99,7 +99,10 @@ public:
                 void* p = nullptr;
                 return hipMalloc(&p, bytes) == hipSuccess ? p : nullptr;
             },
-            [](void* p) { (void)hipFree(p); }, 256, 64ull << 20));
+            [](void* p) { (void)hipFree(p); }, 256, 64ull << 20,
+            mm_policy == MM_PLAIN     ? utils::ArenaBufferManager::kPlain
+                : mm_policy == MM_COMPACT ? utils::ArenaBufferManager::kCompact
+                                          : utils::ArenaBufferManager::kBestFit));
         return RC_SUCCESS;
     }
     hipStream_t GetStream() const { return stream_; }
@@ -173,7 +176,7 @@ public:
             return RC_SUCCESS;
         }
         owned_.reset(new LlmHipDevice());
-        auto rc = owned_->Init((int)options.device_id, options.runtime_stream);
+        auto rc = owned_->Init((int)options.device_id, options.runtime_stream, options.mm_policy);
         if (rc != RC_SUCCESS) return rc;
         device_ = owned_.get();
         return RC_SUCCESS;
@@ -1101,7 +1104,7 @@ Engine* EngineFactory::Create(const EngineOptions& options) {
 
 DeviceContext* EngineFactory::CreateDeviceContext(const DeviceOptions& options) {
     auto dev = new LlmHipDevice();
-    if (dev->Init(options.device_id, options.stream) != RC_SUCCESS) {
+    if (dev->Init(options.device_id, options.stream, options.mm_policy) != RC_SUCCESS) {
         delete dev;
         return nullptr;
     }

@@ -49,6 +49,61 @@ def test_arena_known_answers_of_the_reference_buffer_manager_tests(eng):
     eng.pplnn_hip_arena_destroy(a)
 
 
+def test_arena_follows_the_engine_memory_policy(eng):
+    """MM_PLAIN / MM_COMPACT / MM_BEST_FIT (include/ppl/nn/engines/llm_cuda/options.h; engine_context.cc:49-59 picks
+    PlainDevice, BufferedDevice or BestFitBufferedDevice): which free piece a request takes, and what a free keeps."""
+    MM_PLAIN, MM_COMPACT, MM_BEST_FIT = 0, 1, 2
+
+    def holes(policy):
+        # one 4096-byte block cut into pieces of 1024 | 512 | 2048 | 512; pieces 0 and 2 are freed: holes of 1024 at
+        # the start and 2048 further up, kept apart by piece 1
+        a = eng.pplnn_hip_arena_create_host_with_policy(64, 4096, policy)
+        ptrs = []
+        for n in (1024, 512, 2048, 512):
+            addr, desc = C.c_void_p(), C.c_uint64()
+            assert eng.pplnn_hip_arena_alloc(a, n, C.byref(addr), C.byref(desc)) == 0
+            ptrs.append(addr.value)
+        eng.pplnn_hip_arena_free(a, C.c_void_p(ptrs[0]))
+        eng.pplnn_hip_arena_free(a, C.c_void_p(ptrs[2]))
+        return a, ptrs
+
+    # a 2048-byte request fits only the upper hole under either policy; a 700-byte request tells them apart:
+    # best fit and compact both take the 1024-byte hole here, so ask for the case where they differ: 1500 bytes do not
+    # fit the low hole, 900 bytes fit both -- compact takes the LOWEST address, best fit the SMALLEST piece
+    a, ptrs = holes(MM_COMPACT)
+    addr, desc = C.c_void_p(), C.c_uint64()
+    assert eng.pplnn_hip_arena_alloc(a, 900, C.byref(addr), C.byref(desc)) == 0 and addr.value == ptrs[0]
+    eng.pplnn_hip_arena_destroy(a)
+    a, ptrs = holes(MM_BEST_FIT)
+    assert eng.pplnn_hip_arena_alloc(a, 900, C.byref(addr), C.byref(desc)) == 0 and addr.value == ptrs[0]
+    eng.pplnn_hip_arena_destroy(a)
+    # now the low hole is the LARGER one: 2048 | 512 | 1024 | 512 with pieces 0 and 2 freed
+    for policy, want in ((MM_COMPACT, 0), (MM_BEST_FIT, 2)):
+        a = eng.pplnn_hip_arena_create_host_with_policy(64, 4096, policy)
+        ptrs = []
+        for n in (2048, 512, 1024, 512):
+            assert eng.pplnn_hip_arena_alloc(a, n, C.byref(addr), C.byref(desc)) == 0
+            ptrs.append(addr.value)
+        eng.pplnn_hip_arena_free(a, C.c_void_p(ptrs[0]))
+        eng.pplnn_hip_arena_free(a, C.c_void_p(ptrs[2]))
+        assert eng.pplnn_hip_arena_alloc(a, 900, C.byref(addr), C.byref(desc)) == 0
+        assert addr.value == ptrs[want]
+        assert eng.pplnn_hip_arena_buffered_bytes(a) == 4096
+        eng.pplnn_hip_arena_destroy(a)
+    # plain: every request is its own raw allocation and goes back when freed
+    a = eng.pplnn_hip_arena_create_host_with_policy(64, 4096, MM_PLAIN)
+    assert eng.pplnn_hip_arena_alloc(a, 1000, C.byref(addr), C.byref(desc)) == 0
+    assert eng.pplnn_hip_arena_buffered_bytes(a) == 1024 and eng.pplnn_hip_arena_used_bytes(a) == 1024
+    other = C.c_void_p()
+    assert eng.pplnn_hip_arena_alloc(a, 64, C.byref(other), C.byref(desc)) == 0
+    assert eng.pplnn_hip_arena_buffered_bytes(a) == 1024 + 64
+    eng.pplnn_hip_arena_free(a, addr)
+    assert eng.pplnn_hip_arena_buffered_bytes(a) == 64 and eng.pplnn_hip_arena_used_bytes(a) == 64
+    eng.pplnn_hip_arena_free(a, other)
+    assert eng.pplnn_hip_arena_buffered_bytes(a) == 0
+    eng.pplnn_hip_arena_destroy(a)
+
+
 def _load(eng, buf):
     b = eng.pplnn_hip_builder_create()
     rc = eng.pplnn_hip_builder_load_model(b, buf, len(buf))

@@ -17,9 +17,9 @@ def _i64(*dims):
 
 
 class Session:
-    def __init__(self, eng, model_bytes, configure=()):
+    def __init__(self, eng, model_bytes, configure=(), mm_policy=1):
         self.eng = eng
-        self.engine = eng.pplnn_hip_engine_create(0, 1)
+        self.engine = eng.pplnn_hip_engine_create(0, mm_policy)  # 0 MM_PLAIN, 1 MM_COMPACT, 2 MM_BEST_FIT
         assert self.engine
         for opt, val in configure:
             assert eng.pplnn_hip_engine_configure_u32(self.engine, opt, val) == 0
@@ -84,8 +84,8 @@ def _prepare_slab(b, t, hiplib):
     return cache, scale
 
 
-@pytest.mark.parametrize("cache_prefill", [0, 1])
-def test_mhca_graph_through_the_engine(hiplib, cache_prefill):
+@pytest.mark.parametrize("cache_prefill,mm_policy", [(0, 1), (1, 1), (0, 0), (1, 2)])
+def test_mhca_graph_through_the_engine(hiplib, cache_prefill, mm_policy):
     import torch
     eng = harness.pkg.load_engine_library()
     b = workloads.Batch(32, 8, 128, [1, 1, 1, 1, 70, 200], [500, 3, 77, 1300, 0, 0], 4, num_layer=2, layer_idx=1,
@@ -93,7 +93,7 @@ def test_mhca_graph_through_the_engine(hiplib, cache_prefill):
     t = workloads.make_tensors(b, seed=77)
     ref = harness.run_oracle(b, t, cache_prefill=cache_prefill)
     cache, scale = _prepare_slab(b, t, hiplib)
-    s = Session(eng, ow.mhca_model(32, 8, 128, 2, 1), configure=[(1005, cache_prefill)])
+    s = Session(eng, ow.mhca_model(32, 8, 128, 2, 1), configure=[(1005, cache_prefill)], mm_policy=mm_policy)
     assert eng.pplnn_hip_runtime_input_count(s.rt) == 12 and eng.pplnn_hip_runtime_output_count(s.rt) == 1
     assert eng.pplnn_hip_runtime_set_profiling(s.rt, 1) == 0
     s.set_device_tensor(0, harness.to_dev(t["query"]))
