@@ -240,7 +240,7 @@ pplhip_retcode pplhip_kv_cache_forward(const pplhip_kv_cache_args* args, void* s
  * The queries of a sequence are its LAST seqlen keys: with is_causal, query i of sequence b attends to keys
  * 0 .. (kvlen_b - seqlen_b) + i; without, to all kvlen_b keys. kvlen_b >= seqlen_b >= 1 is required.
  * MultiHeadCacheAttention == MultiHeadAttention applied to the outputs of KeyValueCache.
- * head_dim: a multiple of 32 up to 256 (128 with at most 16 query heads per kv head and no mask runs the tuned kernel,
+ * head_dim: a multiple of 16 up to 256 (128 with at most 16 query heads per kv head and no mask runs the tuned kernel,
  * everything else the general one); no alibi.
  */
 typedef struct pplhip_mha_args {

@@ -57,7 +57,7 @@ static pplhip_retcode validate_common(int num_kv_heads, int head_dim, int num_la
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "bad num_kv_heads/num_layer/layer_idx (%d/%d/%d)", num_kv_heads,
                     num_layer, layer_idx);
     if (!generic_head_dim_supported(head_dim))
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 32 between 32 and 256", head_dim);
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 16 between 16 and 256", head_dim);
     if (!cache) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "cache pointer is null");
     if (!scale)
         PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support quantized cache but scale not found");
@@ -321,7 +321,7 @@ pplhip_retcode pplhip_mha_forward(const pplhip_mha_args* a, void* stream) {
     if (!a) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
     if (a->is_alibi) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "currently only support is_alibi == false");
     if (!generic_head_dim_supported(a->head_dim))
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 32 between 32 and 256", a->head_dim);
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 16 between 16 and 256", a->head_dim);
     {
         const pplhip_retcode rcm = validate_mask(a->d_attn_mask, a->attn_mask_stride_h, a->attn_mask_stride_q);
         if (rcm != PPLHIP_RC_SUCCESS) return rcm;

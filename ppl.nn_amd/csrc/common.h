@@ -181,7 +181,7 @@ pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan*
 pplhip_retcode launch_decode_and_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws,
                                          hipStream_t stream);
 pplhip_retcode launch_mha(const pplhip_mha_args* a, hipStream_t stream);
-// the general attention kernel: any head_dim that is a multiple of 32 up to 256, any number of query heads per kv
+// the general attention kernel: any head_dim that is a multiple of 16 up to 256, any number of query heads per kv
 // head, optional attn_mask. The MHCA form reads the slab, which must already hold the call's new tokens.
 bool generic_head_dim_supported(int head_dim);
 // nsplit pieces per decode sequence (generic_decode_splits), their partial results in `ws` (generic_workspace_bytes)

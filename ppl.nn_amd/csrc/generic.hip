@@ -1,6 +1,10 @@
 // The attention kernels for everything the specialised kernels (decode.hip, prefill.hip: head_dim 128, at most 16 query
-// heads per kv head, no mask) do not take: any head_dim that is a multiple of 32 up to 256, any number of query heads
+// heads per kv head, no mask) do not take: any head_dim that is a multiple of 16 up to 256, any number of query heads
 // per kv head, and an additive attn_mask; for MultiHeadCacheAttention and MultiHeadAttention.
+// The kernels are compiled for head dims that are multiples of 32 (DH). Another head_dim (80, 112, ...) runs the next
+// larger DH with the channels past head_dim held as zeros where rows enter LDS or registers (zero query and key
+// channels add nothing to a score, zero value channels give output channels that are not stored); rows in memory keep
+// their real length. Such calls go through the tile kernel only.
 //
 // generic_attention_kernel (the tile kernel: prompts, MultiHeadAttention, decode tokens with more than 16 query heads
 // per kv head). Rows of a workgroup are (query token, query head of the kv head) pairs of ONE (sequence, kv head): row
@@ -39,6 +43,7 @@ struct GenericParams {
     int64_t mask_stride_h, mask_stride_q;
     half_t* out; // [S, H, DH]
     int32_t batch, num_heads, kv_heads, rep;
+    int32_t head_dim; // channels of a row in q / k16 / v16 / out and of a head in the slab (<= the kernel's DH)
     int32_t first_fp16_seq; // sequences [0, first_fp16_seq) read the slab, the others the fp16 rows
     int32_t k16_holds_new_tokens; // the fp16 rows are the sequences' NEW tokens only (MultiHeadCacheAttention's
                                   // current_key / current_value), packed by seqstarts: such a sequence has seqlen keys
@@ -124,6 +129,7 @@ void generic_attention_kernel(const GenericParams p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r_lane = lane & 15, g = lane >> 4;
+    const int hd = p.head_dim; // <= DH; rows in memory are hd channels long
     // the lane's rows: one in each of the wave's RB blocks of 16
     bool valid[RB];
     int64_t tok[RB], row_limit[RB];
@@ -156,9 +162,16 @@ void generic_attention_kernel(const GenericParams p) {
     const bool masked = p.mask != nullptr;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-        const half_t* qp = p.q + ((s0 + tok[rb]) * p.num_heads + head[rb]) * DH + 8 * g;
+        const half_t* qp = p.q + ((s0 + tok[rb]) * p.num_heads + head[rb]) * hd + 8 * g;
 #pragma unroll
-        for (int kc = 0; kc < KC2; ++kc) qf[rb][kc] = *reinterpret_cast<const half8_t*>(qp + 32 * kc);
+        for (int kc = 0; kc < KC2; ++kc) {
+            if (32 * kc + 8 * g < hd) {
+                qf[rb][kc] = *reinterpret_cast<const half8_t*>(qp + 32 * kc);
+            } else { // a padding channel group
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qf[rb][kc][e] = (half_t)0.f;
+            }
+        }
         mrow[rb] = masked ? p.mask + (int64_t)head[rb] * p.mask_stride_h + (s0 + tok[rb]) * p.mask_stride_q + kv_first
                           : nullptr;
     }
@@ -194,14 +207,14 @@ void generic_attention_kernel(const GenericParams p) {
     // a paged slab looks every token up.
     const bool paged = from_slab && p.pages.page_shift != 0;
     const int64_t seq_tok0 = from_slab && !paged ? p.pages.cachestarts[b] : 0;
-    const int64_t tile_stride = from_slab ? (int64_t)BN * p.addr.stride_s : (int64_t)BN * p.kv_heads * DH;
+    const int64_t tile_stride = from_slab ? (int64_t)BN * p.addr.stride_s : (int64_t)BN * p.kv_heads * hd;
     int64_t koff[NCH];
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
         const int c = tid + 256 * n;
         const int r = c / CH, ch = c - r * CH;
         koff[n] = from_slab ? p.addr.row(seq_tok0 + kv_begin + r, 0, kvh) + ch * 8
-                            : ((k16_row0 + kv_begin + r) * p.kv_heads + kvh) * DH + ch * 8;
+                            : ((k16_row0 + kv_begin + r) * p.kv_heads + kvh) * hd + ch * 8;
     }
     auto fetch = [&](int64_t kv0) {
         const int64_t left64 = kvlen - kv0;
@@ -210,7 +223,7 @@ void generic_attention_kernel(const GenericParams p) {
         for (int n = 0; n < NCH; ++n) {
             const int c = tid + 256 * n;
             const int r = c / CH, ch = c - r * CH;
-            if (c < BN * CH && r < left) {
+            if (c < BN * CH && r < left && ch * 8 < hd) { // (chunks past head_dim are padding: zeros)
                 if (from_slab) {
                     int64_t rk = koff[n];
                     if (paged) rk = p.addr.row(p.pages.token(b, kv0 + r), 0, kvh) + ch * 8;
@@ -418,12 +431,12 @@ void generic_attention_kernel(const GenericParams p) {
         }
         // a row whose keys were all masked out has no distribution: zeros
         const float inv_l = l > 0.f ? 1.0f / l : 0.f;
-        half_t* dst = p.out + ((s0 + tok[rb]) * p.num_heads + head[rb]) * DH + 4 * g;
+        half_t* dst = p.out + ((s0 + tok[rb]) * p.num_heads + head[rb]) * hd + 4 * g;
 #pragma unroll
         for (int db = 0; db < KC; ++db) {
             const half4_t r = {(half_t)(o[rb][db][0] * inv_l), (half_t)(o[rb][db][1] * inv_l),
                                (half_t)(o[rb][db][2] * inv_l), (half_t)(o[rb][db][3] * inv_l)};
-            *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
+            if (16 * db + 4 * g < hd) *reinterpret_cast<half4_t*>(dst + 16 * db) = r;
         }
     }
 }
@@ -753,7 +766,7 @@ __global__ __launch_bounds__(256) void generic_merge_kernel(const GenericParams 
     }
     const float inv = L > 0.f ? 1.0f / L : 0.f; // (no piece with unmasked keys: zeros)
     const half4_t r = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv), (half_t)(acc[2] * inv), (half_t)(acc[3] * inv)};
-    *reinterpret_cast<half4_t*>(p.out + row * DH + d4) = r;
+    if (d4 < p.head_dim) *reinterpret_cast<half4_t*>(p.out + row * p.head_dim + d4) = r;
 }
 
 // two kv heads per wave of the decode kernel: head_dim up to 96 (registers), heads next to each other in the slab
@@ -799,22 +812,27 @@ tiles_launched:
 }
 
 bool generic_head_dim_supported(int head_dim) {
-    return head_dim >= 32 && head_dim <= 256 && head_dim % 32 == 0;
+    return head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0;
 }
+// the head_dim the kernels are compiled for: the next multiple of 32
+static int generic_kernel_head_dim(int head_dim) { return (head_dim + 31) / 32 * 32; }
 
 static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max_seqlen, hipStream_t stream) {
     if (!generic_head_dim_supported(head_dim))
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 32 between 32 and 256", head_dim);
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 16 between 16 and 256", head_dim);
     p.scale_log2 = kLog2e / sqrtf((float)head_dim);
+    p.head_dim = head_dim;
+    const int dh = generic_kernel_head_dim(head_dim);
+    const bool padded = dh != head_dim;
     // tiles of 128 rows (two blocks of 16 per wave) where a sequence has more than 64 rows
-    const int row_blocks = gen_two_row_blocks(head_dim) && max_seqlen * p.rep > kGenRows ? 2 : 1;
+    const int row_blocks = gen_two_row_blocks(dh) && max_seqlen * p.rep > kGenRows ? 2 : 1;
     const int64_t tiles = (max_seqlen * p.rep + kGenRows * row_blocks - 1) / (kGenRows * row_blocks);
     if (tiles <= 0 || p.batch <= 0) return PPLHIP_RC_SUCCESS;
     // p.split_seqs: the decode sequences (the first of the batch, one new token each, all of whose keys are in the slab)
     if (p.nsplit < 1) p.nsplit = 1;
     p.first_seq = 0;
     int64_t blocks, decode_blocks = 0;
-    if (p.split_seqs > 0 && p.rep <= 16 && (p.pages.page_shift == 0 || p.pages.page_shift >= 4)) {
+    if (p.split_seqs > 0 && p.rep <= 16 && !padded && (p.pages.page_shift == 0 || p.pages.page_shift >= 4)) {
         // generic_decode_kernel takes them; the tile kernel the rest of the batch
         if (p.nsplit == 1) p.piece_tokens = 0x7fffffc0; // the whole sequence
         decode_blocks = ((int64_t)p.split_seqs * p.nsplit * (p.kv_heads / generic_decode_heads_per_wave(p, head_dim)) + 3) / 4;
@@ -829,7 +847,7 @@ static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max
     if (tiles > 0x7fffffffLL || blocks > 0x7fffffffLL || decode_blocks > 0x7fffffffLL)
         PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "attention: too many row tiles");
     p.tiles_max = (int32_t)tiles;
-    switch (head_dim) {
+    switch (dh) {
         case 32: launch_one<32>(p, blocks, decode_blocks, row_blocks, stream); break;
         case 64: launch_one<64>(p, blocks, decode_blocks, row_blocks, stream); break;
         case 96: launch_one<96>(p, blocks, decode_blocks, row_blocks, stream); break;
@@ -865,7 +883,7 @@ static int generic_piece_tokens(int64_t max_kvlen, int nsplit) {
 }
 uint64_t generic_workspace_bytes(const pplhip_mhca_args* a, int nsplit) {
     if (nsplit <= 1) return 0;
-    return (uint64_t)a->decoding_batches * a->num_heads * nsplit * (a->head_dim + 2) * sizeof(float);
+    return (uint64_t)a->decoding_batches * a->num_heads * nsplit * (generic_kernel_head_dim(a->head_dim) + 2) * sizeof(float);
 }
 
 // MultiHeadCacheAttention through the general kernel; the new tokens are already in the slab.
@@ -875,7 +893,9 @@ pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* 
     p.split_seqs = (int32_t)a->decoding_batches;
     p.piece_tokens = generic_piece_tokens(a->max_kvlen, p.nsplit);
     p.part_o = (float*)ws;
-    p.part_ml = p.nsplit > 1 ? (float*)ws + (size_t)a->decoding_batches * a->num_heads * p.nsplit * a->head_dim : nullptr;
+    p.part_ml = p.nsplit > 1 ? (float*)ws + (size_t)a->decoding_batches * a->num_heads * p.nsplit *
+                                                generic_kernel_head_dim(a->head_dim)
+                             : nullptr;
     if (p.nsplit > 1 && ws == nullptr)
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "attention: needs the workspace reported by pplhip_mhca_prepare");
     p.q = (const half_t*)a->d_query;

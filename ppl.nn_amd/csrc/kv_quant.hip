@@ -20,8 +20,9 @@ struct QuantWriteParams {
     CacheAddr addr;
     int32_t batch;
     int32_t kv_heads;
-    int32_t per_tok; // 4-group units per token: 2 * kv_heads * (head_dim / 32)
-    int32_t units_per_head; // head_dim / 32
+    int32_t per_tok; // 4-group units per token: 2 * kv_heads * units_per_head
+    int32_t units_per_head; // ceil(head_dim / 32): the last unit of a head holds two groups when head_dim % 32 == 16
+    int32_t groups_per_head; // head_dim / 8 (even)
     uint32_t inv_units_per_head; // ceil(65536 / units_per_head): r / units_per_head == (r * inv) >> 16 for r < 8192
     int32_t blocks_per_tok, tok_per_block; // one of the two is 1
     uint32_t inv_per_tok; // ceil(65536 / per_tok)
@@ -30,8 +31,9 @@ struct QuantWriteParams {
 
 // One thread owns four consecutive groups (64 B of fp16 in, 32 B of int8 + 8 B of scales out) so that enough bytes
 // are in flight per CU to cover the memory latency. Thread -> (token, K or V, head, quarter of the head) without
-// integer division: a token has per_tok = 2 * kv_heads * (head_dim / 32) such units; a block covers 256 / per_tok
-// whole tokens, one token, or a 256-unit slice of one.
+// integer division: a token has per_tok = 2 * kv_heads * ceil(head_dim / 32) such units; a block covers 256 / per_tok
+// whole tokens, one token, or a 256-unit slice of one. head_dim is a multiple of 16: a head's last unit holds four
+// groups or two.
 __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWriteParams p) {
     int64_t t; // packed new-token index
     int r; // unit index inside the token
@@ -52,11 +54,14 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     const int kv = hi >= p.kv_heads;
     const int head = hi - kv * p.kv_heads;
     // the values do not depend on which sequence the token belongs to: their loads go out before the look-up
+    const bool four = grp + 4 <= p.groups_per_head; // (else two: the rest of the unit lies past the head's row)
     const uint4* src = reinterpret_cast<const uint4*>((kv ? p.value : p.key) +
-                                                      ((t * p.kv_heads + head) * (4 * p.units_per_head) + grp) * 8);
+                                                      ((t * p.kv_heads + head) * p.groups_per_head + grp) * 8);
     uint4 raw[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) raw[i] = src[i];
+    raw[0] = src[0];
+    raw[1] = src[1];
+    raw[2] = four ? src[2] : make_uint4(0, 0, 0, 0);
+    raw[3] = four ? src[3] : make_uint4(0, 0, 0, 0);
     // decode sequences come first and hold one token each, so for them the packed token index IS the sequence index:
     // two independent loads settle it; only prompt tokens pay for a search of the table
     int b;
@@ -79,12 +84,12 @@ __global__ __launch_bounds__(256) void kv_quantize_write_kernel(const QuantWrite
     const int64_t row = p.addr.row(tok, kv, head);
     uint4* dst = reinterpret_cast<uint4*>(p.cache + row + grp * 8); // rows and grp * 8 are multiples of 16
     dst[0] = make_uint4(q[0].x, q[0].y, q[1].x, q[1].y);
-    dst[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
+    if (four) dst[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
     uint32_t packed[2];
     __builtin_memcpy(packed, sc, 8);
     uint32_t* sdst = reinterpret_cast<uint32_t*>(p.scale + row / kQuantGroup + grp); // row / 8 and grp are even
     sdst[0] = packed[0];
-    sdst[1] = packed[1];
+    if (four) sdst[1] = packed[1];
 }
 
 pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream_t stream, int64_t first_token,
@@ -103,9 +108,10 @@ pplhip_retcode launch_kv_quantize_write(const pplhip_kv_write_args* a, hipStream
     p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
     p.batch = (int32_t)a->batch;
     p.kv_heads = a->num_kv_heads;
-    if (a->head_dim <= 0 || a->head_dim % (4 * kQuantGroup) || a->head_dim > 256)
-        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: head_dim must be a multiple of 32, at most 256");
-    p.units_per_head = a->head_dim / (4 * kQuantGroup);
+    if (a->head_dim <= 0 || a->head_dim % (2 * kQuantGroup) || a->head_dim > 256)
+        PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: head_dim must be a multiple of 16, at most 256");
+    p.groups_per_head = a->head_dim / kQuantGroup;
+    p.units_per_head = (p.groups_per_head + 3) / 4;
     p.inv_units_per_head = (65536u + (uint32_t)p.units_per_head - 1) / (uint32_t)p.units_per_head;
     p.per_tok = 2 * a->num_kv_heads * p.units_per_head;
     if (p.per_tok >= 8192) PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "kv_quantize_write: too many kv heads (%d)", a->num_kv_heads);
@@ -224,15 +230,15 @@ struct GatherParams {
     int32_t batch;
     int32_t kv_heads;
     int32_t groups_per_head;
-    int64_t total_groups; // total_kv_tokens * 2 * kv_heads * groups_per_head
+    int64_t total_units; // total_kv_tokens * 2 * kv_heads * ceil(groups_per_head / 4)
 };
 
 // A thread takes four groups (32 channels) of one (token, K or V, head): 32 bytes of int8 and four scales in, 64 bytes
 // of fp16 out; the index arithmetic (three divisions) is spent once per 32 channels.
 __global__ __launch_bounds__(256) void kv_gather_dequant_kernel(const GatherParams p) {
     const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // unit of four groups
-    if (u >= p.total_groups / 4) return;
-    const int uph = p.groups_per_head / 4; // units per head (head_dim is a multiple of 32)
+    if (u >= p.total_units) return;
+    const int uph = (p.groups_per_head + 3) / 4; // units per head (the last holds two groups when head_dim % 32 == 16)
     const int per_kv = p.kv_heads * uph;
     const int per_tok = 2 * per_kv;
     // packed kv-token index (a 32-bit division where the numbers allow it)
@@ -254,9 +260,10 @@ __global__ __launch_bounds__(256) void kv_gather_dequant_kernel(const GatherPara
     const int64_t tok = p.cachestarts[b] + (j - p.kvstarts[b]);
     const int64_t row = p.addr.row(tok, kv, head);
     const uint4* src = reinterpret_cast<const uint4*>(p.cache + row + grp * 8); // rows and grp * 8: multiples of 16
-    const uint4 q0 = src[0], q1 = src[1];
+    const bool four = grp + 4 <= p.groups_per_head;
+    const uint4 q0 = src[0], q1 = four ? src[1] : make_uint4(0, 0, 0, 0);
     const uint32_t* ssrc = reinterpret_cast<const uint32_t*>(p.scale + row / kQuantGroup + grp);
-    const uint32_t sw[2] = {ssrc[0], ssrc[1]};
+    const uint32_t sw[2] = {ssrc[0], four ? ssrc[1] : 0u};
     const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
     uint4* dst = reinterpret_cast<uint4*>((kv ? p.value_out : p.key_out) +
                                           ((j * p.kv_heads + head) * p.groups_per_head + grp) * 8);
@@ -268,7 +275,7 @@ __global__ __launch_bounds__(256) void kv_gather_dequant_kernel(const GatherPara
         const half8_t o = dequant8(qw[2 * g], qw[2 * g + 1], sc); // = fp16(float(q) * float(scale)), one rounding
         uint4 packed;
         __builtin_memcpy(&packed, &o, 16);
-        dst[g] = packed;
+        if (g < 2 || four) dst[g] = packed;
     }
 }
 
@@ -286,8 +293,8 @@ pplhip_retcode launch_kv_gather_dequant(const pplhip_kv_cache_args* a, hipStream
     p.batch = (int32_t)w->batch;
     p.kv_heads = w->num_kv_heads;
     p.groups_per_head = w->head_dim / kQuantGroup;
-    p.total_groups = a->total_kv_tokens * 2 * (int64_t)w->num_kv_heads * p.groups_per_head;
-    const int64_t blocks = (p.total_groups / 4 + 255) / 256;
+    p.total_units = a->total_kv_tokens * 2 * (int64_t)w->num_kv_heads * ((p.groups_per_head + 3) / 4);
+    const int64_t blocks = (p.total_units + 255) / 256;
     if (blocks > 0x7fffffffLL) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "kv_gather_dequant: too many groups");
     hipLaunchKernelGGL(kv_gather_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     PPLHIP_CHECK_LAUNCH("kv_gather_dequant");

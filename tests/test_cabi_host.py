@@ -94,7 +94,7 @@ def test_prepare_accepts_valid_and_sizes_workspace(hiplib):
      cabi.RC_UNSUPPORTED),
     (lambda a: (setattr(a, "cache_mode", 1), setattr(a, "cachestart_stride_b", 4), setattr(a, "page_size", 32)),
      cabi.RC_UNSUPPORTED),
-    (lambda a: setattr(a, "head_dim", 80), cabi.RC_UNSUPPORTED),  # multiples of 32 up to 256
+    (lambda a: setattr(a, "head_dim", 72), cabi.RC_UNSUPPORTED),  # multiples of 16 up to 256
     (lambda a: setattr(a, "head_dim", 288), cabi.RC_UNSUPPORTED),
     (lambda a: setattr(a, "num_kv_heads", 3), cabi.RC_INVALID_VALUE),
     (lambda a: setattr(a, "layer_idx", 5), cabi.RC_INVALID_VALUE),

@@ -122,7 +122,7 @@ def test_mhca_graph_through_the_engine(hiplib, cache_prefill, mm_policy):
     s.close()
 
 
-@pytest.mark.parametrize("head_dim,mask_rank", [(64, 0), (64, 3), (128, 2), (256, 0)])
+@pytest.mark.parametrize("head_dim,mask_rank", [(64, 0), (64, 3), (128, 2), (256, 0), (80, 0), (112, 3)])
 def test_mhca_graph_other_head_dims_and_attn_mask(hiplib, head_dim, mask_rank):
     """The same graph with a head_dim other than 128 and / or the optional 13th input attn_mask: the engine reads the
     mask's strides off its shape and the call runs the general kernel."""

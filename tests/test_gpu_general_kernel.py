@@ -39,6 +39,20 @@ def test_head_dims_mixed_batch(Dh, H, KVH):
     check(b, workloads.make_tensors(b, seed=Dh + H), f"head_dim {Dh}")
 
 
+@pytest.mark.parametrize("Dh,H,KVH", [(80, 8, 2), (112, 5, 5), (48, 6, 1), (16, 4, 2), (144, 8, 2), (240, 6, 1), (176, 34, 2)])
+def test_head_dims_that_are_not_multiples_of_32(Dh, H, KVH):
+    """head_dim 80, 112, ...: the kernels run the next multiple of 32 with the channels past head_dim held as zeros;
+    rows in memory (queries, fp16 keys, slab heads, outputs) keep their real length, so the neighbouring head's
+    channels must neither be read into a score nor be overwritten. Decode sequences long enough for pieces, prompts
+    over the tile edges, with and without cache-prefill."""
+    b = workloads.Batch(H, KVH, Dh, [1, 1, 1, 1, 7, 65, 130], [700, 1, 63, 64, 0, 0, 33], 4, num_layer=2, layer_idx=1,
+                        name="general_padded")
+    t = workloads.make_tensors(b, seed=Dh + H)
+    check(b, t, f"head_dim {Dh}")
+    check(b, t, f"head_dim {Dh}, cache-prefill", cache_prefill=1)
+    check(b, t, f"head_dim {Dh}, cache_layout 3", layout=3)
+
+
 @pytest.mark.parametrize("H,KVH", [(34, 2), (20, 1), (48, 2)])
 def test_more_than_16_query_heads_per_kv_head(H, KVH):
     b = workloads.Batch(H, KVH, 128, [1, 1, 40, 3], [500, 17, 0, 0], 2, name="general_rep")
@@ -57,7 +71,7 @@ def test_attn_mask(Dh, per_head, causal):
     assert np.abs(plain["output_f64"] - ref["output_f64"]).max() > 1e-3  # the mask matters
 
 
-@pytest.mark.parametrize("H,KVH,Dh", [(8, 2, 64), (6, 6, 96), (34, 2, 128), (4, 1, 256)])
+@pytest.mark.parametrize("H,KVH,Dh", [(8, 2, 64), (6, 6, 96), (34, 2, 128), (4, 1, 256), (8, 2, 80)])
 def test_long_decode_sequences_are_cut_into_pieces(H, KVH, Dh):
     """Decode sequences long enough for the plan to share their keys out among several workgroups: pieces that end
     inside a tile, pieces past a short sequence's end (empty), one sequence of exactly one piece; with a paged slab
@@ -137,7 +151,7 @@ def test_cache_prefill_paged_and_layout_3():
     assert np.array_equal(got3["output"][nd:].view(np.uint16), flat["output"][nd:].view(np.uint16))
 
 
-@pytest.mark.parametrize("Dh,mask_on", [(64, False), (96, True), (256, False), (128, True)])
+@pytest.mark.parametrize("Dh,mask_on", [(64, False), (96, True), (256, False), (128, True), (80, False), (112, True)])
 def test_multi_head_attention_general(Dh, mask_on):
     b = workloads.Batch(8, 2, Dh, [1, 1, 7, 130, 64], [300, 0, 0, 70, 64], 2, name="general_mha")
     t = workloads.make_tensors(b, seed=31)
@@ -163,10 +177,12 @@ def test_general_kernel_agrees_with_the_tuned_kernels():
     assert d.max() <= 2 * (2e-3 + 1e-2 * np.abs(ref["output_f64"]).max())
 
 
-def test_key_value_cache_op_other_head_dim(hiplib, olib):
-    """KeyValueCache (quantise-write + gather) at head_dim 96: slab and gathered rows bit-exact."""
+@pytest.mark.parametrize("Dh", [96, 80, 16])
+def test_key_value_cache_op_other_head_dim(hiplib, olib, Dh):
+    """KeyValueCache (quantise-write + gather) at head_dim 96 and at head dims whose last unit of four quantisation
+    groups is half empty: slab and gathered rows bit-exact."""
     import torch
-    b = workloads.Batch(3, 3, 96, [1, 6, 40], [9, 0, 3], 0, num_layer=2, layer_idx=1, slack_tokens=2)
+    b = workloads.Batch(3, 3, Dh, [1, 6, 40], [9, 0, 3], 0, num_layer=2, layer_idx=1, slack_tokens=2)
     t = workloads.make_tensors(b, seed=9)
     zeros = np.zeros(b.batch, np.int64)
     total_kv = int(b.kvstarts[-1])
@@ -186,8 +202,8 @@ def test_key_value_cache_op_other_head_dim(hiplib, olib):
         a.d_kvstarts = ptr(tabs["ks"])
         a.total_kv_tokens, a.max_kvlen = total_kv, b.max_kvlen
         a.num_repeat, a.cache_mode, a.cache_layout = 1, 0, 0
-        ko = conv(np.zeros((total_kv, 3, 96), np.float16))
-        vo = conv(np.zeros((total_kv, 3, 96), np.float16))
+        ko = conv(np.zeros((total_kv, 3, Dh), np.float16))
+        vo = conv(np.zeros((total_kv, 3, Dh), np.float16))
         a.d_key_out, a.d_value_out = ptr(ko), ptr(vo)
         assert lib_fwd(C.byref(a), *stream_args) == 0
         return cache, scale, ko, vo
