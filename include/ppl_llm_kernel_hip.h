@@ -142,7 +142,10 @@ typedef struct pplhip_mhca_plan {
                                 The caller may clear it before forward to stay on the second route. */
     int32_t prefill_staging_offset_256; /* where the staging rows start in the workspace, in units of 256 bytes */
     int32_t general_kernel; /* 1 = the call runs the general attention kernel (head_dim other than 128, more than 16
-                               query heads per kv head, or an attn_mask): write kernel + one attention launch */
+                               query heads per kv head, or an attn_mask): write kernel + one attention launch. With
+                               decode_num_ranges > 0 (head_dim 64 / 32 whose kv heads are neighbours in the slab and
+                               pair up / go in fours, no mask) the decode sequences of such a call run the decode
+                               kernel over those groups of kv heads and the general kernel takes the prompts. */
     int32_t general_decode_splits; /* general kernel only: pieces the longest decode sequence's keys (max_kvlen) are
                                       cut into, shorter sequences into as many pieces of that length as they fill
                                       (partial results go through the workspace and a merge launch); 0 or 1 = none.

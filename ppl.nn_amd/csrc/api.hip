@@ -83,7 +83,8 @@ static bool needs_general_kernel(int head_dim, int num_heads, int num_kv_heads, 
 static uint64_t decode_workspace_bytes(const pplhip_mhca_args* a, int64_t ranges) {
     if (a->decoding_batches <= 0 || ranges <= 0) return 0;
     const uint64_t rows = ((uint64_t)ranges + (uint64_t)a->decoding_batches) * a->num_heads;
-    return rows * (a->head_dim + 2) * sizeof(float) + (uint64_t)ranges * sizeof(int32_t);
+    // (rows of 128 channels also for the head dims that run this kernel over groups of kv heads)
+    return rows * (128 + 2) * sizeof(float) + (uint64_t)ranges * sizeof(int32_t);
 }
 
 static pplhip_retcode validate_mask(const void* mask, int64_t stride_h, int64_t stride_q) {
@@ -173,6 +174,32 @@ pplhip_retcode pplhip_init(void) {
     return noalloc_scratch_of_current_device(&scratch);
 }
 
+// The decode decomposition: the kernel cuts the decode sequences' cached tokens, laid end to end, into S equal ranges
+// on the device; the host only picks S from the chip size. One workgroup (4 waves) per range and group of <= 4 kv heads
+// (`kv_heads` of them as the kernel sees them), two resident workgroups per CU. Sets decode_num_ranges,
+// decode_heads_per_block and workspace_bytes.
+static pplhip_retcode plan_decode_ranges(const pplhip_mhca_args* a, int kv_heads, pplhip_mhca_plan* plan) {
+    const int64_t nd = a->decoding_batches;
+    const int hpb = decode_heads_per_block(kv_heads);
+    const int64_t groups = kv_heads / hpb;
+    const int64_t slots = (int64_t)device_cu_count() * decode_blocks_per_cu();
+    // halves of a slot: every workgroup streams the same number of bytes, so one workgroup per slot (a single,
+    // perfectly filled round) measures best; the knob moves it to half or twice that
+    const int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
+    // ranges x groups workgroups must not spill over the slots (a second, nearly empty round doubles the time:
+    // 40 kv heads = 10 groups took 56 ranges = 560 workgroups on 512 slots), so the quotient rounds DOWN
+    int64_t ranges = slots * half_slots / 2 / groups;
+    // never more ranges than 128-token pieces of the worst case (every sequence max_kvlen long)
+    const int64_t cap = (nd * a->max_kvlen + 127) / 128;
+    if (ranges > cap) ranges = cap;
+    if (ranges < 8) ranges = 8;
+    if (ranges > 0x3fffffff) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many ranges");
+    plan->decode_num_ranges = (int32_t)ranges;
+    plan->decode_heads_per_block = hpb;
+    plan->workspace_bytes = decode_workspace_bytes(a, ranges);
+    return PPLHIP_RC_SUCCESS;
+}
+
 pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* plan) {
     if (!a || !plan) PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "null argument block");
     memset(plan, 0, sizeof(*plan));
@@ -211,6 +238,17 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     if (needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask)) {
         // write kernel + one launch of the general attention kernel (+ the merge of the decode sequences' pieces)
         plan->general_kernel = 1;
+        const int vheads = a->decoding_batches > 0 ? decode_virtual_heads(a) : 0;
+        if (vheads > 0) {
+            // head_dim 64 / 32: the decode sequences run the head_dim-128 decode kernel over groups of 2 / 4 kv heads
+            // (decode_num_ranges > 0 says so); the general kernel takes the prompts
+            plan->decode_waves_per_block = decode_waves_per_block();
+            const pplhip_retcode rc = plan_decode_ranges(a, vheads, plan);
+            if (rc != PPLHIP_RC_SUCCESS) return rc;
+            plan->general_decode_splits = 1;
+            plan->workspace_bytes = (plan->workspace_bytes + 255) / 256 * 256;
+            return PPLHIP_RC_SUCCESS;
+        }
         plan->general_decode_splits = generic_decode_splits(a, device_cu_count());
         plan->workspace_bytes = (generic_workspace_bytes(a, plan->general_decode_splits) + 255) / 256 * 256;
         return PPLHIP_RC_SUCCESS;
@@ -220,25 +258,9 @@ pplhip_retcode pplhip_mhca_prepare(const pplhip_mhca_args* a, pplhip_mhca_plan* 
     // device; the host only picks S from the chip size. One workgroup (4 waves) per range and group of <= 4 kv heads,
     // two resident workgroups per CU.
     plan->decode_waves_per_block = decode_waves_per_block();
-    const int64_t nd = a->decoding_batches;
-    if (nd > 0) {
-        const int hpb = decode_heads_per_block(a->num_kv_heads);
-        const int64_t groups = a->num_kv_heads / hpb;
-        const int64_t slots = (int64_t)device_cu_count() * decode_blocks_per_cu();
-        // halves of a slot: every workgroup streams the same number of bytes, so one workgroup per slot (a single,
-        // perfectly filled round) measures best; the knob moves it to half or twice that
-        const int64_t half_slots = a->specify_decoding_attn_split_k == 0 ? 1 : a->specify_decoding_attn_split_k == 1 ? 2 : 4;
-        // ranges x groups workgroups must not spill over the slots (a second, nearly empty round doubles the time:
-        // 40 kv heads = 10 groups took 56 ranges = 560 workgroups on 512 slots), so the quotient rounds DOWN
-        int64_t ranges = slots * half_slots / 2 / groups;
-        // never more ranges than 128-token pieces of the worst case (every sequence max_kvlen long)
-        const int64_t cap = (nd * a->max_kvlen + 127) / 128;
-        if (ranges > cap) ranges = cap;
-        if (ranges < 8) ranges = 8;
-        if (ranges > 0x3fffffff) PPLHIP_FAIL(PPLHIP_RC_OUT_OF_RANGE, "decode: too many ranges");
-        plan->decode_num_ranges = (int32_t)ranges;
-        plan->decode_heads_per_block = hpb;
-        plan->workspace_bytes = decode_workspace_bytes(a, ranges);
+    if (a->decoding_batches > 0) {
+        const pplhip_retcode rc = plan_decode_ranges(a, a->num_kv_heads, plan);
+        if (rc != PPLHIP_RC_SUCCESS) return rc;
     }
     // ---- prefill
     plan->prefill_q_tile = 128;
@@ -262,11 +284,17 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "workspace of %llu bytes (256-byte aligned) required",
                     (unsigned long long)plan->workspace_bytes);
     const bool general = needs_general_kernel(a->head_dim, a->num_heads, a->num_kv_heads, a->d_attn_mask);
-    if ((plan->general_kernel != 0) != general || (!general && a->decoding_batches > 0 && plan->decode_num_ranges <= 0))
+    // (head_dim 64 / 32: the decode sequences may run the head_dim-128 decode kernel over groups of kv heads)
+    const bool grouped_decode = general && a->decoding_batches > 0 && plan->decode_num_ranges > 0;
+    if ((plan->general_kernel != 0) != general || (!general && a->decoding_batches > 0 && plan->decode_num_ranges <= 0) ||
+        (grouped_decode && decode_virtual_heads(a) <= 0))
         PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
     // the plan is checked against the arguments before anything is enqueued: a rejected call leaves the slab untouched,
     // and the kernels never write past the workspace the plan declares
-    if (general) {
+    if (grouped_decode) {
+        if (decode_workspace_bytes(a, plan->decode_num_ranges) > plan->workspace_bytes)
+            PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
+    } else if (general) {
         if (plan->general_decode_splits < 0 || plan->general_decode_splits > 64 ||
             generic_workspace_bytes(a, plan->general_decode_splits) > plan->workspace_bytes)
             PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "plan was not produced by pplhip_mhca_prepare for these arguments");
@@ -288,6 +316,13 @@ pplhip_retcode pplhip_mhca_forward(const pplhip_mhca_args* a, const pplhip_mhca_
         // attend over the slab
         pplhip_retcode rcw = launch_kv_quantize_write(&w, s);
         if (rcw != PPLHIP_RC_SUCCESS) return rcw;
+        if (grouped_decode) {
+            // the decode sequences through the decode kernel (their new tokens are in the slab already), the prompts
+            // through the general kernel
+            rcw = launch_decode(a, plan, d_workspace, s, true);
+            if (rcw != PPLHIP_RC_SUCCESS) return rcw;
+            return a->batch > a->decoding_batches ? launch_generic_mhca(a, 1, nullptr, s, true) : PPLHIP_RC_SUCCESS;
+        }
         return launch_generic_mhca(a, plan->general_decode_splits, d_workspace, s);
     }
     // the decode kernel quantises the decode sequences' new tokens (the first decoding_batches packed tokens) into the

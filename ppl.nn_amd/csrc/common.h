@@ -172,10 +172,15 @@ pplhip_retcode launch_kv_stage_prefill(const pplhip_mhca_args* a, half_t* key_ou
 // whether (and where in the workspace) a cache-prefill call stages its K/V as fp16: see pplhip_mhca_plan
 int64_t prefill_staging_tokens(const pplhip_mhca_args* a);
 int decode_heads_per_block(int kv_heads);
+// head dims 64 / 32 whose decode sequences run the head_dim-128 decode kernel over groups of 2 / 4 neighbouring kv
+// heads: the number of such groups, or 0 when the call does not qualify
+int decode_virtual_heads(const pplhip_mhca_args* a);
 bool prefill_writes_new_tokens(const pplhip_mhca_args* a);
 int decode_blocks_per_cu();
 int decode_waves_per_block();
-pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
+// new_tokens_in_slab: the decode sequences' new tokens were quantised into the slab by an earlier launch
+pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream,
+                             bool new_tokens_in_slab = false);
 pplhip_retcode launch_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream);
 // both, in one launch where the call has decode sequences and prompts
 pplhip_retcode launch_decode_and_prefill(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws,
@@ -187,7 +192,9 @@ bool generic_head_dim_supported(int head_dim);
 // nsplit pieces per decode sequence (generic_decode_splits), their partial results in `ws` (generic_workspace_bytes)
 int generic_decode_splits(const pplhip_mhca_args* a, int cu_count);
 uint64_t generic_workspace_bytes(const pplhip_mhca_args* a, int nsplit);
-pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* ws, hipStream_t stream);
+// prompts_only: the decode sequences of the call are somebody else's (the decode kernel's)
+pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* ws, hipStream_t stream,
+                                   bool prompts_only = false);
 pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream);
 // w != null: the launch also quantises the rotated keys and the values of the new tokens into the slab
 pplhip_retcode launch_rope(const pplhip_rope_args* a, const pplhip_kv_write_args* w, hipStream_t stream);

@@ -80,6 +80,12 @@ struct DecodeParams {
     int32_t num_ranges; // S
     int32_t hpb; // kv heads per workgroup: min(kv_heads, 4), a power of two dividing kv_heads
     int32_t merge_by_boundary; // merge kernel: blockIdx.y counts range boundaries instead of sequences
+    // Head dims 64 and 32: 2 (4) kv heads that lie next to each other in the slab are streamed as ONE kv head of 128
+    // channels ("virtual" head: kv_heads, rep and addr.stride_h above are the virtual ones, rep = 2 (4) x the real
+    // number of query heads per kv head, at most 16). A query head's 64 (32) channels sit in its own part of the
+    // 128-channel query operand, zeros elsewhere, so its scores come out of the other heads' channels as + 0; of its
+    // 128 output channels only its own part means anything and is stored. sub_shift = log2(128 / head_dim): 0, 1, 2.
+    int32_t sub_shift;
     int32_t new_tokens_written_elsewhere; // the launch's write-only workgroups put the decode sequences' new tokens
                                           // into the slab: the decode waves only patch their stage buffers
     float score_scale; // log2(e) / sqrt(Dh)
@@ -583,6 +589,21 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
         }
     };
 
+    // Virtual heads (sub_shift > 0): which part of the 128 channels is the column's head's, and which the lane holds
+    const int row_len = kDh >> p.sub_shift; // head_dim: channels of a row of the query / output tensors
+    const int chan_off = (32 * kq) & (row_len - 1); // the lane's 32 channels inside such a row
+    // the lane's channels belong to the head in column m (columns past rep copy column 0)
+    const bool q_keep = ((32 * kq) >> (7 - p.sub_shift)) == ((m < p.rep ? m : 0) / (p.rep >> p.sub_shift));
+    auto keep_own_channels = [&](half8_t (&q)[2][2]) { // (after the query loads have landed)
+        if (!q_keep) {
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) q[jj][i][e] = (half_t)0.f;
+        }
+    };
     // Q^T as the B operand, kept for a whole segment: q[j][i] = Q[head m][32*kq + 16*j + 8*i .. +7]
     // four query pieces (+ the lane's group of the sequence's new token)
     constexpr int kQueryLoads = 5;
@@ -599,16 +620,21 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
         }
         // Columns m >= rep of the MFMA have no query head: they carry a copy of head 0 of the group, whose results
         // are never stored.
-        const half_t* qp = p.q + (((int64_t)g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (m < p.rep ? m : 0)) * kDh;
+        // (a row of the query tensor holds head_dim = row_len channels; the lane's 32 channels of the 128-channel
+        // operand are channels chan_off .. + 31 of that row when they belong to the column's head, see q_keep)
+        const half_t* qp =
+            p.q + (((int64_t)g.qrow * p.num_heads) + (int64_t)kvh * p.rep + (m < p.rep ? m : 0)) * row_len + chan_off;
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                if (untracked) load16_untracked(q[jj][i], qp + 32 * kq + 16 * jj + 8 * i);
-                else q[jj][i] = *reinterpret_cast<const half8_t*>(qp + 32 * kq + 16 * jj + 8 * i);
+                if (untracked) load16_untracked(q[jj][i], qp + 16 * jj + 8 * i);
+                else q[jj][i] = *reinterpret_cast<const half8_t*>(qp + 16 * jj + 8 * i);
             }
-        if (!untracked) // the wait for these loads happens HERE, not in front of every stage's first MFMA
+        if (!untracked) { // the wait for these loads happens HERE, not in front of every stage's first MFMA
             asm volatile("" : "+v"(q[0][0]), "+v"(q[0][1]), "+v"(q[1][0]), "+v"(q[1][1]), "+v"(newtok));
+            keep_own_channels(q);
+        }
     };
 
     // When every wave owns a whole kv head (no token split inside the workgroup) nothing is combined through LDS, the
@@ -727,7 +753,9 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
             if (m < p.rep) {
                 const int head = kvh * p.rep + m;
                 if (cur.whole_sequence) {
-                    half_t* dst = p.out + ((int64_t)cur.qrow * p.num_heads + head) * kDh + 32 * kq;
+                    // (virtual heads: only the head's own channels are output; every lane group issues its stores
+                    // or none, the count behind the next stage 0 stays a lower bound)
+                    half_t* dst = p.out + ((int64_t)cur.qrow * p.num_heads + head) * row_len + chan_off;
                     const float inv_l = 1.0f / l_tot;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -736,7 +764,7 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
                         for (int i = 0; i < 8; ++i) o[i] = (half_t)(ss.oacc[i][e] * inv_l);
                         uint4 packed;
                         __builtin_memcpy(&packed, o, 16);
-                        *reinterpret_cast<uint4*>(dst + 8 * e) = packed;
+                        if (q_keep) *reinterpret_cast<uint4*>(dst + 8 * e) = packed;
                     }
                 } else {
                     const int64_t prow = (s_idx + cur.b) * p.num_heads + head;
@@ -787,7 +815,8 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
                 }
                 const int head = (hg * p.hpb + kl) * p.rep + h;
                 if (cur.whole_sequence) {
-                    p.out[((int64_t)cur.qrow * p.num_heads + head) * kDh + d] = (half_t)(acc / l);
+                    if ((d >> (7 - p.sub_shift)) == h / (p.rep >> p.sub_shift)) // (virtual heads: the head's own channels)
+                        p.out[((int64_t)cur.qrow * p.num_heads + head) * row_len + (d & (row_len - 1))] = (half_t)(acc / l);
                 } else {
                     const int64_t prow = (s_idx + cur.b) * p.num_heads + head;
                     p.part_acc[prow * kDh + d] = acc;
@@ -814,6 +843,7 @@ __device__ __forceinline__ void decode_workgroup(const DecodeParams& p, uint32_t
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                 for (int i = 0; i < 2; ++i) qB[jj][i] = qN[jj][i];
+            keep_own_channels(qB);
             newB = newN;
             cur_in_flight = true;
         } else {
@@ -913,7 +943,10 @@ __global__ __launch_bounds__(32 * kMergeGroups) void decode_merge_kernel(const D
             a += w * red[i][d];
             L += w * red[i][kDh + 1];
         }
-        p.out[(p.seqstarts[b] * p.num_heads + head) * kDh + d] = (half_t)(a / L);
+        // (virtual heads, see DecodeParams::sub_shift: only the head's own channels are output)
+        const int row_len = kDh >> p.sub_shift;
+        if ((d >> (7 - p.sub_shift)) == (head % p.rep) / (p.rep >> p.sub_shift))
+            p.out[(p.seqstarts[b] * p.num_heads + head) * row_len + (d & (row_len - 1))] = (half_t)(a / L);
     }
 }
 
@@ -923,6 +956,17 @@ int decode_blocks_per_cu() {
 
 int decode_waves_per_block() {
     return kDecodeWaves;
+}
+
+// Head dims 64 and 32 run the decode kernel with 2 (4) neighbouring kv heads as one head of 128 channels when the
+// heads are neighbours in the slab, their number divides, and the query heads of such a group fit the 16 columns.
+// (The number of kv heads the kernel then sees: num_kv_heads >> shift; 0 = not this way.)
+int decode_virtual_heads(const pplhip_mhca_args* a) {
+    const int shift = a->head_dim == 64 ? 1 : a->head_dim == 32 ? 2 : -1;
+    if (shift < 0 || a->d_attn_mask != nullptr || a->num_kv_heads <= 0) return 0;
+    if (a->num_kv_heads % (1 << shift) || a->cache_stride_h != a->head_dim) return 0;
+    if (a->num_heads % a->num_kv_heads || ((a->num_heads / a->num_kv_heads) << shift) > 16) return 0;
+    return a->num_kv_heads >> shift;
 }
 
 int decode_heads_per_block(int kv_heads) {
@@ -949,9 +993,13 @@ static pplhip_retcode reserve_decode_lds(std::atomic<uint64_t>& done, std::initi
 }
 
 // Fills the launch parameters of the decode sequences' attention; *blocks: workgroups of the launch.
+// a->head_dim 128, or 64 / 32 where decode_virtual_heads() allows it.
 static pplhip_retcode decode_setup(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, DecodeParams* out,
                                    int64_t* out_blocks) {
     const int nd = (int)a->decoding_batches;
+    const int sub_shift = a->head_dim == 128 ? 0 : a->head_dim == 64 ? 1 : 2;
+    if (a->head_dim != (kDh >> sub_shift) || (sub_shift && !decode_virtual_heads(a)))
+        PPLHIP_FAIL(PPLHIP_RC_INVALID_VALUE, "decode: head_dim %d does not run this kernel", a->head_dim);
     DecodeParams p;
     p.q = (const half_t*)a->d_query;
     p.cur_key = (const half_t*)a->d_current_key;
@@ -964,11 +1012,13 @@ static pplhip_retcode decode_setup(const pplhip_mhca_args* a, const pplhip_mhca_
     p.cs_stride_b = a->cachestart_stride_b;
     p.page_shift = page_shift_of(a->cache_mode, a->page_size);
     p.out = (half_t*)a->d_output;
-    p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->layer_idx};
+    p.addr = CacheAddr{a->cache_stride_s, a->cache_stride_l, a->cache_stride_h << sub_shift, a->cache_stride_kv,
+                       a->layer_idx};
     p.nd = nd;
     p.num_heads = a->num_heads;
-    p.kv_heads = a->num_kv_heads;
-    p.rep = a->num_heads / a->num_kv_heads;
+    p.kv_heads = a->num_kv_heads >> sub_shift;
+    p.rep = (a->num_heads / a->num_kv_heads) << sub_shift;
+    p.sub_shift = sub_shift;
     p.num_ranges = plan->decode_num_ranges;
     p.hpb = decode_heads_per_block(p.kv_heads);
     p.score_scale = 1.4426950408889634f / sqrtf((float)a->head_dim);
@@ -1004,12 +1054,14 @@ static pplhip_retcode launch_decode_merge(const DecodeParams& p, hipStream_t str
     return PPLHIP_RC_SUCCESS;
 }
 
-pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream) {
+pplhip_retcode launch_decode(const pplhip_mhca_args* a, const pplhip_mhca_plan* plan, void* ws, hipStream_t stream,
+                             bool new_tokens_in_slab) {
     if (a->decoding_batches == 0) return PPLHIP_RC_SUCCESS;
     DecodeParams p;
     int64_t blocks;
     pplhip_retcode rc = decode_setup(a, plan, ws, &p, &blocks);
     if (rc != PPLHIP_RC_SUCCESS) return rc;
+    p.new_tokens_written_elsewhere = new_tokens_in_slab;
     const size_t lds_bytes = kDecodeLdsBytes; // stage buffers; the final combine (4 * rep * 130 floats) reuses them
     static std::atomic<uint64_t> lds_opted_in{0};
     rc = reserve_decode_lds(lds_opted_in, {reinterpret_cast<const void*>(decode_int8kv_kernel<false, false>),

@@ -817,7 +817,9 @@ bool generic_head_dim_supported(int head_dim) {
 // the head_dim the kernels are compiled for: the next multiple of 32
 static int generic_kernel_head_dim(int head_dim) { return (head_dim + 31) / 32 * 32; }
 
-static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max_seqlen, hipStream_t stream) {
+// skip_first: the tile kernel leaves out the first `skip_first` sequences (decode sequences that another kernel serves)
+static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max_seqlen, hipStream_t stream,
+                                     int skip_first = 0) {
     if (!generic_head_dim_supported(head_dim))
         PPLHIP_FAIL(PPLHIP_RC_UNSUPPORTED, "head_dim %d: must be a multiple of 16 between 16 and 256", head_dim);
     p.scale_log2 = kLog2e / sqrtf((float)head_dim);
@@ -832,7 +834,12 @@ static pplhip_retcode launch_generic(GenericParams& p, int head_dim, int64_t max
     if (p.nsplit < 1) p.nsplit = 1;
     p.first_seq = 0;
     int64_t blocks, decode_blocks = 0;
-    if (p.split_seqs > 0 && p.rep <= 16 && !padded && (p.pages.page_shift == 0 || p.pages.page_shift >= 4)) {
+    if (skip_first > 0) {
+        p.nsplit = 1, p.split_seqs = 0;
+        p.first_seq = skip_first;
+        const int64_t groups = tiles * (int64_t)(p.batch - skip_first);
+        blocks = (groups + 7) / 8 * 8 * p.kv_heads;
+    } else if (p.split_seqs > 0 && p.rep <= 16 && !padded && (p.pages.page_shift == 0 || p.pages.page_shift >= 4)) {
         // generic_decode_kernel takes them; the tile kernel the rest of the batch
         if (p.nsplit == 1) p.piece_tokens = 0x7fffffc0; // the whole sequence
         decode_blocks = ((int64_t)p.split_seqs * p.nsplit * (p.kv_heads / generic_decode_heads_per_wave(p, head_dim)) + 3) / 4;
@@ -887,7 +894,8 @@ uint64_t generic_workspace_bytes(const pplhip_mhca_args* a, int nsplit) {
 }
 
 // MultiHeadCacheAttention through the general kernel; the new tokens are already in the slab.
-pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* ws, hipStream_t stream) {
+pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* ws, hipStream_t stream,
+                                   bool prompts_only) {
     GenericParams p;
     p.nsplit = nsplit < 1 ? 1 : nsplit;
     p.split_seqs = (int32_t)a->decoding_batches;
@@ -922,7 +930,7 @@ pplhip_retcode launch_generic_mhca(const pplhip_mhca_args* a, int nsplit, void* 
     p.k16_holds_new_tokens = 1;
     p.is_causal = a->is_causal;
     const int64_t max_rows_tokens = a->batch > a->decoding_batches ? a->max_seqlen : 1;
-    return launch_generic(p, a->head_dim, max_rows_tokens, stream);
+    return launch_generic(p, a->head_dim, max_rows_tokens, stream, prompts_only ? (int)a->decoding_batches : 0);
 }
 
 pplhip_retcode launch_generic_mha(const pplhip_mha_args* a, hipStream_t stream) {

@@ -140,6 +140,40 @@ def test_prepare_routes_other_shapes_to_the_general_kernel(hiplib, mutate):
     assert plan.general_decode_splits <= 1 and plan.workspace_bytes == 0
 
 
+def test_prepare_plans_head_dim_64_and_32_decode_over_groups_of_kv_heads(hiplib):
+    """head_dim 64 (32) with kv heads that are neighbours in the slab and pair up (go in fours): the general plan
+    carries the decode kernel's ranges for the decode sequences; anything that breaks the grouping (odd kv heads, more
+    than 16 query heads per group, heads apart in the slab, a mask) plans the general decode kernel."""
+    def plan_of(H, KVH, Dh, stride_h=None, mask=False):
+        b = workloads.Batch(H, KVH, Dh, [1] * 40 + [9], [3000] * 40 + [0], 40)
+        a = cabi.MhcaArgs()
+        fake = lambda t: C.c_void_p(0x1000)
+        harness.fill_mhca_args(a, b, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, ptr=fake, split_k=1)
+        if stride_h is not None:
+            a.cache_stride_h = stride_h
+        if mask:
+            a.d_attn_mask, a.attn_mask_stride_q = 0x10, 4096
+        plan = cabi.MhcaPlan()
+        assert hiplib.pplhip_mhca_prepare(C.byref(a), C.byref(plan)) == cabi.RC_SUCCESS, hiplib.pplhip_last_error()
+        assert plan.general_kernel == 1
+        return a, plan
+
+    a, plan = plan_of(32, 8, 64)  # 4 groups of 2 kv heads, 8 query heads each: one workgroup per range
+    assert plan.decode_num_ranges == 512 and plan.decode_heads_per_block == 4 and plan.general_decode_splits == 1
+    assert plan.workspace_bytes >= (512 + 40) * 32 * 130 * 4 + 512 * 4 and plan.workspace_bytes % 256 == 0
+    a, plan = plan_of(32, 8, 32)  # 2 groups of 4 kv heads, 16 query heads each
+    assert plan.decode_num_ranges == 512 and plan.decode_heads_per_block == 2
+    for args in ((28, 7, 64), (72, 8, 64), (40, 8, 32)):  # odd kv heads; 18 and 20 query heads per group
+        a, plan = plan_of(*args)
+        assert plan.decode_num_ranges == 0 and plan.general_decode_splits > 1
+    a, plan = plan_of(32, 8, 64, stride_h=4096)  # heads apart in the slab (cache_layout 3)
+    assert plan.decode_num_ranges == 0
+    a, plan = plan_of(32, 8, 64, mask=True)
+    assert plan.decode_num_ranges == 0
+    a, plan = plan_of(32, 8, 96)
+    assert plan.decode_num_ranges == 0
+
+
 @pytest.mark.parametrize("kvh", [1, 2, 3, 4, 5, 8, 12, 16, 32, 40, 64])
 def test_decode_plan_fills_one_round_of_workgroup_slots(hiplib, kvh):
     """The decode launch runs (ranges x groups of <= 4 kv heads) workgroups, two per compute unit: with the default

@@ -21,8 +21,11 @@ def check(b, t, what, pieces=None, **kw):
     ref = harness.run_oracle(b, t, **kw)
     got = harness.run_device(b, t, plan_out=plans, **kw)
     assert plans[0].general_kernel == 1
-    assert (plans[0].workspace_bytes == 0) == (plans[0].general_decode_splits <= 1)
-    if pieces is not None:
+    # head_dim 64 / 32 with kv heads that pair up in the slab: the decode sequences run the head_dim-128 decode kernel
+    # over groups of kv heads (its ranges and workspace), the general kernel takes the prompts
+    grouped = plans[0].decode_num_ranges > 0
+    assert grouped or (plans[0].workspace_bytes == 0) == (plans[0].general_decode_splits <= 1)
+    if pieces is not None and not grouped:
         assert plans[0].general_decode_splits == pieces
     assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
     assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
@@ -51,6 +54,38 @@ def test_head_dims_that_are_not_multiples_of_32(Dh, H, KVH):
     check(b, t, f"head_dim {Dh}")
     check(b, t, f"head_dim {Dh}, cache-prefill", cache_prefill=1)
     check(b, t, f"head_dim {Dh}, cache_layout 3", layout=3)
+
+
+@pytest.mark.parametrize("Dh,H,KVH", [(64, 8, 2), (64, 32, 8), (64, 16, 16), (64, 6, 6), (32, 16, 4), (32, 8, 8)])
+def test_head_dim_64_and_32_decode_sequences_run_the_decode_kernel_over_groups_of_kv_heads(Dh, H, KVH):
+    """Two (four) kv heads that are neighbours in the slab are streamed as one head of 128 channels by the head_dim-128
+    decode kernel, every query head's channels in its own part of the 128-channel query operand: ragged decode
+    sequences (short, one stage, many stages, split over ranges), with prompts in the same call, contiguous and paged
+    (same bits); heads that are not neighbours (cache_layout 3) keep the general decode kernel."""
+    b = workloads.Batch(H, KVH, Dh, [1] * 7 + [70, 5], [2000, 5, 0, 319, 1300, 31, 32, 0, 0], 7, num_layer=2,
+                        layer_idx=1, name="grouped_heads")
+    t = workloads.make_tensors(b, seed=H + Dh)
+    plans = []
+    ref = harness.run_oracle(b, t)
+    got = harness.run_device(b, t, plan_out=plans)
+    assert plans[0].general_kernel == 1 and plans[0].decode_num_ranges > 0 and plans[0].workspace_bytes > 0
+    assert np.array_equal(ref["cache"], got["cache"]) and np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16))
+    harness.assert_attn_close(got["output"], ref["output_f64"], what=f"grouped kv heads, head_dim {Dh}")
+    paged = harness.PagedLayout(b, page_size=64, seed=3)
+    gotp = harness.run_device(b, t, paged=paged)
+    assert np.array_equal(gotp["output"].view(np.uint16), got["output"].view(np.uint16))
+    plans3 = []
+    got3 = harness.run_device(b, t, plan_out=plans3, layout=3)
+    assert plans3[0].general_kernel == 1 and plans3[0].decode_num_ranges == 0
+    harness.assert_attn_close(got3["output"], ref["output_f64"], what="cache_layout 3 keeps the general decode kernel")
+    # decode only, and the split knob at its two other settings
+    bd = workloads.Batch(H, KVH, Dh, [1] * 5, [4000, 700, 64, 1, 129], 5, name="grouped_heads_decode_only")
+    td = workloads.make_tensors(bd, seed=7)
+    refd = harness.run_oracle(bd, td)
+    for split_k in (0, 1, 2):
+        gd = harness.run_device(bd, td, split_k=split_k)
+        assert np.array_equal(refd["cache"], gd["cache"])
+        harness.assert_attn_close(gd["output"], refd["output_f64"], what=f"decode only, split knob {split_k}")
 
 
 @pytest.mark.parametrize("H,KVH", [(34, 2), (20, 1), (48, 2)])
