@@ -742,18 +742,23 @@ def main():
                       "staged": int(cdb.plan.prefill_staging)})
         del cdb
         torch.cuda.empty_cache()
-        # the general kernel (other head dims, attn_mask, > 16 query heads per kv head): the cfg2 shapes at head_dim 64
+        # other head dims (the plan's general_kernel route): the cfg2 shapes at head_dim 64, whose decode sequences
+        # run the decode kernel over pairs of kv heads (decode_ranges > 0), and at head_dim 96, where they run the
+        # general decode kernel
         gen = {}
-        gd = workloads.Batch(32, 8, 64, dec_b.seqlens, dec_b.start_pos, dec_b.decoding_batches, name="cfg2 decode part, Dh 64")
-        gdb = DeviceBatch(pkg, lib, gd, seed=7, n_slabs=N_SLABS)
-        g_mean, g_med, g_n = timed_robust(gdb.step)
-        gen["decode_cfg2_shape_head_dim_64"] = {
-            "ms_per_step": g_med, "ms_per_step_mean": g_mean, "calls_timed": g_n,
-            "achieved_GBs": gd.decode_bytes() / (g_med * 1e-3) / 1e9,
-            "frac_of_hbm_peak": gd.decode_bytes() / (g_med * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "general_kernel": int(gdb.plan.general_kernel)}
-        del gdb
-        torch.cuda.empty_cache()
+        for gdh in (64, 96):
+            gd = workloads.Batch(32, 8, gdh, dec_b.seqlens, dec_b.start_pos, dec_b.decoding_batches,
+                                 name="cfg2 decode part, Dh %d" % gdh)
+            gdb = DeviceBatch(pkg, lib, gd, seed=7, n_slabs=N_SLABS)
+            g_mean, g_med, g_n = timed_robust(gdb.step)
+            gen["decode_cfg2_shape_head_dim_%d" % gdh] = {
+                "ms_per_step": g_med, "ms_per_step_mean": g_mean, "calls_timed": g_n,
+                "achieved_GBs": gd.decode_bytes() / (g_med * 1e-3) / 1e9,
+                "frac_of_hbm_peak": gd.decode_bytes() / (g_med * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "general_kernel": int(gdb.plan.general_kernel), "decode_ranges": int(gdb.plan.decode_num_ranges),
+                "general_decode_splits": int(gdb.plan.general_decode_splits)}
+            del gdb
+            torch.cuda.empty_cache()
         gp = workloads.Batch(32, 8, 64, _np.full(4, 2048, _np.int64), _np.zeros(4, _np.int64), 0, name="4x2048 prefill, Dh 64")
         gpb = DeviceBatch(pkg, lib, gp, seed=8, n_slabs=1)
         gen["prefill_4x2048_head_dim_64"] = prefill_entry(gpb, gp, {"general_kernel": int(gpb.plan.general_kernel)})
