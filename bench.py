@@ -711,11 +711,15 @@ def main():
     if args.workload == "cfg2" and not args.no_other_configs and want("other"):
         # the other decode configurations at their full sizes
         others = {}
-        for name, ob in (("cfg1 Llama-2-7B pure decode (H32/KVH32/Dh128): 64 seqs kv~U[128,2048]",
-                          workloads.cfg1_llama2_7b_decode()),
-                         ("cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]",
-                          workloads.cfg3_long_context())):
-            odb = DeviceBatch(pkg, lib, ob, seed=4, n_slabs=N_SLABS)
+        # (cfg1 twice: in cache_layout 0 the scale rows of 32 kv heads are 128 bytes per token and workgroup at a 2 KB
+        # stride, which the memory system serves at two thirds of the K/V rows' rate; in cache_layout 3 a head's
+        # tokens are neighbours)
+        for name, ob, olayout in (("cfg1 Llama-2-7B pure decode (H32/KVH32/Dh128): 64 seqs kv~U[128,2048]",
+                                   workloads.cfg1_llama2_7b_decode(), 0),
+                                  ("cfg1 in cache_layout 3 (L, 2, KVH, MaxT, Dh)", workloads.cfg1_llama2_7b_decode(), 3),
+                                  ("cfg3 long-context decode (H8/KVH1/Dh128): 8 seqs kv~U[32768,131072]",
+                                   workloads.cfg3_long_context(), 0)):
+            odb = DeviceBatch(pkg, lib, ob, seed=4, n_slabs=N_SLABS, layout=olayout)
             o_mean, o_med, o_n = timed_robust(odb.step)
             o_gbs = ob.decode_bytes() / (o_med * 1e-3) / 1e9
             others[name] = {"tokens_per_s": ob.decoding_batches / (o_med * 1e-3), "ms_per_step": o_med,
