@@ -552,3 +552,42 @@ def test_hundreds_of_decode_sequences(KVH):
     hist[[7, 150, 299]] = [3000, 1777, 2500]
     b = workloads.Batch(8, KVH, 128, [1] * 300 + [40, 3], hist.tolist() + [0, 0], 300, name="300 decode sequences")
     check(b, workloads.make_tensors(b, seed=82))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_batches_through_the_tuned_kernels(seed):
+    """Seeded random batches at head_dim 128: any number of kv heads (workgroups of 1, 2 or 4 heads, range counts that
+    are no multiple of 8), 0 .. 39 decode sequences whose lengths sit on and around the stage, tile and page edges,
+    prompts with and without cache-prefill (and history), contiguous / paged / cache_layout 3 slabs, every split knob.
+    Slab bytes and scales bit-exact, outputs within tolerance."""
+    rng = np.random.default_rng(5000 + seed)
+    KVH = int(rng.choice([1, 2, 3, 4, 5, 8, 10, 12]))
+    rep = int(rng.choice([1, 2, 4, 8, 16]))
+    nd = int(rng.integers(0, 40))
+    npf = int(rng.integers(0, 4)) if nd else int(rng.integers(1, 4))
+    edges = [1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 1023, 1024, 1025]
+    hist = [int(rng.choice(edges)) - 1 if rng.random() < 0.4 else int(rng.integers(0, 3000)) for _ in range(nd)]
+    cp = int(rng.random() < 0.3)
+    seqlens = [1] * nd + [int(rng.integers(1, 400)) for _ in range(npf)]
+    start = hist + [int(rng.integers(0, 300)) if cp else 0 for _ in range(npf)]
+    b = workloads.Batch(KVH * rep, KVH, 128, seqlens, start, nd, num_layer=int(rng.integers(1, 3)), layer_idx=0,
+                        is_causal=1, slack_tokens=int(rng.integers(0, 3)), name="random_tuned")
+    t = workloads.make_tensors(b, seed=seed)
+    kw = {}
+    how = int(rng.integers(0, 4))
+    if how == 1:
+        kw["paged"] = harness.PagedLayout(b, page_size=int(rng.choice([64, 128, 256])), seed=seed)
+    elif how == 2:
+        kw["layout"] = 3
+    if cp:
+        kw["cache_prefill"] = 1
+    split_k = int(rng.integers(0, 3))
+    print(f"case random tuned, seed {seed}: H={b.num_heads} KVH={KVH} nd={nd} prompts={npf} split_k={split_k} {sorted(kw)}",
+          flush=True)
+    ref = harness.run_oracle(b, t, **kw)
+    plans = []
+    got = harness.run_device(b, t, split_k=split_k, plan_out=plans, **kw)
+    assert plans[0].general_kernel == 0
+    assert np.array_equal(ref["cache"], got["cache"]), "int8 cache bytes differ"
+    assert np.array_equal(ref["scale"].view(np.uint16), got["scale"].view(np.uint16)), "fp16 scales differ"
+    harness.assert_attn_close(got["output"], ref["output_f64"], what=f"random tuned batch, seed {seed}")
